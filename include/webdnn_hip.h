@@ -1,0 +1,209 @@
+/*
+ * webdnn_hip.h — C ABI of libwebdnn_hip.so, the native side of the `hip`
+ * backend for the WebDNN descriptor runner.
+ *
+ * The reference has no C header for this path: its native precedent is the
+ * WASM worker protocol (integer buffer ids + `extern "C"` kernels taking raw
+ * float pointers and int/float scalars):
+ *   src/descriptor_runner/backend/wasm/wasmContextImpl.ts:113-163
+ *       (alloc / destroy / write / read / runKernel messages)
+ *   src/shader/wasm/pre.js:4-91            (id -> pointer table, dispatch)
+ *   src/shader/wasm/src/core/allocation.cpp:4-15   (webdnn_malloc/free)
+ *   src/shader/wasm/src/kernels/standard/gemm.cpp:19-104 (kernel_gemm_*)
+ * Each entry point below names the reference interface it stands in for.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative WDH_E* code on
+ *     failure; it never aborts or throws.  wdh_last_error() returns a
+ *     message for the last failure on the calling thread.
+ *   - device buffers are named by opaque positive 64-bit handles
+ *     (wdh_alloc); 0 means "no tensor" where a tensor is optional.
+ *   - all work is enqueued on ONE HIP stream owned by the library; calls
+ *     return as soon as the work is enqueued.  wdh_read() and wdh_sync()
+ *     are the only blocking calls.
+ *   - all tensors are dense row-major; float tensors are IEEE fp32,
+ *     index tensors int32 (the runner clips ONNX int64 to int32:
+ *     src/descriptor_runner/core/runnerImpl.ts:167-198).
+ *   - strides are in ELEMENTS, not bytes.
+ *   - the library is not re-entrant: call it from one thread at a time
+ *     (the descriptor runner is single-threaded:
+ *     src/descriptor_runner/core/runnerImpl.ts:377-542).
+ */
+#ifndef WEBDNN_HIP_H_
+#define WEBDNN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WDH_OK 0
+#define WDH_ENODEV (-1)   /* no usable gfx950 device / driver            */
+#define WDH_EINVAL (-2)   /* bad argument (shape, handle, stride, op id) */
+#define WDH_ENOMEM (-3)   /* device or pinned-host allocation failed     */
+#define WDH_EHIP (-4)     /* a HIP runtime call failed                   */
+#define WDH_ESTATE (-5)   /* library not initialised                     */
+
+typedef int64_t wdh_buf;
+
+/* ---- lifetime -------------------------------------------------------- */
+
+/* Replaces WebDNNWasmContextImpl.initialize() (worker start-up),
+ * backend/wasm/wasmContextImpl.ts:39-73.  Selects `device`, creates the
+ * stream, the pinned staging buffers and the buffer pool.  WDH_ENODEV when
+ * there is no device: the host context must turn that into a thrown Error so
+ * that load() skips the backend (src/descriptor_runner/index.ts:68-79). */
+int wdh_init(int device);
+void wdh_shutdown(void);
+/* Message for the most recent failure on this thread ("" if none). */
+const char *wdh_last_error(void);
+/* Device facts used for roofline arithmetic (name is NUL-terminated). */
+int wdh_device_info(char *name, int name_cap, int *compute_units,
+                    int *clock_mhz, uint64_t *hbm_bytes);
+
+/* ---- buffers --------------------------------------------------------- */
+
+/* Replaces the `alloc` message, wasmContextImpl.ts:128-134 and
+ * webdnn_malloc, allocation.cpp:4-9.  Returns a handle > 0, or 0 on failure
+ * (see wdh_last_error).  Zero-byte requests succeed.  Contents are
+ * undefined.  Blocks come from a size-bucketed pool of hipMalloc memory. */
+wdh_buf wdh_alloc(size_t bytes);
+/* Replaces `destroy`, wasmContextImpl.ts:136-141.  The block returns to the
+ * pool; work already enqueued on the stream still sees valid memory because
+ * later users are ordered behind it on the same stream. */
+int wdh_free(wdh_buf h);
+/* Replaces `write`, wasmContextImpl.ts:143-151: host -> device through
+ * pinned staging + hipMemcpyAsync.  `src` may be reused on return. */
+int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes);
+/* Replaces `read`, wasmContextImpl.ts:153-163: device -> host; blocks until
+ * every previously enqueued kernel and this copy have finished. */
+int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes);
+/* Device-to-device copy; replaces kernel_copy,
+ * src/shader/wasm/src/kernels/standard/copy.cpp:6-8. */
+int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
+             size_t bytes);
+int wdh_sync(void);
+/* Pool accounting: bytes handed out, bytes cached in the pool, high-water
+ * mark of hipMalloc'ed bytes (cf. perfTotalMemory,
+ * backend/wasm/wasmTensorImpl.ts:29-35).  Any pointer may be NULL. */
+int wdh_mem_stats(uint64_t *in_use, uint64_t *cached, uint64_t *peak);
+/* Return cached blocks to the driver (cf. deallocateToBytes,
+ * backend/webgl/webglContextImpl.ts:541-568). */
+int wdh_trim(size_t keep_bytes);
+
+/* ---- timing (measurePerformance, core/runnerImpl.ts:368-375,533-541) -- */
+
+#define WDH_MAX_EVENTS 4096
+int wdh_event_record(int id);              /* 0 <= id < WDH_MAX_EVENTS */
+int wdh_event_elapsed_ms(int start_id, int stop_id, float *ms); /* blocks */
+
+/* ---- epilogues shared by gemm / conv ---------------------------------- */
+
+#define WDH_EPI_NONE 0
+#define WDH_EPI_RELU 1      /* y = max(y, 0) with Math.max semantics      */
+
+/* ---- Gemm / MatMul ----------------------------------------------------
+ * Replaces CpuGemm.run (operators/cpu/operators/standard/gemm.ts:21-61),
+ * CpuMatMul.calcDim2/calcDim3 (.../matmul.ts:58-111) and the WASM
+ * kernel_gemm_transa{0,1}_transb{0,1}[_c] family (gemm.cpp:19-104).
+ *
+ *   for b < batch, i < m, j < n:
+ *     acc          = sum_{x<k} A[b*sAb + i*sA0 + x*sA1] * B[b*sBb + x*sB0 + j*sB1]
+ *     Y[(b*m+i)*n+j] = epi( f32(alpha*acc) + beta * C[i*sC0 + j*sC1] )
+ *
+ * C == 0 means no C term (MatMul; Gemm without bias).  sC0/sC1 come from the
+ * unidirectional broadcast of C to [m,n] (operatorUtil.ts:178-209), so either
+ * may be 0.  sAb/sBb may be 0 (batch broadcast, base/matmul.ts:60-70).
+ * transA/transB are expressed through the strides exactly as
+ * base/gemm.ts:39-56 does.  At least one of (sA0,sA1) and one of (sB0,sB1)
+ * must be 1 or the extent along it 1 (dense operands).
+ * `R` (0 = none) is an optional residual of shape [batch,m,n] added after the
+ * C term and before the epilogue; it exists for fused MatMul+Add graphs. */
+int wdh_gemm(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
+             int n, int k, int64_t sAb, int64_t sA0, int64_t sA1, int64_t sBb,
+             int64_t sB0, int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
+             float beta, int epilogue, wdh_buf R);
+
+/* ---- Conv (2-D, NCHW) ------------------------------------------------
+ * Replaces CpuConv.run = im2col + matmul + transpose + bias
+ * (operators/cpu/operators/standard/conv.ts:134-333) and the four WebGPU
+ * dispatches (operators/webgpu/operators/standard/conv.ts:13-120).
+ *   X [n, c, h, w]   W [cout, c/group, kh, kw]   Bias [cout] or 0
+ *   Y [n, cout, oh, ow],  oh = floor((h+pt+pb-dh*(kh-1)-1)/sh)+1 (base/conv.ts:43-59)
+ *   Y = epi( f32(sum) + bias[co] (+ R) );  R: optional residual shaped like Y. */
+int wdh_conv2d(wdh_buf X, wdh_buf W, wdh_buf Bias, wdh_buf Y, int n, int c,
+               int h, int w, int cout, int kh, int kw, int pt, int pl, int pb,
+               int pr, int sh, int sw, int dh, int dw, int group, int epilogue,
+               wdh_buf R);
+
+/* ---- elementwise -------------------------------------------------------
+ * Replaces Binary7 (operators/cpu/operators/standard/binary7.ts:16-68) and
+ * kernel_{add,sub,mul,div,pow}_d0..d6 (binary7s.cpp:9-22).  ndim <= 6;
+ * strides come from broadcastMulti (operatorUtil.ts:211-245): 0 on broadcast
+ * axes.  dtype: 0 = float32, 1 = int32 (Pow: float32 only here). */
+#define WDH_BIN_ADD 0
+#define WDH_BIN_SUB 1
+#define WDH_BIN_MUL 2
+#define WDH_BIN_DIV 3
+#define WDH_BIN_POW 4
+int wdh_binary(int op, int dtype, wdh_buf L, wdh_buf R, wdh_buf Y, int ndim,
+               const int32_t *out_shape, const int64_t *strides_l,
+               const int64_t *strides_r);
+
+/* Replaces CPUUnary (operators/cpu/operators/standard/unary.ts:10-32) and
+ * kernel_{relu,sigmoid,sqrt,exp,tanh,...} (unarys.cpp:11-17).
+ * dtype 1 (int32) is accepted for RELU, ABS and NEG only. */
+#define WDH_UN_RELU 0
+#define WDH_UN_SIGMOID 1   /* (tanh(x/2)+1)/2, unary.ts:158-164 */
+#define WDH_UN_SQRT 2
+#define WDH_UN_EXP 3
+#define WDH_UN_TANH 4
+#define WDH_UN_ABS 5
+#define WDH_UN_NEG 6
+#define WDH_UN_RECIPROCAL 7
+int wdh_unary(int op, int dtype, wdh_buf X, wdh_buf Y, size_t length);
+
+/* ---- row reductions ----------------------------------------------------
+ * Softmax over the last axis: X viewed as [outer, len]; replaces
+ * Softmax.run (operators/cpu/operators/standard/softmax.ts:34-57). */
+int wdh_softmax(wdh_buf X, wdh_buf Y, int64_t outer, int len);
+/* LayerNormalization over the last axis (ONNX opset 17, biased variance).
+ * The reference has no such operator on any backend; this is what the
+ * decomposed ReduceMean/Sub/Pow/Sqrt/Div/Mul/Add subgraph
+ * (operators/cpu/operators/standard/reduce.ts:369-405 + binary7/unary)
+ * computes.  Gamma/Beta are [len] or 0 (1 / 0 respectively). */
+int wdh_layernorm(wdh_buf X, wdh_buf Gamma, wdh_buf Beta, wdh_buf Y,
+                  int64_t outer, int len, float eps);
+/* ReduceMean over the trailing `len` elements of each of `outer` rows;
+ * replaces ReduceMean (reduce.ts:369-405) for trailing-axes reductions. */
+int wdh_reduce_mean(wdh_buf X, wdh_buf Y, int64_t outer, int len);
+
+/* ---- pooling -------------------------------------------------------------
+ * Replaces CpuMaxPool.maxpool (operators/cpu/operators/standard/maxpool.ts:58-112);
+ * pads/out sizes come from MaxPool.calcShape (operators/base/maxpool.ts:32-137).
+ * Cells outside the input are skipped; a window with no valid cell yields -inf. */
+int wdh_maxpool2d(wdh_buf X, wdh_buf Y, int n, int c, int h, int w, int oh,
+                  int ow, int kh, int kw, int pt, int pl, int sh, int sw,
+                  int dh, int dw);
+/* Replaces CpuGlobalAveragePool.run (globalaveragepool.ts:12-41) +
+ * averagepool() (rawcomputation/averagepool.ts:1-46): Y[nc] = mean over hw. */
+int wdh_global_avgpool(wdh_buf X, wdh_buf Y, int64_t nc, int hw);
+
+/* ---- layout --------------------------------------------------------------
+ * Replaces CPUTranspose.copyNd (operators/cpu/operators/standard/transpose.ts:46-168):
+ * Y[dense index over out_shape] = X[sum_i idx_i * in_strides[i]];
+ * ndim <= 6; elem_bytes must be 4. */
+int wdh_transpose(wdh_buf X, wdh_buf Y, int ndim, const int32_t *out_shape,
+                  const int64_t *in_strides);
+/* Replaces Gather (operators/cpu/operators/standard/gather.ts:20-33), widened
+ * to the general axis form: data viewed as [outer, axis_len, inner], int32
+ * indices[n_idx] (negative indices wrap once) -> Y [outer, n_idx, inner]. */
+int wdh_gather(wdh_buf Data, wdh_buf Indices, wdh_buf Y, int64_t outer,
+               int axis_len, int64_t inner, int64_t n_idx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WEBDNN_HIP_H_ */

@@ -1,0 +1,282 @@
+"""TEST INFRASTRUCTURE ONLY — numpy face of the CPU oracle (oracle/webdnn_cpu_ref.c).
+
+Only tests/, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py`` may import this module; the product (``webdnn_amd``) never does.
+
+Each function takes ONNX-level arguments (numpy arrays + attributes) like the
+reference operator it restates, returns a new numpy array, and raises
+``RefThrows`` where the reference operator throws.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "liboracle.so")
+
+
+class RefThrows(Exception):
+    """The reference operator would throw for these arguments."""
+
+
+def build():
+    subprocess.run(["make", "-C", _HERE, "-s", "-B"], check=True)
+    return _LIB_PATH
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    return ctypes.CDLL(_LIB_PATH)
+
+
+_lib = _load()
+_i64p = ctypes.POINTER(ctypes.c_int64)
+_vp = ctypes.c_void_p
+
+
+def set_threads(n):
+    """OpenMP threads for the outer loops (results do not depend on it)."""
+    _lib.ref_set_threads(int(n))
+
+
+def _dims(shape):
+    arr = (ctypes.c_int64 * max(len(shape), 1))(*[int(s) for s in shape])
+    return arr, len(shape)
+
+
+def _ints(values):
+    values = list(values) if values is not None else []
+    arr = (ctypes.c_int64 * max(len(values), 1))(*[int(v) for v in values])
+    return arr, len(values)
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_vp) if a is not None else None
+
+
+def _check(rc, what):
+    if rc == -2:
+        raise MemoryError(what)
+    if rc < 0:
+        raise RefThrows(what)
+    return rc
+
+
+def gemm(A, B, C=None, alpha=1.0, beta=1.0, transA=0, transB=0):
+    A, B = _f32(A), _f32(B)
+    C = _f32(C) if C is not None else None
+    dA, nA = _dims(A.shape)
+    dB, nB = _dims(B.shape)
+    dC, nC = _dims(C.shape) if C is not None else _dims(())
+    m, n = ctypes.c_int64(), ctypes.c_int64()
+    # attributes are fp32 in the ONNX file, read back as JS doubles
+    alpha = float(np.float32(alpha))
+    beta = float(np.float32(beta))
+    args = lambda y: (_ptr(A), dA, nA, _ptr(B), dB, nB, _ptr(C), dC, nC,
+                      ctypes.c_double(alpha), ctypes.c_double(beta), int(transA), int(transB),
+                      y, ctypes.byref(m), ctypes.byref(n))
+    _check(_lib.ref_gemm(*args(None)), "Gemm: shape")
+    Y = np.empty((m.value, n.value), dtype=np.float32)
+    _check(_lib.ref_gemm(*args(_ptr(Y))), "Gemm")
+    return Y
+
+
+def matmul(A, B):
+    A, B = _f32(A), _f32(B)
+    dA, nA = _dims(A.shape)
+    dB, nB = _dims(B.shape)
+    out = (ctypes.c_int64 * 8)()
+    nd = _check(_lib.ref_matmul(_ptr(A), dA, nA, _ptr(B), dB, nB, None, out), "MatMul: shape")
+    Y = np.empty(tuple(out[i] for i in range(nd)), dtype=np.float32)
+    _check(_lib.ref_matmul(_ptr(A), dA, nA, _ptr(B), dB, nB, _ptr(Y), out), "MatMul")
+    return Y
+
+
+def conv(X, W, B=None, dilations=None, group=1, kernel_shape=None, pads=None, strides=None):
+    X, W = _f32(X), _f32(W)
+    B = _f32(B) if B is not None else None
+    dX, nX = _dims(X.shape)
+    dW, _ = _dims(W.shape)
+    dil, ndil = _ints(dilations)
+    ks, nks = _ints(kernel_shape)
+    pd, npd = _ints(pads)
+    st, nst = _ints(strides)
+    out = (ctypes.c_int64 * 4)()
+    args = lambda y: (_ptr(X), dX, nX, _ptr(W), dW, _ptr(B), dil, ndil, ctypes.c_int64(group),
+                      ks, nks, pd, npd, st, nst, y, out)
+    _check(_lib.ref_conv(*args(None)), "Conv: shape")
+    Y = np.empty(tuple(out[i] for i in range(4)), dtype=np.float32)
+    _check(_lib.ref_conv(*args(_ptr(Y))), "Conv")
+    return Y
+
+
+_BIN = {"Add": 0, "Sub": 1, "Mul": 2, "Div": 3, "Pow": 4}
+
+
+def binary(op, L, R):
+    L, R = np.ascontiguousarray(L), np.ascontiguousarray(R)
+    if L.dtype != R.dtype:
+        raise RefThrows("Binary: input dataTypes mismatch")
+    if L.dtype == np.float32:
+        dtype = 0
+    elif L.dtype == np.int32:
+        dtype = 1
+    else:
+        raise RefThrows("Binary: dataType not supported")
+    dL, nL = _dims(L.shape)
+    dR, nR = _dims(R.shape)
+    out = (ctypes.c_int64 * 8)()
+    nd = _check(_lib.ref_binary(_BIN[op], dtype, _ptr(L), dL, nL, _ptr(R), dR, nR, None, out),
+                "Binary: broadcast")
+    Y = np.empty(tuple(out[i] for i in range(nd)), dtype=L.dtype)
+    _check(_lib.ref_binary(_BIN[op], dtype, _ptr(L), dL, nL, _ptr(R), dR, nR, _ptr(Y), out), "Binary")
+    return Y
+
+
+_UN = {"Relu": 0, "Sigmoid": 1, "Sqrt": 2, "Exp": 3, "Tanh": 4, "Abs": 5, "Neg": 6, "Reciprocal": 7}
+
+
+def unary(op, X):
+    X = np.ascontiguousarray(X)
+    if X.dtype == np.float32:
+        dtype = 0
+    elif X.dtype == np.int32:
+        dtype = 1
+    else:
+        raise RefThrows("Unary: DataType not supported")
+    Y = np.empty_like(X)
+    _check(_lib.ref_unary(_UN[op], dtype, _ptr(X), _ptr(Y), ctypes.c_int64(X.size)), "Unary")
+    return Y
+
+
+def softmax(X, axis=-1):
+    X = _f32(X)
+    d, n = _dims(X.shape)
+    Y = np.empty_like(X)
+    _check(_lib.ref_softmax(_ptr(X), d, n, ctypes.c_int64(axis), _ptr(Y)), "Softmax")
+    return Y
+
+
+_AUTO_PAD = {"NOTSET": 0, "SAME_UPPER": 1, "SAME_LOWER": 2, "VALID": 3}
+
+
+def maxpool(X, kernel_shape, auto_pad="NOTSET", ceil_mode=0, dilations=None, pads=None,
+            strides=None, n_outputs=1, return_pads=False):
+    X = _f32(X)
+    if auto_pad not in _AUTO_PAD:
+        raise RefThrows("Unknown auto_pad")
+    dX, nX = _dims(X.shape)
+    dil, ndil = _ints(dilations)
+    ks, _ = _ints(kernel_shape)
+    pd, npd = _ints(pads)
+    st, nst = _ints(strides)
+    out = (ctypes.c_int64 * 4)()
+    pads_out = (ctypes.c_int64 * 4)()
+    args = lambda y: (_ptr(X), dX, nX, _AUTO_PAD[auto_pad], int(ceil_mode), dil, ndil, ks, pd, npd,
+                      st, nst, int(n_outputs), y, out, pads_out)
+    _check(_lib.ref_maxpool(*args(None)), "MaxPool: shape")
+    Y = np.empty(tuple(out[i] for i in range(4)), dtype=np.float32)
+    _check(_lib.ref_maxpool(*args(_ptr(Y))), "MaxPool")
+    if return_pads:
+        return Y, [pads_out[i] for i in range(4)]
+    return Y
+
+
+def global_average_pool(X):
+    X = _f32(X)
+    d, n = _dims(X.shape)
+    if n != 4:
+        raise RefThrows("GlobalAveragePool other than 2D")
+    Y = np.empty((X.shape[0], X.shape[1], 1, 1), dtype=np.float32)
+    _check(_lib.ref_global_average_pool(_ptr(X), d, n, _ptr(Y)), "GlobalAveragePool")
+    return Y
+
+
+def transpose(X, perm=None):
+    X = np.ascontiguousarray(X)
+    assert X.dtype.itemsize == 4
+    d, n = _dims(X.shape)
+    pm, npm = _ints(perm)
+    out = (ctypes.c_int64 * 8)()
+    _check(_lib.ref_transpose(None, d, n, pm, npm, None, out), "Transpose: shape")
+    Y = np.empty(tuple(out[i] for i in range(n)), dtype=X.dtype)
+    _check(_lib.ref_transpose(_ptr(X), d, n, pm, npm, _ptr(Y), out), "Transpose")
+    return Y
+
+
+def reduce_mean_last(X):
+    """ReduceMean over the last axis, keepdims=1."""
+    X = _f32(X)
+    length = X.shape[-1]
+    outer = X.size // length if length else 0
+    Y = np.empty(X.shape[:-1] + (1,), dtype=np.float32)
+    _check(_lib.ref_reduce_mean_trailing(_ptr(X), ctypes.c_int64(outer), ctypes.c_int64(length),
+                                         _ptr(Y)), "ReduceMean")
+    return Y
+
+
+def gather(data, indices, axis=0):
+    data = np.ascontiguousarray(data)
+    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    Y = np.empty((), dtype=data.dtype)
+    _check(_lib.ref_gather(_ptr(data), data.ndim, _ptr(indices), indices.ndim,
+                           ctypes.c_int64(axis), _ptr(Y)), "Gather")
+    return Y
+
+
+def layernorm_decomposed(X, gamma=None, beta=None, eps=1e-5):
+    X = _f32(X)
+    gamma = _f32(gamma) if gamma is not None else None
+    beta = _f32(beta) if beta is not None else None
+    length = X.shape[-1]
+    outer = X.size // length if length else 0
+    Y = np.empty_like(X)
+    _check(_lib.ref_layernorm_decomposed(_ptr(X), ctypes.c_int64(outer), ctypes.c_int64(length),
+                                         _ptr(gamma), _ptr(beta), ctypes.c_float(eps), _ptr(Y)),
+           "LayerNormalization")
+    return Y
+
+
+def flatten(X, axis=1):
+    """operators/base/flatten.ts:7-17 + cpu flatten.ts:11-20 (shares the buffer)."""
+    if axis != 1:
+        raise RefThrows("Flatten: only axis === 1 is supported")
+    X = np.asarray(X)
+    return X.reshape(X.shape[0], int(np.prod(X.shape[1:], dtype=np.int64)))
+
+
+def reshape(X, shape, allowzero=0):
+    """operators/base/reshape5.ts:16-75, written out (no numpy -1 inference)."""
+    X = np.asarray(X)
+    shape = [int(s) for s in np.asarray(shape).reshape(-1)]
+    explicit, minus = 1, -1
+    for i, s in enumerate(shape):
+        if s > 0:
+            explicit *= s
+        elif s == 0 and not allowzero:
+            explicit *= X.shape[i]
+        elif s == -1:
+            if minus >= 0:
+                raise RefThrows("Reshape: multiple -1 dimensions")
+            minus = i
+        elif s < -1:
+            raise RefThrows("Reshape: negative dimension")
+    if minus >= 0 and explicit <= 0:
+        raise RefThrows("Reshape: cannot infer -1")
+    out = []
+    for i, s in enumerate(shape):
+        if s > 0 or (s == 0 and allowzero):
+            out.append(s)
+        elif s == 0:
+            out.append(X.shape[i])
+        else:
+            out.append(X.size // explicit)
+    return X.reshape(out)

@@ -1,0 +1,81 @@
+"""Builds the native pieces of the hip backend in-tree.
+
+  libwebdnn_hip.so   HIP kernels + C ABI (include/webdnn_hip.h), gfx950 only
+  webdnn_hip.node    N-API addon that exposes the C ABI to the Node.js host
+
+Run as ``python -m webdnn_amd.build``.  hipcc cross-compiles for gfx950, so no
+GPU is needed to build.
+"""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "webdnn_amd", "csrc")
+LIBDIR = os.path.join(ROOT, "webdnn_amd", "lib")
+LIB = os.path.join(LIBDIR, "libwebdnn_hip.so")
+ADDON_SRC = os.path.join(ROOT, "webdnn_amd", "napi", "addon.c")
+ADDON = os.path.join(LIBDIR, "webdnn_hip.node")
+
+HIP_SOURCES = ["runtime.hip", "gemm.hip", "elementwise.hip", "reduce.hip", "pool_layout.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    # fp32 add/mul must not fuse: Add/Mul results are compared bit for bit
+    "-ffp-contract=off",
+    # packed fp32 instructions are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    if out.strip():
+        print(out)
+
+
+def build_library(verbose=True):
+    os.makedirs(LIBDIR, exist_ok=True)
+    objs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
+        cmd = ["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+               "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print("[build] hipcc", src)
+        _run(cmd)
+        objs.append(obj)
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
+    for obj in objs:
+        os.remove(obj)
+    return LIB
+
+
+def build_addon(verbose=True):
+    if not os.path.exists(ADDON_SRC):
+        return None
+    if verbose:
+        print("[build] gcc addon.c")
+    _run(["gcc", "-O2", "-fPIC", "-shared", "-std=c11", "-Wall",
+          "-I", "/usr/include/node", "-I", os.path.join(ROOT, "include"),
+          ADDON_SRC, "-o", ADDON, "-ldl"])
+    return ADDON
+
+
+def build_all(verbose=True):
+    lib = build_library(verbose)
+    addon = build_addon(verbose)
+    return lib, addon
+
+
+if __name__ == "__main__":
+    build_all()
+    print("built", LIB)
+    sys.exit(0)

@@ -1,0 +1,55 @@
+// Internal helpers shared by the translation units of libwebdnn_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "webdnn_hip.h"
+
+namespace wdh {
+
+// Records `code` + a printf-style message as the calling thread's last error
+// and returns `code`, so call sites can `return fail(...)`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+bool initialised();
+hipStream_t stream();
+int compute_units();
+
+// Handle -> device pointer.  Returns nullptr (and records WDH_EINVAL) for an
+// unknown handle.  A zero-byte buffer resolves to a non-null dummy pointer.
+void *resolve(wdh_buf h, size_t *bytes);
+
+// Resolves `h` and checks that it holds at least `need` bytes.
+// On failure returns false after recording the error (`what` names the operand).
+bool operand(wdh_buf h, size_t need, const char *what, void **out);
+
+// Frees the per-geometry tap tables of the conv kernel (called at shutdown).
+void release_conv_tables();
+
+}  // namespace wdh
+
+#define WDH_REQUIRE_INIT()                                                   \
+  do {                                                                       \
+    if (!wdh::initialised())                                                 \
+      return wdh::fail(WDH_ESTATE, "%s: wdh_init() has not succeeded",       \
+                       __func__);                                            \
+  } while (0)
+
+#define WDH_HIP_CHECK(expr)                                                  \
+  do {                                                                       \
+    hipError_t e_ = (expr);                                                  \
+    if (e_ != hipSuccess)                                                    \
+      return wdh::fail(WDH_EHIP, "%s: %s failed: %s", __func__, #expr,       \
+                       hipGetErrorString(e_));                               \
+  } while (0)
+
+// Checked after every kernel launch: catches bad launch configurations.
+#define WDH_LAUNCH_CHECK()                                                   \
+  do {                                                                       \
+    hipError_t e_ = hipGetLastError();                                       \
+    if (e_ != hipSuccess)                                                    \
+      return wdh::fail(WDH_EHIP, "%s: kernel launch failed: %s", __func__,   \
+                       hipGetErrorString(e_));                               \
+  } while (0)

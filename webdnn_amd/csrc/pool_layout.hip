@@ -1,0 +1,276 @@
+// MaxPool (2-D, NCHW), Transpose (rank <= 6 gather-copy) and Gather.
+// All three move bytes without arithmetic on them, so results are bit-exact.
+//
+// Reference semantics:
+//   MaxPool   : src/descriptor_runner/operators/cpu/operators/standard/maxpool.ts:58-112
+//   Transpose : src/descriptor_runner/operators/cpu/operators/standard/transpose.ts:46-168
+//   Gather    : src/descriptor_runner/operators/cpu/operators/standard/gather.ts:20-33
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int MAXD = 6;
+
+// ---- max pooling -------------------------------------------------------------
+// One thread per output cell, consecutive threads along ow, so stores are
+// coalesced and the overlapping input windows of neighbouring threads are
+// served by the vector L1.
+struct PoolParams {
+  const float *X;
+  float *Y;
+  long long total;  // n*c*oh*ow
+  int h, w, oh, ow, kh, kw, pt, pl, sh, sw, dh, dw;
+};
+
+__global__ __launch_bounds__(256) void maxpool2d_kernel(PoolParams p) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
+       i += stride) {
+    const int ox = (int)(i % p.ow);
+    const long long t = i / p.ow;
+    const int oy = (int)(t % p.oh);
+    const long long plane = t / p.oh;  // n*c + c
+    const float *x = p.X + plane * p.h * p.w;
+    float mv = -INFINITY;
+    for (int ky = 0; ky < p.kh; ky++) {
+      const int iy = oy * p.sh - p.pt + ky * p.dh;
+      if ((unsigned)iy >= (unsigned)p.h) continue;
+      for (int kx = 0; kx < p.kw; kx++) {
+        const int ix = ox * p.sw - p.pl + kx * p.dw;
+        if ((unsigned)ix >= (unsigned)p.w) continue;
+        const float v = x[iy * p.w + ix];
+        if (v > mv) mv = v;  // strict, NaN never selected: maxpool.ts:98-101
+      }
+    }
+    p.Y[i] = mv;
+  }
+}
+
+// ---- transpose -----------------------------------------------------------------
+struct GatherCopyParams {
+  const uint32_t *X;
+  uint32_t *Y;
+  long long total;
+  int ndim;
+  unsigned shape[MAXD];   // output shape
+  long long sin[MAXD];    // input stride of each output axis
+};
+
+// Generic: thread per output element.  Coalesced on the output side always,
+// on the input side when the last output axis has input stride 1.
+__global__ __launch_bounds__(256) void gather_copy_kernel(GatherCopyParams p) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
+       i += stride) {
+    long long rem = i, off = 0;
+#pragma unroll
+    for (int d = MAXD - 1; d >= 0; d--) {
+      if (d < p.ndim) {
+        long long q = rem / p.shape[d];
+        off += (rem - q * p.shape[d]) * p.sin[d];
+        rem = q;
+      }
+    }
+    p.Y[i] = p.X[off];
+  }
+}
+
+// Tiled: when the input-contiguous axis `a` is not the last output axis, a
+// workgroup moves a 64x64 tile spanned by (axis a, last axis) through LDS:
+// reads run along axis a (contiguous in X), writes along the last axis
+// (contiguous in Y).  The 65-float row pitch keeps both phases free of bank
+// conflicts.  All remaining axes are folded into blockIdx.z.
+struct TileParams {
+  const uint32_t *X;
+  uint32_t *Y;
+  int ndim;               // number of "outer" axes (excluding a and last)
+  unsigned oshape[MAXD];  // extents of the outer axes
+  long long osin[MAXD];   // their input strides
+  long long osout[MAXD];  // their output strides
+  unsigned na, nl;        // extents of axis a and of the last axis
+  long long a_out;        // output stride of axis a (its input stride is 1)
+  long long l_in;         // input stride of the last axis (its output stride is 1)
+};
+
+__global__ __launch_bounds__(256) void transpose_tiled_kernel(TileParams p) {
+  __shared__ uint32_t tile[64][65];
+  long long rem = blockIdx.z, in_off = 0, out_off = 0;
+#pragma unroll
+  for (int d = MAXD - 1; d >= 0; d--) {
+    if (d < p.ndim) {
+      long long q = rem / p.oshape[d];
+      long long c = rem - q * p.oshape[d];
+      rem = q;
+      in_off += c * p.osin[d];
+      out_off += c * p.osout[d];
+    }
+  }
+  const unsigned a0 = blockIdx.x * 64, l0 = blockIdx.y * 64;
+  const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  // read: tx runs along axis a
+  for (unsigned r = ty; r < 64; r += 4) {
+    unsigned a = a0 + tx, l = l0 + r;
+    if (a < p.na && l < p.nl) tile[r][tx] = p.X[in_off + (long long)l * p.l_in + a];
+  }
+  __syncthreads();
+  // write: tx runs along the last axis
+  for (unsigned r = ty; r < 64; r += 4) {
+    unsigned a = a0 + r, l = l0 + tx;
+    if (a < p.na && l < p.nl) p.Y[out_off + (long long)a * p.a_out + l] = tile[tx][r];
+  }
+}
+
+__global__ __launch_bounds__(256) void gather_axis_kernel(
+    const uint32_t *__restrict__ D, const int *__restrict__ Idx,
+    uint32_t *__restrict__ Y, long long outer, int axis_len, long long inner,
+    long long n_idx) {
+  const long long total = outer * n_idx * inner;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += stride) {
+    long long in = i % inner;
+    long long t = i / inner;
+    long long j = t % n_idx;
+    long long o = t / n_idx;
+    int ix = Idx[j];
+    if (ix < 0) ix += axis_len;
+    // out-of-range indices read element 0 rather than stray memory
+    if (ix < 0 || ix >= axis_len) ix = 0;
+    Y[i] = D[(o * axis_len + ix) * inner + in];
+  }
+}
+
+unsigned grid_for(long long items) {
+  long long blocks = (items + 255) / 256;
+  long long cap = (long long)wdh::compute_units() * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+}  // namespace
+
+using wdh::fail;
+
+extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
+                             int oh, int ow, int kh, int kw, int pt, int pl, int sh,
+                             int sw, int dh, int dw) {
+  WDH_REQUIRE_INIT();
+  if (n < 0 || c < 0 || h <= 0 || w <= 0 || oh < 0 || ow < 0 || kh <= 0 || kw <= 0 ||
+      sh <= 0 || sw <= 0 || dh <= 0 || dw <= 0 || pt < 0 || pl < 0)
+    return fail(WDH_EINVAL, "wdh_maxpool2d: bad geometry");
+  // every input read is bounds-checked in the kernel, so an (oh, ow) larger than
+  // the geometry implies only yields windows that lie in the padding (-inf)
+  PoolParams p;
+  p.total = (long long)n * c * oh * ow;
+  if (p.total == 0) return WDH_OK;
+  void *px, *py;
+  if (!wdh::operand(hX, (size_t)n * c * h * w * 4, "wdh_maxpool2d: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)p.total * 4, "wdh_maxpool2d: Y", &py)) return WDH_EINVAL;
+  p.X = (const float *)px; p.Y = (float *)py;
+  p.h = h; p.w = w; p.oh = oh; p.ow = ow; p.kh = kh; p.kw = kw;
+  p.pt = pt; p.pl = pl; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(p.total)), dim3(256), 0,
+                     wdh::stream(), p);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
+                             const int32_t *out_shape, const int64_t *in_strides) {
+  WDH_REQUIRE_INIT();
+  if (ndim < 0 || ndim > MAXD)
+    return fail(WDH_EINVAL, "wdh_transpose: ndim %d outside 0..%d", ndim, MAXD);
+  if (ndim > 0 && (!out_shape || !in_strides))
+    return fail(WDH_EINVAL, "wdh_transpose: NULL shape or strides");
+  // drop extent-1 axes; merge neighbours that are contiguous in the input
+  unsigned shape[MAXD];
+  long long sin[MAXD];
+  int nd = 0;
+  long long total = 1, span = 1;
+  for (int d = 0; d < ndim; d++) {
+    if (out_shape[d] < 0 || in_strides[d] < 0)
+      return fail(WDH_EINVAL, "wdh_transpose: negative extent or stride");
+    total *= out_shape[d];
+    if (out_shape[d] == 1) continue;
+    span += (long long)(out_shape[d] - 1) * in_strides[d];
+    if (nd > 0 && sin[nd - 1] == in_strides[d] * out_shape[d] &&
+        (unsigned long long)shape[nd - 1] * out_shape[d] <= 0xffffffffULL) {
+      shape[nd - 1] *= out_shape[d];
+      sin[nd - 1] = in_strides[d];
+    } else {
+      shape[nd] = out_shape[d];
+      sin[nd] = in_strides[d];
+      nd++;
+    }
+  }
+  if (total == 0) return WDH_OK;
+  void *px, *py;
+  if (!wdh::operand(hX, (size_t)span * 4, "wdh_transpose: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)total * 4, "wdh_transpose: Y", &py)) return WDH_EINVAL;
+  hipStream_t st = wdh::stream();
+  if (nd <= 1 && (nd == 0 || sin[0] == 1)) {  // identity permutation
+    WDH_HIP_CHECK(hipMemcpyAsync(py, px, (size_t)total * 4, hipMemcpyDeviceToDevice, st));
+    return WDH_OK;
+  }
+  // output strides of the collapsed axes
+  long long sout[MAXD];
+  {
+    long long acc = 1;
+    for (int d = nd - 1; d >= 0; d--) { sout[d] = acc; acc *= shape[d]; }
+  }
+  int a = -1;
+  for (int d = 0; d < nd; d++)
+    if (sin[d] == 1) a = d;
+  if (a >= 0 && a != nd - 1 && shape[a] >= 16 && shape[nd - 1] >= 16) {
+    TileParams t = {};
+    t.X = (const uint32_t *)px; t.Y = (uint32_t *)py;
+    long long nouter = 1;
+    for (int d = 0; d < nd - 1; d++) {
+      if (d == a) continue;
+      t.oshape[t.ndim] = shape[d];
+      t.osin[t.ndim] = sin[d];
+      t.osout[t.ndim] = sout[d];
+      t.ndim++;
+      nouter *= shape[d];
+    }
+    t.na = shape[a]; t.nl = shape[nd - 1];
+    t.a_out = sout[a]; t.l_in = sin[nd - 1];
+    unsigned gx = (t.na + 63) / 64, gy = (t.nl + 63) / 64;
+    if (nouter <= 65535 && gy <= 65535) {
+      hipLaunchKernelGGL(transpose_tiled_kernel, dim3(gx, gy, (unsigned)nouter),
+                         dim3(256), 0, st, t);
+      WDH_LAUNCH_CHECK();
+      return WDH_OK;
+    }
+  }
+  GatherCopyParams g = {};
+  g.X = (const uint32_t *)px; g.Y = (uint32_t *)py;
+  g.total = total; g.ndim = nd;
+  for (int d = 0; d < nd; d++) { g.shape[d] = shape[d]; g.sin[d] = sin[d]; }
+  hipLaunchKernelGGL(gather_copy_kernel, dim3(grid_for(total)), dim3(256), 0, st, g);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+extern "C" int wdh_gather(wdh_buf hD, wdh_buf hI, wdh_buf hY, int64_t outer,
+                          int axis_len, int64_t inner, int64_t n_idx) {
+  WDH_REQUIRE_INIT();
+  if (outer < 0 || axis_len < 0 || inner < 0 || n_idx < 0)
+    return fail(WDH_EINVAL, "wdh_gather: negative extent");
+  const long long total = (long long)outer * n_idx * inner;
+  if (total == 0) return WDH_OK;
+  if (axis_len == 0) return fail(WDH_EINVAL, "wdh_gather: empty axis");
+  void *pd, *pi, *py;
+  if (!wdh::operand(hD, (size_t)outer * axis_len * inner * 4, "wdh_gather: Data", &pd)) return WDH_EINVAL;
+  if (!wdh::operand(hI, (size_t)n_idx * 4, "wdh_gather: Indices", &pi)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)total * 4, "wdh_gather: Y", &py)) return WDH_EINVAL;
+  hipLaunchKernelGGL(gather_axis_kernel, dim3(grid_for(total)), dim3(256), 0,
+                     wdh::stream(), (const uint32_t *)pd, (const int *)pi,
+                     (uint32_t *)py, (long long)outer, axis_len, (long long)inner,
+                     (long long)n_idx);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}

@@ -1,0 +1,404 @@
+// Runtime of libwebdnn_hip.so: device selection, the single stream, the
+// handle table, a size-bucketed device-memory pool, pinned staging for
+// host<->device copies, and event timing.
+//
+// Stands in for the WASM worker's buffer-id protocol of the reference
+// (src/descriptor_runner/backend/wasm/wasmContextImpl.ts:113-163,
+//  src/shader/wasm/pre.js:4-91, src/shader/wasm/src/core/allocation.cpp:4-15).
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+constexpr size_t kStagingBytes = 32u << 20;  // per pinned buffer, two of them
+constexpr size_t kSmallGranule = 512;        // allocation rounding below 1 MiB
+constexpr size_t kLargeGranule = 1u << 20;   // and above
+
+thread_local char g_error[512] = "";
+
+struct Slot {
+  void *ptr = nullptr;   // nullptr => slot is free
+  size_t bytes = 0;      // bytes the caller asked for
+  size_t cap = 0;        // bytes of the underlying block
+};
+
+struct Runtime {
+  bool ready = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t prop;
+  // handle table; handle = index + 1
+  std::vector<Slot> slots;
+  std::vector<int64_t> free_slots;
+  // pool: capacity -> cached blocks
+  std::multimap<size_t, void *> cache;
+  uint64_t in_use = 0, cached = 0, reserved = 0, peak = 0;
+  // pinned staging, ping-pong
+  void *stage[2] = {nullptr, nullptr};
+  hipEvent_t stage_done[2] = {nullptr, nullptr};
+  bool stage_busy[2] = {false, false};
+  // timing events, created lazily
+  hipEvent_t events[WDH_MAX_EVENTS] = {};
+  // one-element dummy so that zero-byte buffers have a valid address
+  void *dummy = nullptr;
+};
+
+Runtime g;
+
+size_t round_up(size_t bytes) {
+  if (bytes == 0) return kSmallGranule;
+  size_t gran = bytes < (1u << 20) ? kSmallGranule : kLargeGranule;
+  return (bytes + gran - 1) / gran * gran;
+}
+
+void release_cache(size_t keep) {
+  // Blocks may still be referenced by enqueued work: drain the stream first.
+  if (g.cached <= keep) return;
+  (void)hipStreamSynchronize(g.stream);
+  for (auto it = g.cache.begin(); it != g.cache.end() && g.cached > keep;) {
+    (void)hipFree(it->second);
+    g.cached -= it->first;
+    g.reserved -= it->first;
+    it = g.cache.erase(it);
+  }
+}
+
+}  // namespace
+
+namespace wdh {
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void clear_error() { g_error[0] = '\0'; }
+bool initialised() { return g.ready; }
+hipStream_t stream() { return g.stream; }
+int compute_units() { return g.prop.multiProcessorCount; }
+
+void *resolve(wdh_buf h, size_t *bytes) {
+  if (h <= 0 || (size_t)h > g.slots.size() || g.slots[h - 1].ptr == nullptr) {
+    fail(WDH_EINVAL, "unknown buffer handle %lld", (long long)h);
+    return nullptr;
+  }
+  const Slot &s = g.slots[h - 1];
+  if (bytes) *bytes = s.bytes;
+  return s.ptr;
+}
+
+bool operand(wdh_buf h, size_t need, const char *what, void **out) {
+  size_t have = 0;
+  void *p = resolve(h, &have);
+  if (!p) {
+    char prev[400];
+    snprintf(prev, sizeof(prev), "%s", g_error);
+    fail(WDH_EINVAL, "%s: %s", what, prev);
+    return false;
+  }
+  if (have < need) {
+    fail(WDH_EINVAL, "%s: buffer holds %zu bytes, operation needs %zu", what,
+         have, need);
+    return false;
+  }
+  *out = p;
+  return true;
+}
+
+}  // namespace wdh
+
+using wdh::fail;
+
+extern "C" {
+
+const char *wdh_last_error(void) { return g_error; }
+
+int wdh_init(int device) {
+  if (g.ready) {
+    if (device == g.device) return WDH_OK;
+    return fail(WDH_EINVAL, "wdh_init: already initialised on device %d",
+                g.device);
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return fail(WDH_ENODEV, "wdh_init: no HIP device (%s)",
+                e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+  }
+  if (device < 0 || device >= count)
+    return fail(WDH_ENODEV, "wdh_init: device %d out of range (have %d)",
+                device, count);
+  WDH_HIP_CHECK(hipSetDevice(device));
+  WDH_HIP_CHECK(hipGetDeviceProperties(&g.prop, device));
+  if (strncmp(g.prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(WDH_ENODEV,
+                "wdh_init: device %d is %s; this library holds gfx950 code only",
+                device, g.prop.gcnArchName);
+  WDH_HIP_CHECK(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
+  for (int i = 0; i < 2; i++) {
+    if (hipHostMalloc(&g.stage[i], kStagingBytes, hipHostMallocDefault) !=
+        hipSuccess)
+      return fail(WDH_ENOMEM, "wdh_init: pinned staging allocation failed");
+    WDH_HIP_CHECK(
+        hipEventCreateWithFlags(&g.stage_done[i], hipEventDisableTiming));
+    g.stage_busy[i] = false;
+  }
+  WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
+  g.device = device;
+  g.ready = true;
+  wdh::clear_error();
+  return WDH_OK;
+}
+
+void wdh_shutdown(void) {
+  if (!g.ready) return;
+  (void)hipStreamSynchronize(g.stream);
+  wdh::release_conv_tables();
+  for (auto &s : g.slots)
+    if (s.ptr && s.ptr != g.dummy) (void)hipFree(s.ptr);
+  g.slots.clear();
+  g.free_slots.clear();
+  for (auto &kv : g.cache) (void)hipFree(kv.second);
+  g.cache.clear();
+  g.in_use = g.cached = g.reserved = g.peak = 0;
+  for (int i = 0; i < 2; i++) {
+    if (g.stage[i]) (void)hipHostFree(g.stage[i]);
+    if (g.stage_done[i]) (void)hipEventDestroy(g.stage_done[i]);
+    g.stage[i] = nullptr;
+    g.stage_done[i] = nullptr;
+  }
+  for (auto &ev : g.events) {
+    if (ev) (void)hipEventDestroy(ev);
+    ev = nullptr;
+  }
+  if (g.dummy) (void)hipFree(g.dummy);
+  g.dummy = nullptr;
+  (void)hipStreamDestroy(g.stream);
+  g.stream = nullptr;
+  g.ready = false;
+  g.device = -1;
+}
+
+int wdh_device_info(char *name, int name_cap, int *compute_units,
+                    int *clock_mhz, uint64_t *hbm_bytes) {
+  WDH_REQUIRE_INIT();
+  if (name && name_cap > 0) snprintf(name, name_cap, "%s", g.prop.gcnArchName);
+  if (compute_units) *compute_units = g.prop.multiProcessorCount;
+  if (clock_mhz) *clock_mhz = g.prop.clockRate / 1000;
+  if (hbm_bytes) *hbm_bytes = g.prop.totalGlobalMem;
+  return WDH_OK;
+}
+
+wdh_buf wdh_alloc(size_t bytes) {
+  if (!g.ready) {
+    fail(WDH_ESTATE, "wdh_alloc: wdh_init() has not succeeded");
+    return 0;
+  }
+  Slot s;
+  s.bytes = bytes;
+  if (bytes == 0) {
+    s.ptr = g.dummy;
+    s.cap = 0;
+  } else {
+    size_t cap = round_up(bytes);
+    auto it = g.cache.lower_bound(cap);
+    if (it != g.cache.end() && it->first <= cap + cap / 4) {
+      s.ptr = it->second;
+      s.cap = it->first;
+      g.cached -= s.cap;
+      g.cache.erase(it);
+    } else {
+      void *p = nullptr;
+      hipError_t e = hipMalloc(&p, cap);
+      if (e != hipSuccess) {
+        // give cached blocks back to the driver and retry once
+        (void)hipGetLastError();
+        release_cache(0);
+        e = hipMalloc(&p, cap);
+      }
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        fail(WDH_ENOMEM, "wdh_alloc: hipMalloc(%zu) failed: %s", cap,
+             hipGetErrorString(e));
+        return 0;
+      }
+      s.ptr = p;
+      s.cap = cap;
+      g.reserved += cap;
+      if (g.reserved > g.peak) g.peak = g.reserved;
+    }
+    g.in_use += s.cap;
+  }
+  int64_t idx;
+  if (!g.free_slots.empty()) {
+    idx = g.free_slots.back();
+    g.free_slots.pop_back();
+    g.slots[idx] = s;
+  } else {
+    idx = (int64_t)g.slots.size();
+    g.slots.push_back(s);
+  }
+  return idx + 1;
+}
+
+int wdh_free(wdh_buf h) {
+  WDH_REQUIRE_INIT();
+  if (h <= 0 || (size_t)h > g.slots.size() || g.slots[h - 1].ptr == nullptr)
+    return fail(WDH_EINVAL, "wdh_free: unknown buffer handle %lld",
+                (long long)h);
+  Slot &s = g.slots[h - 1];
+  if (s.cap) {
+    g.cache.emplace(s.cap, s.ptr);
+    g.cached += s.cap;
+    g.in_use -= s.cap;
+  }
+  s = Slot();
+  g.free_slots.push_back(h - 1);
+  return WDH_OK;
+}
+
+int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
+  WDH_REQUIRE_INIT();
+  size_t have = 0;
+  char *dst = (char *)wdh::resolve(h, &have);
+  if (!dst) return WDH_EINVAL;
+  if (dst_offset > have || bytes > have - dst_offset)
+    return fail(WDH_EINVAL, "wdh_write: %zu bytes at offset %zu exceed buffer of %zu",
+                bytes, dst_offset, have);
+  if (bytes && !src) return fail(WDH_EINVAL, "wdh_write: src is NULL");
+  const char *s = (const char *)src;
+  size_t done = 0;
+  int which = 0;
+  while (done < bytes) {
+    size_t chunk = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
+    if (g.stage_busy[which]) {
+      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[which]));
+      g.stage_busy[which] = false;
+    }
+    memcpy(g.stage[which], s + done, chunk);
+    WDH_HIP_CHECK(hipMemcpyAsync(dst + dst_offset + done, g.stage[which], chunk,
+                                 hipMemcpyHostToDevice, g.stream));
+    WDH_HIP_CHECK(hipEventRecord(g.stage_done[which], g.stream));
+    g.stage_busy[which] = true;
+    done += chunk;
+    which ^= 1;
+  }
+  return WDH_OK;
+}
+
+int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
+  WDH_REQUIRE_INIT();
+  size_t have = 0;
+  const char *src = (const char *)wdh::resolve(h, &have);
+  if (!src) return WDH_EINVAL;
+  if (src_offset > have || bytes > have - src_offset)
+    return fail(WDH_EINVAL, "wdh_read: %zu bytes at offset %zu exceed buffer of %zu",
+                bytes, src_offset, have);
+  if (bytes && !dst) return fail(WDH_EINVAL, "wdh_read: dst is NULL");
+  // staging buffers may still carry an in-flight upload
+  for (int i = 0; i < 2; i++)
+    if (g.stage_busy[i]) {
+      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[i]));
+      g.stage_busy[i] = false;
+    }
+  char *d = (char *)dst;
+  size_t issued = 0, copied = 0;
+  size_t chunk_of[2] = {0, 0};
+  int which = 0;
+  // ping-pong: the D2H of chunk i+1 overlaps the host memcpy of chunk i
+  if (bytes) {
+    chunk_of[0] = bytes < kStagingBytes ? bytes : kStagingBytes;
+    WDH_HIP_CHECK(hipMemcpyAsync(g.stage[0], src + src_offset, chunk_of[0],
+                                 hipMemcpyDeviceToHost, g.stream));
+    WDH_HIP_CHECK(hipEventRecord(g.stage_done[0], g.stream));
+    issued = chunk_of[0];
+  } else {
+    WDH_HIP_CHECK(hipStreamSynchronize(g.stream));
+  }
+  while (copied < bytes) {
+    int next = which ^ 1;
+    if (issued < bytes) {
+      chunk_of[next] =
+          bytes - issued < kStagingBytes ? bytes - issued : kStagingBytes;
+      WDH_HIP_CHECK(hipMemcpyAsync(g.stage[next], src + src_offset + issued,
+                                   chunk_of[next], hipMemcpyDeviceToHost,
+                                   g.stream));
+      WDH_HIP_CHECK(hipEventRecord(g.stage_done[next], g.stream));
+      issued += chunk_of[next];
+    }
+    WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[which]));
+    memcpy(d + copied, g.stage[which], chunk_of[which]);
+    copied += chunk_of[which];
+    which = next;
+  }
+  return WDH_OK;
+}
+
+int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
+             size_t bytes) {
+  WDH_REQUIRE_INIT();
+  size_t dhave = 0, shave = 0;
+  char *d = (char *)wdh::resolve(dst, &dhave);
+  if (!d) return WDH_EINVAL;
+  const char *s = (const char *)wdh::resolve(src, &shave);
+  if (!s) return WDH_EINVAL;
+  if (dst_offset > dhave || bytes > dhave - dst_offset || src_offset > shave ||
+      bytes > shave - src_offset)
+    return fail(WDH_EINVAL, "wdh_copy: range exceeds a buffer");
+  if (bytes)
+    WDH_HIP_CHECK(hipMemcpyAsync(d + dst_offset, s + src_offset, bytes,
+                                 hipMemcpyDeviceToDevice, g.stream));
+  return WDH_OK;
+}
+
+int wdh_sync(void) {
+  WDH_REQUIRE_INIT();
+  WDH_HIP_CHECK(hipStreamSynchronize(g.stream));
+  return WDH_OK;
+}
+
+int wdh_mem_stats(uint64_t *in_use, uint64_t *cached, uint64_t *peak) {
+  WDH_REQUIRE_INIT();
+  if (in_use) *in_use = g.in_use;
+  if (cached) *cached = g.cached;
+  if (peak) *peak = g.peak;
+  return WDH_OK;
+}
+
+int wdh_trim(size_t keep_bytes) {
+  WDH_REQUIRE_INIT();
+  release_cache(keep_bytes);
+  return WDH_OK;
+}
+
+int wdh_event_record(int id) {
+  WDH_REQUIRE_INIT();
+  if (id < 0 || id >= WDH_MAX_EVENTS)
+    return fail(WDH_EINVAL, "wdh_event_record: id %d out of range", id);
+  if (!g.events[id]) WDH_HIP_CHECK(hipEventCreate(&g.events[id]));
+  WDH_HIP_CHECK(hipEventRecord(g.events[id], g.stream));
+  return WDH_OK;
+}
+
+int wdh_event_elapsed_ms(int start_id, int stop_id, float *ms) {
+  WDH_REQUIRE_INIT();
+  if (start_id < 0 || start_id >= WDH_MAX_EVENTS || stop_id < 0 ||
+      stop_id >= WDH_MAX_EVENTS || !g.events[start_id] || !g.events[stop_id])
+    return fail(WDH_EINVAL, "wdh_event_elapsed_ms: event not recorded");
+  if (!ms) return fail(WDH_EINVAL, "wdh_event_elapsed_ms: ms is NULL");
+  WDH_HIP_CHECK(hipEventSynchronize(g.events[stop_id]));
+  WDH_HIP_CHECK(hipEventElapsedTime(ms, g.events[start_id], g.events[stop_id]));
+  return WDH_OK;
+}
+
+}  // extern "C"
