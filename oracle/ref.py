@@ -54,7 +54,7 @@ def _ints(values):
 
 
 def _f32(a):
-    a = np.ascontiguousarray(a, dtype=np.float32)
+    a = np.asarray(a, dtype=np.float32, order="C")
     return a
 
 
@@ -122,7 +122,7 @@ _BIN = {"Add": 0, "Sub": 1, "Mul": 2, "Div": 3, "Pow": 4}
 
 
 def binary(op, L, R):
-    L, R = np.ascontiguousarray(L), np.ascontiguousarray(R)
+    L, R = np.asarray(L, order="C"), np.asarray(R, order="C")
     if L.dtype != R.dtype:
         raise RefThrows("Binary: input dataTypes mismatch")
     if L.dtype == np.float32:
@@ -145,7 +145,7 @@ _UN = {"Relu": 0, "Sigmoid": 1, "Sqrt": 2, "Exp": 3, "Tanh": 4, "Abs": 5, "Neg":
 
 
 def unary(op, X):
-    X = np.ascontiguousarray(X)
+    X = np.asarray(X, order="C")
     if X.dtype == np.float32:
         dtype = 0
     elif X.dtype == np.int32:
@@ -201,7 +201,7 @@ def global_average_pool(X):
 
 
 def transpose(X, perm=None):
-    X = np.ascontiguousarray(X)
+    X = np.asarray(X, order="C")
     assert X.dtype.itemsize == 4
     d, n = _dims(X.shape)
     pm, npm = _ints(perm)
@@ -224,8 +224,8 @@ def reduce_mean_last(X):
 
 
 def gather(data, indices, axis=0):
-    data = np.ascontiguousarray(data)
-    indices = np.ascontiguousarray(indices, dtype=np.int32)
+    data = np.asarray(data, order="C")
+    indices = np.asarray(indices, dtype=np.int32, order="C")
     Y = np.empty((), dtype=data.dtype)
     _check(_lib.ref_gather(_ptr(data), data.ndim, _ptr(indices), indices.ndim,
                            ctypes.c_int64(axis), _ptr(Y)), "Gather")

@@ -1,0 +1,459 @@
+"""Parity of the hip backend with the oracle, through the C ABI, on a real MI355X.
+
+Criteria (BASELINE.json north_star): bit-exact for indexing / layout / selection ops and for
+fp32 Add/Sub/Mul/Div/Relu; max|diff| <= 1e-4 * max|ref| for Gemm / MatMul / Conv.  Softmax and
+LayerNormalization, for which north_star names no figure, use 1e-6 and 1e-5 of max|ref| (the
+oracle evaluates exp in double and rounds once; the kernel evaluates it in fp32).
+"""
+import ctypes
+import itertools
+
+import numpy as np
+import pytest
+
+import kat_runner
+from oracle import ref
+from util import assert_bit_exact, assert_close_max, load_kat
+from webdnn_amd import capi
+from webdnn_amd import hostops as H
+
+pytestmark = pytest.mark.gpu
+
+GEMM_TOL = 1e-4
+RNG = np.random.default_rng(2024)
+
+
+def uni(*shape, lo=-1.0, hi=1.0):
+    return RNG.uniform(lo, hi, shape).astype(np.float32)
+
+
+def nrm(*shape, std=1.0):
+    return (RNG.standard_normal(shape) * std).astype(np.float32)
+
+
+# ------------------------------------------------------------------ known answers
+CASES = load_kat()
+
+
+@pytest.mark.parametrize("case", CASES, ids=[kat_runner.case_id(c) for c in CASES])
+def test_known_answers_bit_exact(ctx, case):
+    assert_bit_exact(kat_runner.run_hip(ctx, case), kat_runner.expected(case), case["op"])
+
+
+# ------------------------------------------------------------------ Gemm
+def hip_gemm(ctx, A, B, C=None, alpha=1.0, beta=1.0, ta=0, tb=0, epilogue=None):
+    tc = ctx.move_tensor(C) if C is not None else None
+    return H.gemm(ctx, ctx.move_tensor(A), ctx.move_tensor(B), tc, alpha, beta, ta, tb, epilogue).get_data()
+
+
+def test_gemm_config1(ctx):
+    """BASELINE config 1: A[256,512], B[1024,512] transB=1, C[1024], alpha=beta=1."""
+    A, B, C = uni(256, 512), uni(1024, 512), uni(1024)
+    assert_close_max(hip_gemm(ctx, A, B, C, 1.0, 1.0, 0, 1), ref.gemm(A, B, C, 1.0, 1.0, 0, 1), GEMM_TOL, "C1")
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product((0, 1), (0, 1))))
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (7, 5, 3), (128, 128, 16), (129, 127, 17), (130, 250, 37),
+                                   (64, 300, 1), (1, 513, 40), (257, 1, 33), (100, 92, 256), (32, 1000, 2048)])
+def test_gemm_shapes_and_transposes(ctx, m, n, k, ta, tb):
+    A = uni(k, m) if ta else uni(m, k)
+    B = uni(n, k) if tb else uni(k, n)
+    C = uni(n)
+    got = hip_gemm(ctx, A, B, C, 0.75, -1.25, ta, tb)
+    assert_close_max(got, ref.gemm(A, B, C, 0.75, -1.25, ta, tb), GEMM_TOL, "gemm")
+
+
+@pytest.mark.parametrize("cshape", [(45,), (1, 45), (33, 1), (33, 45), (1,), (), (1, 1)])
+def test_gemm_c_broadcast(ctx, cshape):
+    A, B, C = uni(33, 20), uni(20, 45), uni(*cshape)
+    assert_close_max(hip_gemm(ctx, A, B, C, 1.0, 0.5), ref.gemm(A, B, C, 1.0, 0.5), GEMM_TOL, "C%s" % (cshape,))
+
+
+def test_gemm_invariants_and_edges(ctx):
+    A, B, C = uni(40, 24), uni(24, 36), uni(36)
+    # alpha = 0 -> beta * C exactly; beta = 0 == no C
+    assert_bit_exact(hip_gemm(ctx, A, B, C, 0.0, 2.0), ref.gemm(A, B, C, 0.0, 2.0), "alpha=0")
+    assert_bit_exact(hip_gemm(ctx, A, B, C, 1.5, 0.0), hip_gemm(ctx, A, B, None, 1.5, 1.0), "beta=0")
+    # transposes are the same product
+    assert_bit_exact(hip_gemm(ctx, np.ascontiguousarray(A.T), B, C, 1, 1, 1, 0), hip_gemm(ctx, A, B, C), "transA")
+    # identity B returns A exactly (one nonzero term per sum)
+    assert_bit_exact(hip_gemm(ctx, A, np.eye(24, dtype=np.float32)), A, "identity")
+    # fused Relu epilogue == Relu(Gemm)
+    y = hip_gemm(ctx, A, B, C)
+    assert_bit_exact(hip_gemm(ctx, A, B, C, epilogue="relu"), np.maximum(y, 0) + 0.0, "relu epilogue")
+    # empty inner dimension: the sum over nothing is 0, the C term remains
+    Z0, Z1, C6 = np.zeros((5, 0), np.float32), np.zeros((0, 6), np.float32), uni(6)
+    assert_bit_exact(hip_gemm(ctx, Z0, Z1, C6), ref.gemm(Z0, Z1, C6), "k=0")
+    e = H.gemm(ctx, ctx.move_tensor(np.zeros((0, 8), np.float32)), ctx.move_tensor(uni(8, 4)))
+    assert e.dims == [0, 4] and e.get_data().shape == (0, 4)
+    with pytest.raises(H.OperatorError):
+        H.gemm(ctx, ctx.move_tensor(uni(3, 4)), ctx.move_tensor(uni(5, 6)))
+    with pytest.raises(H.OperatorError):
+        H.gemm(ctx, ctx.move_tensor(uni(3, 4)), ctx.move_tensor(uni(4, 6)), ctx.move_tensor(uni(5)))
+
+
+def test_gemm_4096_sampled_rows_and_linearity(ctx):
+    """The north-star size.  The oracle checks 48 sampled rows; linearity in A covers the rest:
+    (A1 + A2) B == A1 B + A2 B within fp32 accumulation error."""
+    n = 4096
+    A, B, C = uni(n, n), uni(n, n), uni(n)
+    tb, tc = ctx.move_tensor(B), ctx.move_tensor(C)
+    got = H.gemm(ctx, ctx.move_tensor(A), tb, tc).get_data()
+    rows = RNG.choice(n, 48, replace=False)
+    assert_close_max(got[rows], ref.gemm(A[rows], B, C), GEMM_TOL, "NS-4096 rows")
+    A2 = uni(n, n)
+    got2 = H.gemm(ctx, ctx.move_tensor(A2), tb, None).get_data()
+    both = H.gemm(ctx, ctx.move_tensor(A + A2), tb, tc).get_data()
+    assert_close_max(both, got + got2, GEMM_TOL, "linearity")
+
+
+# ------------------------------------------------------------------ MatMul
+@pytest.mark.parametrize("sa,sb", [((3, 4), (4, 5)), ((2, 3, 4), (4, 5)), ((1, 3, 128), (4, 128, 1)),
+                                   ((4, 3, 6), (4, 6, 2)), ((6,), (6, 3)), ((2, 3, 6), (6,)), ((6,), (6,)),
+                                   ((8, 850, 32), (8, 32, 850)), ((8, 850, 850), (8, 850, 32)),
+                                   ((850, 1, 256), (256, 2048)), ((850, 1, 2048), (2048, 256)),
+                                   ((8, 100, 32), (8, 32, 850)), ((1, 77, 33), (5, 33, 9))])
+def test_matmul_shapes(ctx, sa, sb):
+    A, B = nrm(*sa), nrm(*sb)
+    got = H.matmul(ctx, ctx.move_tensor(A), ctx.move_tensor(B))
+    want = ref.matmul(A, B)
+    assert tuple(got.dims) == want.shape
+    assert_close_max(got.get_data(), want, GEMM_TOL, "matmul %s x %s" % (sa, sb))
+
+
+def test_matmul_rejects_what_the_reference_rejects(ctx):
+    with pytest.raises(H.OperatorError):
+        H.matmul(ctx, ctx.move_tensor(nrm(2, 2, 3, 4)), ctx.move_tensor(nrm(4, 5)))
+    with pytest.raises(H.OperatorError):
+        H.matmul(ctx, ctx.move_tensor(nrm(3, 4)), ctx.move_tensor(nrm(5, 6)))
+
+
+def test_ffn_chain_config2(ctx):
+    """BASELINE config 2: X[8,512,768] -> MatMul W1 -> Add b1 -> Relu -> MatMul W2 -> Add X.
+    Full size on the GPU; the oracle follows 64 sampled token rows (the chain is row-wise)."""
+    X, W1, b1, W2 = nrm(8, 512, 768), nrm(768, 3072, std=0.02), np.zeros(3072, np.float32), nrm(3072, 768, std=0.02)
+    tX, tW1, tb1, tW2 = (ctx.move_tensor(t) for t in (X, W1, b1, W2))
+    h = H.matmul(ctx, tX, tW1)
+    hb = H.binary(ctx, "Add", h, tb1)
+    hr = H.unary(ctx, "Relu", hb)
+    y = H.matmul(ctx, hr, tW2)
+    out = H.binary(ctx, "Add", y, tX).get_data()
+    rows = np.sort(RNG.choice(8 * 512, 64, replace=False))
+    xs = X.reshape(-1, 768)[rows]
+    o_h = ref.matmul(xs, W1)
+    o_hr = ref.unary("Relu", ref.binary("Add", o_h, b1))
+    o_out = ref.binary("Add", ref.matmul(o_hr, W2), xs)
+    assert_close_max(h.get_data().reshape(-1, 3072)[rows], o_h, GEMM_TOL, "MatMul 1")
+    assert_close_max(out.reshape(-1, 768)[rows], o_out, GEMM_TOL, "FFN output")
+    # the fused forms compute the same chain
+    hf = H.matmul(ctx, tX, tW1, bias=tb1, epilogue="relu")
+    assert_bit_exact(hf.get_data(), hr.get_data(), "fused MatMul+Add+Relu")
+    of = H.matmul(ctx, hf, tW2, residual=tX)
+    assert_bit_exact(of.get_data(), out, "fused MatMul+Add(residual)")
+
+
+# ------------------------------------------------------------------ Conv
+def hip_conv(ctx, X, W, B=None, dil=None, group=1, pads=None, strides=None, epilogue=None, R=None):
+    return H.conv(ctx, ctx.move_tensor(X), ctx.move_tensor(W), ctx.move_tensor(B) if B is not None else None,
+                  dil, group, None, pads, strides, epilogue, ctx.move_tensor(R) if R is not None else None).get_data()
+
+
+def he(cout, cin, k):
+    return nrm(cout, cin, k, k, std=float(np.sqrt(2.0 / (cin * k * k))))
+
+
+def test_conv_config3_full(ctx):
+    """BASELINE config 3: X[32,64,56,56] U[0,1], W[64,64,3,3] He-normal, bias zeros, pad 1, then Relu."""
+    X, W, B = uni(32, 64, 56, 56, lo=0), he(64, 64, 3), np.zeros(64, np.float32)
+    want = ref.conv(X, W, B, pads=[1, 1, 1, 1])
+    got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])
+    assert_close_max(got, want, GEMM_TOL, "C3 conv")
+    fused = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1], epilogue="relu")
+    assert_bit_exact(fused, np.maximum(got, 0) + 0.0, "C3 fused Relu")
+    assert_close_max(fused, ref.unary("Relu", want), GEMM_TOL, "C3 conv+relu")
+
+
+CONV_SHAPES = [
+    # n, cin, h, w, cout, k, pads, strides, dil, group  — ResNet-50 layer forms and the reference's
+    # conv1..conv11 attribute mix (test/model_test/make_models.py:623-643)
+    (2, 3, 224, 224, 64, 7, [3, 3, 3, 3], [2, 2], [1, 1], 1),     # stem
+    (2, 64, 56, 56, 256, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),
+    (2, 256, 56, 56, 128, 1, [0, 0, 0, 0], [2, 2], [1, 1], 1),    # strided 1x1 (v1 bottleneck)
+    (2, 256, 56, 56, 512, 1, [0, 0, 0, 0], [2, 2], [1, 1], 1),    # downsample branch
+    (2, 128, 28, 28, 128, 3, [1, 1, 1, 1], [1, 1], [1, 1], 1),
+    (2, 256, 14, 14, 256, 3, [1, 1, 1, 1], [1, 1], [1, 1], 1),
+    (3, 512, 7, 7, 512, 3, [1, 1, 1, 1], [1, 1], [1, 1], 1),
+    (3, 512, 7, 7, 2048, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),
+    (2, 128, 57, 57, 128, 3, [1, 1, 1, 1], [2, 2], [1, 1], 1),    # odd size, stride 2
+    (2, 8, 14, 15, 12, 3, [1, 0, 2, 1], [2, 1], [1, 1], 2),       # groups, asymmetric pads
+    (1, 6, 20, 20, 6, 3, [2, 2, 2, 2], [1, 1], [2, 2], 1),        # dilation 2
+    (2, 16, 9, 9, 16, 3, [1, 1, 1, 1], [1, 1], [1, 1], 16),       # depthwise
+    (1, 5, 6, 7, 3, 2, [0, 0, 0, 0], [1, 1], [1, 1], 1),          # even kernel, no pad
+    (1, 2048, 25, 34, 256, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),   # DETR input projection
+]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES)
+def test_conv_shapes(ctx, shape):
+    n, cin, h, w, cout, k, pads, strides, dil, group = shape
+    X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin // group, k), nrm(cout)
+    want = ref.conv(X, W, B, dil, group, None, pads, strides)
+    got = hip_conv(ctx, X, W, B, dil, group, pads, strides)
+    assert got.shape == want.shape
+    assert_close_max(got, want, GEMM_TOL, "conv %s" % (shape,))
+
+
+def test_conv_residual_epilogue_and_no_bias(ctx):
+    X, W = uni(2, 32, 14, 14, lo=0), he(48, 32, 3)
+    R = nrm(2, 48, 14, 14)
+    plain = hip_conv(ctx, X, W, pads=[1, 1, 1, 1])
+    assert_close_max(plain, ref.conv(X, W, pads=[1, 1, 1, 1]), GEMM_TOL, "no bias")
+    fused = hip_conv(ctx, X, W, pads=[1, 1, 1, 1], epilogue="relu", R=R)
+    assert_bit_exact(fused, np.maximum(plain + R, 0) + 0.0, "conv + residual + relu")
+    with pytest.raises(H.OperatorError):
+        H.conv(ctx, ctx.move_tensor(uni(2, 3, 8)), ctx.move_tensor(uni(4, 3, 3, 3)))
+
+
+def test_conv_1x1_equals_gemm(ctx):
+    X, W = uni(2, 40, 6, 5), uni(24, 40, 1, 1)
+    got = hip_conv(ctx, X, W)
+    for b in range(2):
+        g = hip_gemm(ctx, W.reshape(24, 40), X[b].reshape(40, 30))
+        assert_close_max(got[b].reshape(24, 30), g, 1e-6, "1x1 == gemm")
+
+
+# ------------------------------------------------------------------ elementwise
+@pytest.mark.parametrize("op", ["Add", "Sub", "Mul", "Div"])
+@pytest.mark.parametrize("sl,sr", [((2, 3, 10, 12), ()), ((2, 3, 10, 12), (1, 3, 1, 12)), ((), ()),
+                                   ((2, 3, 10, 12), (2, 3, 10, 12)), ((4, 1), (3,)), ((8, 512, 3072), (3072,)),
+                                   ((2, 1, 3, 1, 2, 1), (1, 2, 1, 2, 1, 3)), ((5, 7), (5, 1)), ((1, 3, 1, 12), (2, 3, 10, 12)),
+                                   ((3, 1031), (3, 1031)), ((2, 64, 7, 7), (1, 64, 1, 1)), ((850, 1, 256), (850, 1, 1))])
+def test_binary_bit_exact(ctx, op, sl, sr):
+    L, R = uni(*sl, lo=-3, hi=3), uni(*sr, lo=-3, hi=3)
+    got = H.binary(ctx, op, ctx.move_tensor(L), ctx.move_tensor(R))
+    want = ref.binary(op, L, R)
+    assert tuple(got.dims) == want.shape
+    assert_bit_exact(got.get_data(), want, "%s %s %s" % (op, sl, sr))
+
+
+def test_binary_special_values_int32_pow_and_errors(ctx):
+    L = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, 3.4e38, 1.0, 1e-39, -1e-39, 2e-38], np.float32)
+    R = np.array([-0.0, 0.0, -np.inf, 1.0, 1.0, 0.5, 3.4e38, 0.0, 1e-39, 3.0, 0.25], np.float32)
+    for op in ("Add", "Sub", "Mul", "Div"):
+        got = H.binary(ctx, op, ctx.move_tensor(L), ctx.move_tensor(R)).get_data()
+        assert_bit_exact(got, ref.binary(op, L, R), op + " specials (incl. denormals)")
+    a = np.array([2147483647, -2147483648, 7, -7, 100000, 5, 0], np.int32)
+    b = np.array([1, -1, 2, 2, 100000, 0, 0], np.int32)
+    for op in ("Add", "Sub", "Mul", "Div"):
+        got = H.binary(ctx, op, ctx.move_tensor(a), ctx.move_tensor(b)).get_data()
+        assert_bit_exact(got, ref.binary(op, a, b), op + " int32")
+    base, ex = uni(4, 50, lo=0.1, hi=4), uni(50, lo=-3, hi=3)
+    got = H.binary(ctx, "Pow", ctx.move_tensor(base), ctx.move_tensor(ex)).get_data()
+    assert_close_max(got, ref.binary("Pow", base, ex), 1e-6, "Pow")
+    with pytest.raises(H.OperatorError):
+        H.binary(ctx, "Add", ctx.move_tensor(uni(2, 3)), ctx.move_tensor(uni(4)))
+    with pytest.raises(H.OperatorError):
+        H.binary(ctx, "Add", ctx.move_tensor(uni(2)), ctx.move_tensor(np.zeros(2, np.int32)))
+
+
+def test_unary(ctx):
+    x = np.array([-2, -0.5, 0, 1, 3, np.nan, -0.0, -np.inf, np.inf, 1e-40, -1e-40], np.float32)
+    assert_bit_exact(H.unary(ctx, "Relu", ctx.move_tensor(x)).get_data(), ref.unary("Relu", x), "Relu specials")
+    big = nrm(8, 512, 3073)
+    assert_bit_exact(H.unary(ctx, "Relu", ctx.move_tensor(big)).get_data(), ref.unary("Relu", big), "Relu big")
+    xi = np.array([-3, 0, 4, -2147483648], np.int32)
+    assert_bit_exact(H.unary(ctx, "Relu", ctx.move_tensor(xi)).get_data(), ref.unary("Relu", xi), "Relu int32")
+    v = uni(1, 100, 4, lo=-20, hi=20)
+    for op, tol in (("Sigmoid", 1e-6), ("Exp", 1e-6), ("Tanh", 1e-6), ("Reciprocal", 1e-7)):
+        assert_close_max(H.unary(ctx, op, ctx.move_tensor(v)).get_data(), ref.unary(op, v), tol, op)
+    p = uni(1000, lo=0, hi=50)
+    assert_bit_exact(H.unary(ctx, "Sqrt", ctx.move_tensor(p)).get_data(), ref.unary("Sqrt", p), "Sqrt")
+    for op in ("Abs", "Neg"):
+        assert_bit_exact(H.unary(ctx, op, ctx.move_tensor(v)).get_data(), ref.unary(op, v), op)
+    with pytest.raises(H.OperatorError):
+        H.unary(ctx, "Sigmoid", ctx.move_tensor(xi))
+
+
+# ------------------------------------------------------------------ row reductions
+@pytest.mark.parametrize("shape", [(8, 850, 850), (8, 100, 850), (8, 100, 100), (3, 4, 5, 6), (7, 1), (5, 64), (3, 129),
+                                   (4, 1025), (2, 2049), (3, 5000), (1, 1)])
+def test_softmax(ctx, shape):
+    x = nrm(*shape, std=3.0)
+    got = H.softmax(ctx, ctx.move_tensor(x)).get_data()
+    assert_close_max(got, ref.softmax(x), 1e-6, "softmax %s" % (shape,))
+    assert np.abs(got.astype(np.float64).sum(-1) - 1).max() < 1e-5
+
+
+def test_softmax_edges(ctx):
+    x = np.array([[0, 1000, 0], [-np.inf, 0, -np.inf], [5, 5, 5]], np.float32)
+    assert_bit_exact(H.softmax(ctx, ctx.move_tensor(x)).get_data(), ref.softmax(x), "one-hot / uniform")
+    with pytest.raises(H.OperatorError):
+        H.softmax(ctx, ctx.move_tensor(nrm(2, 3, 4)), axis=1)
+
+
+@pytest.mark.parametrize("shape", [(850, 1, 256), (100, 1, 256), (6, 2048), (3, 5000), (4, 7), (2, 3, 1)])
+def test_layernorm(ctx, shape):
+    x, g, b = nrm(*shape, std=2.0), nrm(shape[-1]), nrm(shape[-1])
+    got = H.layer_normalization(ctx, ctx.move_tensor(x), ctx.move_tensor(g), ctx.move_tensor(b)).get_data()
+    assert_close_max(got, ref.layernorm_decomposed(x, g, b, 1e-5), 1e-5, "layernorm %s" % (shape,))
+    plain = H.layer_normalization(ctx, ctx.move_tensor(x)).get_data()
+    assert_close_max(plain, ref.layernorm_decomposed(x, None, None, 1e-5), 1e-5, "layernorm no affine")
+
+
+@pytest.mark.parametrize("shape", [(32, 2048, 7, 7), (4, 16, 56, 56), (1, 3, 1, 1), (2, 5, 3, 300)])
+def test_global_average_pool_and_reduce_mean(ctx, shape):
+    x = nrm(*shape)
+    got = H.global_average_pool(ctx, ctx.move_tensor(x))
+    want = ref.global_average_pool(x)
+    assert tuple(got.dims) == want.shape
+    # double sums in another order may differ in the last double bit -> at most 1 fp32 ulp
+    from util import ulp_diff
+    assert ulp_diff(got.get_data(), want).max() <= 1
+    flat = x.reshape(-1, shape[2] * shape[3])
+    rm = H.reduce_mean_last(ctx, ctx.move_tensor(flat)).get_data()
+    assert ulp_diff(rm, ref.reduce_mean_last(flat)).max() <= 1
+
+
+# ------------------------------------------------------------------ MaxPool
+def test_maxpool_resnet_stem_full(ctx):
+    x = nrm(32, 64, 112, 112)
+    got = H.maxpool(ctx, ctx.move_tensor(x), [3, 3], pads=[1, 1, 1, 1], strides=[2, 2]).get_data()
+    assert_bit_exact(got, ref.maxpool(x, [3, 3], pads=[1, 1, 1, 1], strides=[2, 2]), "stem maxpool")
+
+
+@pytest.mark.parametrize("attrs", [
+    dict(kernel_shape=[3, 3], strides=[2, 2]),
+    dict(kernel_shape=[3, 3], strides=[2, 2], ceil_mode=1),
+    dict(kernel_shape=[3, 3], strides=[2, 3], auto_pad="SAME_UPPER"),
+    dict(kernel_shape=[3, 3], strides=[2, 3], auto_pad="SAME_LOWER"),
+    dict(kernel_shape=[3, 3], strides=[2, 3], auto_pad="VALID"),
+    dict(kernel_shape=[2, 2], strides=[2, 2], dilations=[2, 2], pads=[1, 1, 1, 1]),
+    dict(kernel_shape=[2, 2], strides=[3, 3], pads=[1, 1, 1, 1], ceil_mode=1),
+    dict(kernel_shape=[1, 1]),
+])
+def test_maxpool_attributes(ctx, attrs):
+    x = nrm(2, 3, 10, 13)
+    x[0, 0, 0, 0] = np.nan
+    got = H.maxpool(ctx, ctx.move_tensor(x), **attrs)
+    want = ref.maxpool(x, **attrs)
+    assert tuple(got.dims) == want.shape
+    assert_bit_exact(got.get_data(), want, "maxpool %s" % (attrs,))
+
+
+def test_maxpool_errors(ctx):
+    t = ctx.move_tensor(nrm(1, 1, 6, 6))
+    with pytest.raises(H.OperatorError):
+        H.maxpool(ctx, t, [3, 3], n_outputs=2)
+    with pytest.raises(H.OperatorError):
+        H.maxpool(ctx, t, [3, 3], storage_order=1)
+    with pytest.raises(H.OperatorError):
+        H.maxpool(ctx, t, [3, 3], auto_pad="SAME")
+    with pytest.raises(H.OperatorError):
+        H.maxpool(ctx, ctx.move_tensor(nrm(2, 6, 6)), [3, 3])
+
+
+# ------------------------------------------------------------------ layout
+@pytest.mark.parametrize("ndim", [1, 2, 3, 4])
+def test_transpose_all_permutations(ctx, ndim):
+    shape = (19, 70, 3, 33)[:ndim]
+    x = nrm(*shape)
+    t = ctx.move_tensor(x)
+    for perm in itertools.permutations(range(ndim)):
+        got = H.transpose(ctx, t, list(perm)).get_data()
+        assert_bit_exact(got, ref.transpose(x, list(perm)), "perm %s" % (perm,))
+    assert_bit_exact(H.transpose(ctx, t).get_data(), ref.transpose(x), "default perm")
+
+
+@pytest.mark.parametrize("shape,perm", [((1, 256, 850), (2, 0, 1)), ((850, 8, 32), (1, 0, 2)), ((8, 850, 32), (0, 2, 1)),
+                                         ((8, 850, 32), (1, 0, 2)), ((2, 3, 2, 2, 3), (4, 0, 3, 1, 2)),
+                                         ((2, 3, 2, 2, 3, 2), (5, 3, 0, 4, 1, 2)), ((64, 64, 3, 3), (2, 3, 1, 0)),
+                                         ((1000, 2048), (1, 0)), ((3, 1, 5), (2, 1, 0))])
+def test_transpose_model_shapes(ctx, shape, perm):
+    x = nrm(*shape)
+    got = H.transpose(ctx, ctx.move_tensor(x), list(perm)).get_data()
+    assert_bit_exact(got, ref.transpose(x, list(perm)), "%s %s" % (shape, perm))
+    xi = RNG.integers(-2 ** 31, 2 ** 31 - 1, shape).astype(np.int32)
+    assert_bit_exact(H.transpose(ctx, ctx.move_tensor(xi), list(perm)).get_data(), ref.transpose(xi, list(perm)), "int32")
+
+
+def test_flatten_reshape_alias_and_gather(ctx):
+    x = nrm(2, 3, 4, 5)
+    t = ctx.move_tensor(x)
+    f = H.flatten(ctx, t)
+    assert f.dims == [2, 60] and f.handle == t.handle            # shares the buffer (cpu flatten.ts:11-20)
+    assert_bit_exact(f.get_data(), ref.flatten(x), "flatten")
+    r = H.reshape(ctx, t, [0, -1, 5])
+    assert_bit_exact(r.get_data(), ref.reshape(x, [0, -1, 5]), "reshape")
+    t.dispose()                                                   # aliases keep the buffer alive
+    assert_bit_exact(r.get_data(), ref.reshape(x, [0, -1, 5]), "alias outlives source")
+    f.dispose()
+    r.dispose()
+    with pytest.raises(H.OperatorError):
+        H.flatten(ctx, ctx.move_tensor(x), axis=2)
+    data = np.array([5, 6, 7], np.int32)
+    got = H.gather(ctx, ctx.move_tensor(data), ctx.move_tensor(np.array(2, np.int32)))
+    assert got.dims == [] and got.get_data().tolist() == ref.gather(data, np.array(2, np.int32)).tolist()
+    table = nrm(10, 4, 6)
+    idx = np.array([[3, -1], [0, 9]], np.int32)
+    got = H.gather(ctx, ctx.move_tensor(table), ctx.move_tensor(idx), axis=0).get_data()
+    assert_bit_exact(got, table[idx], "gather axis 0")
+    got = H.gather(ctx, ctx.move_tensor(table), ctx.move_tensor(np.array([2, 0, -2], np.int32)), axis=1).get_data()
+    assert_bit_exact(got, np.take(table, [2, 0, -2], axis=1), "gather axis 1")
+
+
+# ------------------------------------------------------------------ runtime
+def test_buffers_offsets_large_copies_and_pool(ctx):
+    n = 20 * 1024 * 1024 + 13                 # 80 MiB: several staging chunks each way
+    x = RNG.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+    t = ctx.move_tensor(x)
+    assert_bit_exact(t.get_data(), x, "large round trip")
+    part = np.empty(1000, np.int32)
+    capi.call("wdh_read", t.handle, 4 * 12345, part.ctypes.data_as(ctypes.c_void_p), part.nbytes)
+    assert_bit_exact(part, x[12345:13345], "offset read")
+    patch = np.arange(50, dtype=np.int32)
+    capi.call("wdh_write", t.handle, 4 * 777, patch.ctypes.data_as(ctypes.c_void_p), patch.nbytes)
+    x[777:827] = patch
+    u = ctx.empty_tensor([n], "int32")
+    capi.call("wdh_copy", u.handle, 0, t.handle, 0, 4 * n)
+    assert_bit_exact(u.get_data(), x, "device copy after patch")
+    before = ctx.mem_stats()
+    t.dispose()
+    u.dispose()
+    after = ctx.mem_stats()
+    assert after["in_use"] < before["in_use"] and after["cached"] > before["cached"]
+    v = ctx.empty_tensor([n], "int32")        # served from the pool: no new reservation
+    assert ctx.mem_stats()["peak"] == after["peak"]
+    v.dispose()
+    z = ctx.empty_tensor([0])
+    assert z.get_data().shape == (0,)
+    z.dispose()
+
+
+def test_errors_are_reported_not_fatal(ctx):
+    with pytest.raises(capi.HipError) as err:
+        capi.call("wdh_free", 123456789)
+    assert "unknown buffer handle" in str(err.value)
+    small = ctx.empty_tensor([4])
+    with pytest.raises(capi.HipError) as err:
+        capi.call("wdh_unary", 0, 0, small.handle, small.handle, 1000)
+    assert "needs" in str(err.value)
+    with pytest.raises(capi.HipError):
+        capi.call("wdh_unary", 99, 0, small.handle, small.handle, 4)
+    with pytest.raises(capi.HipError):
+        capi.call("wdh_gemm", small.handle, small.handle, 0, small.handle, 1, 64, 64, 64, 0, 64, 1, 0, 64, 1, 0, 0,
+                  1.0, 1.0, 0, 0)
+    with pytest.raises(capi.HipError):
+        capi.call("wdh_conv2d", small.handle, small.handle, 0, small.handle, 1, 3, 8, 8, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1,
+                  2, 0, 0)     # channels not divisible by group
+    # the context still works afterwards
+    x = uni(4)
+    small.set_data(x)
+    assert_bit_exact(small.get_data(), x, "still alive")
+    small.dispose()
+    with pytest.raises(H.OperatorError):
+        _ = small.handle
+    ctx.event_record(10)
+    ctx.event_record(11)
+    assert ctx.event_elapsed_ms(10, 11) >= 0.0
+    info = ctx.device_info()
+    assert info["name"].startswith("gfx950") and info["compute_units"] > 0

@@ -109,7 +109,7 @@ class HipTensor:
         return HipTensor(self.context, dims, self.data_type, self._shared)
 
     def set_data(self, array):
-        array = np.ascontiguousarray(array, dtype=_DTYPES[self.data_type])
+        array = np.asarray(array, dtype=_DTYPES[self.data_type], order="C")
         if array.size != self.length:
             raise OperatorError("setData: length mismatch")
         call("wdh_write", self.handle, 0, array.ctypes.data_as(ctypes.c_void_p), array.nbytes)
