@@ -63,6 +63,18 @@ const char *wdh_last_error(void);
 int wdh_device_info(char *name, int name_cap, int *compute_units,
                     int *clock_mhz, uint64_t *hbm_bytes);
 
+/* Backend options (the counterpart of InitOption.backendOptions,
+ * src/descriptor_runner/index.ts:26-30).  Known names:
+ *   "contraction_tile"  -1 = choose per problem (default); 0 = 128x128,
+ *                       1 = 64x256, 2 = 64x128, 3 = 64x64 workgroup tiles for
+ *                       wdh_gemm / wdh_conv2d (a tuning and test hook: every
+ *                       tile shape computes the same result).
+ *   "split_k"           -1 = choose per problem (default); n >= 1 = cut the
+ *                       K loop of wdh_gemm / wdh_conv2d into n chunks whose
+ *                       partial sums are added in chunk order by a second
+ *                       kernel (1 = never split). */
+int wdh_set_option(const char *name, int value);
+
 /* ---- buffers --------------------------------------------------------- */
 
 /* Replaces the `alloc` message, wasmContextImpl.ts:128-134 and

@@ -457,3 +457,56 @@ def test_errors_are_reported_not_fatal(ctx):
     assert ctx.event_elapsed_ms(10, 11) >= 0.0
     info = ctx.device_info()
     assert info["name"].startswith("gfx950") and info["compute_units"] > 0
+
+
+# ------------------------------------------------------------------ tile shapes
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+def test_every_tile_shape_computes_the_same(ctx, tile):
+    """wdh_gemm / wdh_conv2d pick a workgroup tile per problem; every shape must agree."""
+    A, B, C = uni(150, 70), uni(70, 300), uni(300)
+    X, W, Bv = uni(2, 24, 17, 19, lo=0), he(40, 24, 3), nrm(40)
+    At, Bt = uni(70, 150), uni(300, 70)
+    try:
+        ctx.set_option("contraction_tile", tile)
+        g = hip_gemm(ctx, A, B, C)
+        gt = hip_gemm(ctx, At, Bt, C, 1.0, 1.0, 1, 1)
+        c = hip_conv(ctx, X, W, Bv, pads=[1, 1, 1, 1], strides=[2, 1])
+    finally:
+        ctx.set_option("contraction_tile", -1)
+    assert_close_max(g, ref.gemm(A, B, C), GEMM_TOL, "gemm tile %d" % tile)
+    assert_close_max(gt, ref.gemm(At, Bt, C, 1.0, 1.0, 1, 1), GEMM_TOL, "gemm TT tile %d" % tile)
+    assert_close_max(c, ref.conv(X, W, Bv, pads=[1, 1, 1, 1], strides=[2, 1]), GEMM_TOL, "conv tile %d" % tile)
+    with pytest.raises(capi.HipError):
+        ctx.set_option("contraction_tile", 9)
+    with pytest.raises(capi.HipError):
+        ctx.set_option("no_such_option", 1)
+
+
+@pytest.mark.parametrize("split", [1, 2, 5, 64])
+def test_split_k_is_the_same_sum(ctx, split):
+    """Split-K cuts the K loop into chunks reduced by a second kernel in chunk order."""
+    A, B, C = uni(70, 333), uni(333, 90), uni(90)
+    X, W, Bv, R = uni(2, 40, 7, 7, lo=0), he(24, 40, 3), nrm(24), nrm(2, 24, 7, 7)
+    A3, B3 = nrm(3, 50, 200), nrm(3, 200, 30)
+    try:
+        ctx.set_option("split_k", split)
+        g = hip_gemm(ctx, A, B, C, 0.5, 2.0, epilogue="relu")
+        c = hip_conv(ctx, X, W, Bv, pads=[1, 1, 1, 1], epilogue="relu", R=R)
+        m3 = H.matmul(ctx, ctx.move_tensor(A3), ctx.move_tensor(B3)).get_data()
+        cg = hip_conv(ctx, uni(1, 8, 9, 9), he(6, 4, 3), nrm(6), group=2)
+    finally:
+        ctx.set_option("split_k", -1)
+    assert_close_max(g, ref.unary("Relu", ref.gemm(A, B, C, 0.5, 2.0)), GEMM_TOL, "gemm split %d" % split)
+    want = ref.unary("Relu", ref.binary("Add", ref.conv(X, W, Bv, pads=[1, 1, 1, 1]), R))
+    assert_close_max(c, want, GEMM_TOL, "conv split %d" % split)
+    assert_close_max(m3, ref.matmul(A3, B3), GEMM_TOL, "batched matmul split %d" % split)
+    assert cg.shape == (1, 6, 7, 7)
+
+
+def test_split_k_auto_on_deep_small_layers(ctx):
+    """ResNet stage-4 forms (few pixels, long K) take the split path by themselves."""
+    X, W, Bv = uni(4, 512, 7, 7, lo=0), he(512, 512, 3), nrm(512)
+    assert_close_max(hip_conv(ctx, X, W, Bv, pads=[1, 1, 1, 1]), ref.conv(X, W, Bv, pads=[1, 1, 1, 1]), GEMM_TOL,
+                     "3x3 512 @7x7")
+    A, B = uni(64, 4096), uni(4096, 48)
+    assert_close_max(hip_gemm(ctx, A, B), ref.gemm(A, B), GEMM_TOL, "skinny gemm")

@@ -9,7 +9,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libwebdnn_hip.so")
+# WEBDNN_HIP_LIB names another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("WEBDNN_HIP_LIB") or os.path.join(_HERE, "lib", "libwebdnn_hip.so")
 
 # every symbol include/webdnn_hip.h declares, with its signature
 c_buf = ctypes.c_int64
@@ -24,6 +25,7 @@ SIGNATURES = {
     "wdh_last_error": (_c.c_char_p, []),
     "wdh_device_info": (_c.c_int, [_c.c_char_p, _c.c_int, _c.POINTER(_c.c_int),
                                    _c.POINTER(_c.c_int), _u64p]),
+    "wdh_set_option": (_c.c_int, [_c.c_char_p, _c.c_int]),
     "wdh_alloc": (c_buf, [_c.c_size_t]),
     "wdh_free": (_c.c_int, [c_buf]),
     "wdh_write": (_c.c_int, [c_buf, _c.c_size_t, _c.c_void_p, _c.c_size_t]),

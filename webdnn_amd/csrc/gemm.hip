@@ -9,12 +9,15 @@
 // cores, and the rounding points after the sum are kept: alpha*sum is rounded
 // to fp32 before the C/bias term is added).
 //
-// Tiling: one 256-thread workgroup (4 wavefronts of 64) owns a 128x128 tile of
-// the result; each wavefront owns 64x64 = 2x2 v_mfma_f32_32x32x2_f32 tiles
-// (64 accumulator registers per lane).  K advances 16 at a time through two
-// LDS buffers; the next K slab is fetched from global memory into registers
-// while the current one feeds the matrix cores, so there is one barrier per
-// slab.
+// Tiling: one 256-thread workgroup (4 wavefronts of 64) owns a BM x BN tile of
+// the result, split over a WM x WN grid of wavefronts; each wavefront owns
+// MT x NT v_mfma_f32_32x32x2_f32 tiles (16 accumulator registers per lane
+// each).  K advances 16 at a time through two LDS buffers; the next K slab is
+// fetched from global memory into registers while the current one feeds the
+// matrix cores, so there is one barrier per slab.  Tile shapes: 128x128 for
+// large problems, 64x256 / 64x128 when there are at most 64 result rows worth
+// filling (ResNet stage-1 convs have 64 output channels), 64x64 when a larger
+// tile would leave most of the 256 CUs idle.
 //
 // Operand layouts in LDS depend on which index is contiguous in global memory:
 //   "KC" (k contiguous, e.g. A of a non-transposed Gemm, conv weights):
@@ -23,8 +26,16 @@
 //        k = 8*(s/4) + 4*half + s%4 for MFMA step s and lane half (lane/32);
 //        both operands use the same order, so the sum is over the same set.
 //   "MC" (row/column index contiguous, e.g. B of a non-transposed Gemm, the
-//        im2col view of a conv input): tile[k][col], row stride 136 floats;
-//        a lane reads one float per step, lanes 0..31 hit consecutive banks.
+//        im2col view of a conv input): tile[k][col], row stride extent+8
+//        floats; a lane reads one float per step, lanes 0..31 hit consecutive
+//        banks and the two lane halves land 32 banks apart.
+//
+// Conv is Y[co][pixel] = W[co][k] * im2col[k][pixel] with k = (ci, ky, kx) and
+// pixel = (image, oy, ox): M = output channels, N = batch*oh*ow.  The im2col
+// matrix is never materialised: each thread owns one output pixel of the tile
+// and gathers its taps straight from X (NCHW), consecutive lanes reading
+// consecutive addresses; the epilogue scatters rows back to NCHW and fuses
+// bias, residual and Relu.
 #include <string.h>
 
 #include <map>
@@ -37,28 +48,30 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128;
-constexpr int BN = 128;
 constexpr int BK = 16;
 constexpr int NTHREADS = 256;
-constexpr int LDK = BK + 4;    // KC tile row stride (floats)
-constexpr int LDM = 128 + 8;   // MC tile row stride (floats)
-constexpr int TILE_FLOATS = (BM * LDK > BK * LDM) ? BM * LDK : BK * LDM;
+constexpr int LDK = BK + 4;  // KC tile row stride (floats)
+constexpr int MC_PAD = 8;    // MC tile row stride = extent + 8 (floats)
 
-enum BMode { B_KC = 0, B_MC = 1, B_IM2COL = 2 };
+enum BMode { B_KC = 0, B_MC = 1, B_IM2COL = 2, B_IM2COL_BIG = 3 };  // BIG: more than 64 taps
 
 struct ConvGeom {
   int c_in_g;        // input channels per group
   int h, w;          // input spatial size
   int oh, ow;        // output spatial size
-  int kh, kw;
   int pt, pl;        // top / left padding
   int sh, sw;        // strides
   int c_total;       // input channels (all groups)
   int cout_total;    // output channels (all groups)
   int cout_g;        // output channels per group
-  int64_t npix;      // batch * oh * ow
-  const int2 *ktab;  // per k: {offset ci*h*w + ky*dh*w + kx*dw, (ky*dh)<<16 | kx*dw}
+  int ntaps;         // kh*kw
+  long long npix;    // batch * oh * ow
+  // per k = (ci, ky, kx): x = ci*h*w + ky*dh*w + kx*dw (offset from the
+  // receptive field's corner), y = tap index ky*kw+kx (at most 64 taps) or
+  // (ky*dh)<<16 | kx*dw (otherwise); padded with zeros to a multiple of 16
+  const int2 *ktab;
+  // per tap: (ky*dh)<<16 | kx*dw, used to build the per-pixel mask
+  const int *taptab;
 };
 
 struct Params {
@@ -74,6 +87,9 @@ struct Params {
   float alpha, beta;
   int epilogue;
   int tiles_m, tiles_n;
+  int ksplit;       // > 1: K is cut into ksplit chunks (blockIdx.z), partial sums go to `partial`
+  int kchunk;       // chunk length, a multiple of 16
+  float *partial;   // [ksplit][gridDim.y][m][n] raw sums
   ConvGeom cv;
 };
 
@@ -105,21 +121,22 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 }
 
 // ---- global -> register fetch of one K slab ------------------------------
-// KC operand: thread t fetches rows (t>>2) and (t>>2)+64, k offsets 4*(t&3)..+3.
-template <bool VEC>
+// KC operand, EXT rows: thread t fetches rows (t>>2) + 64*i, k offsets 4*(t&3)..+3.
+template <int EXT, bool VEC>
 __device__ __forceinline__ void fetch_kc(const float *__restrict__ base,
                                          long long ld_row, int row0, int nrows,
                                          int k0, int kdim, int tid,
-                                         f32x4 (&reg)[2]) {
-  const int kq = (tid & 3) * 4;
-  const int k = k0 + kq;
+                                         f32x4 (&reg)[EXT / 64]) {
+  const int k = k0 + (tid & 3) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < EXT / 64; i++) {
     int r = row0 + (tid >> 2) + i * 64;
     r = r < nrows ? r : nrows - 1;  // rows past the edge are never stored
     const float *p = base + (long long)r * ld_row + k;
-    if (VEC && k + 3 < kdim) {
-      reg[i] = *reinterpret_cast<const f32x4 *>(p);
+    if (k + 3 < kdim) {
+      // interior: plain loads, nothing between them and the LDS store
+      if (VEC) reg[i] = *reinterpret_cast<const f32x4 *>(p);
+      else reg[i] = f32x4{p[0], p[1], p[2], p[3]};
     } else {
       f32x4 v;
       v.x = (k + 0 < kdim) ? p[0] : 0.0f;
@@ -131,16 +148,18 @@ __device__ __forceinline__ void fetch_kc(const float *__restrict__ base,
   }
 }
 
-// MC operand: thread t fetches k rows (t>>5) and (t>>5)+8, columns 4*(t&31)..+3.
-template <bool VEC>
+// MC operand, EXT columns: EXT/4 threads cover one k row with 16-byte loads.
+template <int EXT, bool VEC>
 __device__ __forceinline__ void fetch_mc(const float *__restrict__ base,
                                          long long ld_k, int col0, int ncols,
                                          int k0, int kdim, int tid,
-                                         f32x4 (&reg)[2]) {
-  const int c = col0 + (tid & 31) * 4;
+                                         f32x4 (&reg)[EXT / 64]) {
+  constexpr int TPR = EXT / 4;          // threads per k row
+  constexpr int RPP = NTHREADS / TPR;   // k rows per pass
+  const int c = col0 + (tid % TPR) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    int k = k0 + (tid >> 5) + i * 8;
+  for (int i = 0; i < EXT / 64; i++) {
+    int k = k0 + tid / TPR + i * RPP;
     if (k < kdim) {
       const float *p = base + (long long)k * ld_k;
       if (VEC && c + 3 < ncols) {
@@ -160,71 +179,105 @@ __device__ __forceinline__ void fetch_mc(const float *__restrict__ base,
   }
 }
 
-// im2col view of X: thread t owns output pixel (t&127) of the tile and k rows
-// (t>>7) + 2*i, i = 0..7.  The k row index is uniform across a wavefront.
+// im2col view of X, EXT pixels: thread t owns pixel (t % EXT) of the tile and
+// the 16*EXT/256 consecutive k rows starting at (t / EXT) * 16*EXT/256.  The k
+// rows are uniform across a wavefront, so their tap-table entries arrive with
+// one scalar load.
 struct PixelCtx {
-  const float *xbase;  // X + (n*c_total + g*c_in_g)*h*w, or null when past the edge
-  int iy0, ix0;
+  const float *xbase;       // X + (image*c_total + group*c_in_g)*h*w (image 0 past the edge)
+  int pbase;                // iy0*w + ix0
+  int iy0, ix0;             // corner of the receptive field (may be negative)
+  unsigned long long mask;  // bit t set: tap t falls inside the input (0 past the edge)
 };
 
-__device__ __forceinline__ void fetch_im2col(const ConvGeom &cv,
-                                             const PixelCtx &px, int k0,
-                                             int kdim, int tid,
-                                             f32x4 (&reg)[2]) {
-  const int khalf = __builtin_amdgcn_readfirstlane(tid >> 7);
-  float v[8];
+template <int EXT, bool MASK>
+__device__ __forceinline__ unsigned fetch_im2col(const ConvGeom &cv,
+                                                 const PixelCtx &px, int k0,
+                                                 int kdim, int tid,
+                                                 f32x4 (&reg)[EXT / 64]) {
+  constexpr int G = NTHREADS / EXT;  // wavefront groups, each owning L consecutive k rows
+  constexpr int L = BK / G;          // loads per thread
+  const int kfirst = k0 + __builtin_amdgcn_readfirstlane(tid / EXT) * L;
+  // the table is padded to a multiple of 16 entries; rows past kdim are
+  // masked by the k < kdim test
+  int2 e[L];
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    int k = k0 + khalf + 2 * i;
-    float val = 0.0f;
-    if (k < kdim) {
-      int2 e = cv.ktab[k];
-      int iy = px.iy0 + (e.y >> 16);
-      int ix = px.ix0 + (e.y & 0xffff);
-      if (px.xbase && (unsigned)iy < (unsigned)cv.h &&
-          (unsigned)ix < (unsigned)cv.w)
-        val = px.xbase[e.x + iy * cv.w + ix];
+  for (int i = 0; i < L; i++) e[i] = cv.ktab[kfirst + i];
+  unsigned okbits = 0;
+#pragma unroll
+  for (int i = 0; i < L; i++) {
+    bool ok;
+    if (MASK) {
+      ok = (px.mask >> e[i].y) & 1ull;
+    } else {
+      const int iy = px.iy0 + (e[i].y >> 16), ix = px.ix0 + (e[i].y & 0xffff);
+      ok = px.mask && (unsigned)iy < (unsigned)cv.h && (unsigned)ix < (unsigned)cv.w;
     }
-    v[i] = val;
+    ok = ok && kfirst + i < kdim;
+    // Unconditional load from a safe address; the value is zeroed when it is
+    // stored to LDS (stash_im2col), so nothing here waits for the load.
+    reg[i >> 2][i & 3] = px.xbase[ok ? px.pbase + e[i].x : 0];
+    okbits |= (ok ? 1u : 0u) << i;
   }
-  reg[0] = f32x4{v[0], v[1], v[2], v[3]};
-  reg[1] = f32x4{v[4], v[5], v[6], v[7]};
+  return okbits;
 }
 
 // ---- register -> LDS -------------------------------------------------------
+template <int EXT>
 __device__ __forceinline__ void stash_kc(float *tile, int tid,
-                                         const f32x4 (&reg)[2]) {
+                                         const f32x4 (&reg)[EXT / 64]) {
 #pragma unroll
-  for (int i = 0; i < 2; i++)
-    *reinterpret_cast<f32x4 *>(tile + ((tid >> 2) + i * 64) * LDK +
-                               (tid & 3) * 4) = reg[i];
+  for (int i = 0; i < EXT / 64; i++)
+    *reinterpret_cast<f32x4 *>(tile + ((tid >> 2) + i * 64) * LDK + (tid & 3) * 4) = reg[i];
 }
+template <int EXT>
 __device__ __forceinline__ void stash_mc(float *tile, int tid,
-                                         const f32x4 (&reg)[2]) {
+                                         const f32x4 (&reg)[EXT / 64]) {
+  constexpr int TPR = EXT / 4, RPP = NTHREADS / TPR, LD = EXT + MC_PAD;
 #pragma unroll
-  for (int i = 0; i < 2; i++)
-    *reinterpret_cast<f32x4 *>(tile + ((tid >> 5) + i * 8) * LDM +
-                               (tid & 31) * 4) = reg[i];
+  for (int i = 0; i < EXT / 64; i++)
+    *reinterpret_cast<f32x4 *>(tile + (tid / TPR + i * RPP) * LD + (tid % TPR) * 4) = reg[i];
 }
+template <int EXT>
 __device__ __forceinline__ void stash_im2col(float *tile, int tid,
-                                             const f32x4 (&reg)[2]) {
-  const int khalf = tid >> 7, pix = tid & 127;
+                                             const f32x4 (&reg)[EXT / 64],
+                                             unsigned okbits) {
+  constexpr int G = NTHREADS / EXT, L = BK / G, LD = EXT + MC_PAD;
+  const int kgroup = tid / EXT, pix = tid % EXT;
 #pragma unroll
-  for (int i = 0; i < 8; i++)
-    tile[(khalf + 2 * i) * LDM + pix] = reg[i >> 2][i & 3];
+  for (int i = 0; i < L; i++)
+    tile[(kgroup * L + i) * LD + pix] = ((okbits >> i) & 1u) ? reg[i >> 2][i & 3] : 0.0f;
 }
 
+constexpr int tile_floats(bool kc, int ext) { return kc ? ext * LDK : BK * (ext + MC_PAD); }
+
 // ---- the kernel -------------------------------------------------------------
-template <bool A_KC, int BMODE, bool VEC>
-__global__ __launch_bounds__(NTHREADS) void contraction_kernel(Params p) {
-  __shared__ __attribute__((aligned(16))) float lds_a[2][TILE_FLOATS];
-  __shared__ __attribute__((aligned(16))) float lds_b[2][TILE_FLOATS];
+// Workgroups per CU the register budget must allow: the 64-accumulator tiles
+// are held to 128 registers so that four of them share a CU, the
+// 16-accumulator tiles to 64 registers so that eight do.
+constexpr int min_blocks(int bm, int bn) {
+  return (bm == 128 && bn == 128) ? 4 : (bm * bn <= 64 * 64 ? 8 : 1);
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE_, bool VEC>
+__global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kernel(Params p) {
+  constexpr bool MASK = BMODE_ == B_IM2COL;
+  constexpr int BMODE = BMODE_ == B_IM2COL_BIG ? (int)B_IM2COL : BMODE_;
+  static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
+  constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
+  static_assert(MT >= 1 && NT >= 1, "tile too small for the wavefront grid");
+  constexpr int A_FLOATS = tile_floats(A_KC, BM);
+  constexpr int B_FLOATS = tile_floats(BMODE == B_KC, BN);
+  constexpr int LDA = BM + MC_PAD, LDB = BN + MC_PAD;
+  __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
+  __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;  // 2x2 wavefronts
+  const int wm = wave / WN, wn = wave % WN;
   const int li = lane & 31, half = lane >> 5;
+  const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
 
   int tm, tn;
   tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, &tm, &tn);
@@ -236,119 +289,162 @@ __global__ __launch_bounds__(NTHREADS) void contraction_kernel(Params p) {
   const long long lda = A_KC ? p.sA0 : p.sA1;
   const long long ldb = (BMODE == B_KC) ? p.sB1 : p.sB0;
 
-  PixelCtx px = {nullptr, 0, 0};
+  PixelCtx px = {p.B, 0, 0, 0, 0ull};
   if (BMODE == B_IM2COL) {
-    long long P = (long long)col0 + (tid & 127);
+    const long long P = (long long)col0 + (tid % BN);
+    const long long plane = (long long)p.cv.h * p.cv.w;
+    px.xbase = p.B + (long long)bz * p.cv.c_in_g * plane;
     if (P < p.cv.npix) {
-      int ohw = p.cv.oh * p.cv.ow;
-      int img = (int)(P / ohw);
-      int q = (int)(P - (long long)img * ohw);
-      int oy = q / p.cv.ow, ox = q - oy * p.cv.ow;
-      px.xbase = p.B + ((long long)img * p.cv.c_total + (long long)bz * p.cv.c_in_g) *
-                           p.cv.h * p.cv.w;
+      const int ohw = p.cv.oh * p.cv.ow;
+      const int img = (int)(P / ohw);
+      const int q = (int)(P - (long long)img * ohw);
+      const int oy = q / p.cv.ow, ox = q - oy * p.cv.ow;
+      px.xbase += (long long)img * p.cv.c_total * plane;
       px.iy0 = oy * p.cv.sh - p.cv.pt;
       px.ix0 = ox * p.cv.sw - p.cv.pl;
+      px.pbase = px.iy0 * p.cv.w + px.ix0;
+      if (MASK) {
+        unsigned long long m = 0;
+        for (int t = 0; t < p.cv.ntaps; t++) {
+          const int d = p.cv.taptab[t];
+          const int iy = px.iy0 + (d >> 16), ix = px.ix0 + (d & 0xffff);
+          if ((unsigned)iy < (unsigned)p.cv.h && (unsigned)ix < (unsigned)p.cv.w)
+            m |= 1ull << t;
+        }
+        px.mask = m;
+      } else {
+        px.mask = 1ull;
+      }
     }
   }
 
-  f32x16 acc[2][2];
+  f32x16 acc[MT][NT];
 #pragma unroll
-  for (int a = 0; a < 2; a++)
+  for (int a = 0; a < MT; a++)
 #pragma unroll
-    for (int b = 0; b < 2; b++)
+    for (int b = 0; b < NT; b++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
 
-  f32x4 ra[2], rb[2];
-  auto fetch = [&](int k0) {
-    if (A_KC)
-      fetch_kc<VEC>(A, lda, row0, p.m, k0, p.k, tid, ra);
-    else
-      fetch_mc<VEC>(A, lda, row0, p.m, k0, p.k, tid, ra);
-    if (BMODE == B_KC)
-      fetch_kc<VEC>(B, ldb, col0, p.n, k0, p.k, tid, rb);
-    else if (BMODE == B_MC)
-      fetch_mc<VEC>(B, ldb, col0, p.n, k0, p.k, tid, rb);
-    else
-      fetch_im2col(p.cv, px, k0, p.k, tid, rb);
+  // this workgroup's share of K
+  const int kbeg = p.ksplit > 1 ? (int)blockIdx.z * p.kchunk : 0;
+  const int kend = p.ksplit > 1 ? (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k) : p.k;
+
+  // Registers that carry one fetched K slab from global memory to LDS.
+  struct Staged {
+    f32x4 a[BM / 64], b[BN / 64];
+    unsigned ok;  // im2col only: which fetched taps lie inside the input
   };
-  auto stash = [&](int buf) {
+  auto fetch = [&](int k0, Staged &st) {
     if (A_KC)
-      stash_kc(lds_a[buf], tid, ra);
+      fetch_kc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
     else
-      stash_mc(lds_a[buf], tid, ra);
+      fetch_mc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
     if (BMODE == B_KC)
-      stash_kc(lds_b[buf], tid, rb);
+      fetch_kc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
     else if (BMODE == B_MC)
-      stash_mc(lds_b[buf], tid, rb);
+      fetch_mc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
     else
-      stash_im2col(lds_b[buf], tid, rb);
+      st.ok = fetch_im2col<BN, MASK>(p.cv, px, k0, kend, tid, st.b);
   };
-
-  const int nslabs = (p.k + BK - 1) / BK;
-  fetch(0);
-  stash(0);
-  __syncthreads();
-
-  for (int s = 0; s < nslabs; s++) {
-    const int cur = s & 1;
-    if (s + 1 < nslabs) fetch((s + 1) * BK);
-
+  auto stash = [&](int buf, const Staged &st) {
+    if (A_KC)
+      stash_kc<BM>(lds_a[buf], tid, st.a);
+    else
+      stash_mc<BM>(lds_a[buf], tid, st.a);
+    if (BMODE == B_KC)
+      stash_kc<BN>(lds_b[buf], tid, st.b);
+    else if (BMODE == B_MC)
+      stash_mc<BN>(lds_b[buf], tid, st.b);
+    else
+      stash_im2col<BN>(lds_b[buf], tid, st.b, st.ok);
+  };
+  // One K slab from LDS buffer `cur` through the matrix cores.
+  auto compute = [&](int cur) {
     const float *ta = lds_a[cur];
     const float *tb = lds_b[cur];
-    f32x4 av[2][2], bv[2][2];
+    f32x4 av[MT][2], bv[NT][2];
     if (A_KC) {
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++)
+      for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
           av[mt][j] = *reinterpret_cast<const f32x4 *>(
-              ta + (wm * 64 + mt * 32 + li) * LDK + 8 * j + 4 * half);
+              ta + (wrow + mt * 32 + li) * LDK + 8 * j + 4 * half);
     }
     if (BMODE == B_KC) {
 #pragma unroll
-      for (int nt = 0; nt < 2; nt++)
+      for (int nt = 0; nt < NT; nt++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
           bv[nt][j] = *reinterpret_cast<const f32x4 *>(
-              tb + (wn * 64 + nt * 32 + li) * LDK + 8 * j + 4 * half);
+              tb + (wcol + nt * 32 + li) * LDK + 8 * j + 4 * half);
     }
 #pragma unroll
     for (int st = 0; st < 8; st++) {
       const int kk = 8 * (st >> 2) + 4 * half + (st & 3);
-      float a_el[2], b_el[2];
+      float a_el[MT], b_el[NT];
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++)
-        a_el[mt] = A_KC ? av[mt][st >> 2][st & 3]
-                        : ta[kk * LDM + wm * 64 + mt * 32 + li];
+      for (int mt = 0; mt < MT; mt++)
+        a_el[mt] = A_KC ? av[mt][st >> 2][st & 3] : ta[kk * LDA + wrow + mt * 32 + li];
 #pragma unroll
-      for (int nt = 0; nt < 2; nt++)
+      for (int nt = 0; nt < NT; nt++)
         b_el[nt] = (BMODE == B_KC) ? bv[nt][st >> 2][st & 3]
-                                   : tb[kk * LDM + wn * 64 + nt * 32 + li];
+                                   : tb[kk * LDB + wcol + nt * 32 + li];
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++)
+      for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int nt = 0; nt < 2; nt++)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-              a_el[mt], b_el[nt], acc[mt][nt], 0, 0, 0);
+        for (int nt = 0; nt < NT; nt++)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_el[mt], b_el[nt],
+                                                             acc[mt][nt], 0, 0, 0);
     }
+  };
 
-    if (s + 1 < nslabs) stash(cur ^ 1);
+  const int nslabs = (kend - kbeg + BK - 1) / BK;
+  Staged st0;
+  fetch(kbeg, st0);
+  stash(0, st0);
+  __syncthreads();
+  // fetch slab s+1 while slab s computes (a second slab in flight was measured
+  // and bought nothing: the loop is not waiting on these loads)
+  for (int s = 0; s < nslabs; s++) {
+    const int cur = s & 1;
+    if (s + 1 < nslabs) fetch(kbeg + (s + 1) * BK, st0);
+    compute(cur);
+    if (s + 1 < nslabs) stash(cur ^ 1, st0);
     __syncthreads();
   }
 
   // ---- epilogue: lane holds column (li) of each 32x32 tile, rows
   // 8*(r/4) + 4*half + r%4 for accumulator register r.
+  if (p.ksplit > 1) {
+    // raw partial sums in plain [z][y][m][n] order; splitk_reduce_kernel adds
+    // the chunks in index order and applies the epilogue
+    float *part = p.partial + ((long long)blockIdx.z * gridDim.y + bz) * p.m * p.n;
 #pragma unroll
-  for (int nt = 0; nt < 2; nt++) {
-    const int col = col0 + wn * 64 + nt * 32 + li;
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = col0 + wcol + nt * 32 + li;
+      if (col >= p.n) continue;
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int row = row0 + wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          if (row < p.m) part[(long long)row * p.n + col] = acc[mt][nt][r];
+        }
+    }
+    return;
+  }
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++) {
+    const int col = col0 + wcol + nt * 32 + li;
     if (col >= p.n) continue;
     long long ybase;     // offset of (row 0, this column) in Y
     long long ystride;   // distance between consecutive rows in Y
     if (BMODE == B_IM2COL) {
-      int ohw = p.cv.oh * p.cv.ow;
-      int img = col / ohw;
-      int q = col - img * ohw;
+      const int ohw = p.cv.oh * p.cv.ow;
+      const int img = col / ohw;
+      const int q = col - img * ohw;
       ybase = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g) * ohw + q;
       ystride = ohw;
     } else {
@@ -356,10 +452,10 @@ __global__ __launch_bounds__(NTHREADS) void contraction_kernel(Params p) {
       ystride = p.n;
     }
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
+    for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int row = row0 + wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        const int row = row0 + wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
         if (row >= p.m) continue;
         float y = p.alpha * acc[mt][nt][r];
         if (p.C) {
@@ -398,17 +494,149 @@ __global__ void contraction_strided_kernel(Params p) {
   p.Y[off] = y;
 }
 
-template <bool A_KC, int BMODE>
-int launch(const Params &p, int nz, bool vec) {
-  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)nz);
+// Second pass of a split-K contraction: adds the ksplit partial sums of each
+// result element in chunk order (so the result does not depend on scheduling)
+// and applies the same epilogue as the single-pass kernel.
+template <bool CONV>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int nz) {
+  const long long per_z = (long long)p.m * p.n;
+  const long long total = per_z * nz;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int bz = (int)(i / per_z);
+    const long long rc = i - (long long)bz * per_z;
+    const int row = (int)(rc / p.n), col = (int)(rc - (long long)row * p.n);
+    float acc = 0.0f;
+    for (int s = 0; s < p.ksplit; s++) acc += p.partial[(long long)s * total + i];
+    float y = p.alpha * acc;
+    long long off;
+    if (CONV) {
+      const int ohw = p.cv.oh * p.cv.ow;
+      const int img = col / ohw, q = col - img * ohw;
+      off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
+      if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
+    } else {
+      off = i;
+      if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
+    }
+    if (p.R) y = y + p.R[off];
+    if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+    p.Y[off] = y;
+  }
+}
+
+// ---- host-side dispatch -------------------------------------------------------
+enum TileId { T128x128 = 0, T64x256 = 1, T64x128 = 2, T64x64 = 3 };
+const int kTileM[] = {128, 64, 64, 64};
+const int kTileN[] = {128, 256, 128, 64};
+
+// Tile choice by a small cost model: every CU works through ceil(tiles/CUs)
+// tiles, each costing its full area (rows or columns beyond the result are
+// wasted matrix-core work) divided by a measured per-shape efficiency (larger
+// tiles re-read less, smaller ones keep more wavefronts in flight).  64x256 is
+// never chosen here; it stays reachable through wdh_set_option.
+TileId pick_tile(int m, int n, int nz) {
+  const TileId cand[] = {T128x128, T64x128, T64x64};
+  const double eff[] = {1.00, 0.95, 0.93};
+  const long long cus = wdh::compute_units();
+  TileId best = T64x64;
+  double best_cost = 0;
+  for (int c = 0; c < 3; c++) {
+    const TileId t = cand[c];
+    const long long tiles =
+        (long long)((m + kTileM[t] - 1) / kTileM[t]) * ((n + kTileN[t] - 1) / kTileN[t]) * nz;
+    const double cost = (double)((tiles + cus - 1) / cus) * kTileM[t] * kTileN[t] / eff[c];
+    if (c == 0 || cost < best_cost) {
+      best = t;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
+int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
+
+// When even the smallest tile leaves the chip short of work (few result
+// elements, long K: ResNet stage-3/4 convs at 14x14 and 7x7), K is cut into
+// chunks that run as separate workgroups.
+int pick_split(long long tiles, int k) {
+  if (g_forced_split >= 1) {
+    int s = g_forced_split;
+    int max_s = (k + BK - 1) / BK;
+    return s < max_s ? s : (max_s > 0 ? max_s : 1);
+  }
+  const long long target = 4LL * wdh::compute_units();
+  if (tiles * 2 >= target) return 1;
+  long long s = (target + tiles - 1) / tiles;
+  const long long max_s = k / (4 * BK);  // keep at least 4 slabs per chunk
+  if (s > max_s) s = max_s;
+  if (s > 32) s = 32;
+  return s < 2 ? 1 : (int)s;
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE>
+int launch_tile(Params &p, int nz, bool vec) {
+  p.tiles_m = (p.m + BM - 1) / BM;
+  p.tiles_n = (p.n + BN - 1) / BN;
+  const long long tiles = (long long)p.tiles_m * p.tiles_n;
+  int split = pick_split(tiles * nz, p.k);
+  wdh_buf scratch = 0;
+  p.ksplit = 1;
+  if (split > 1) {
+    p.kchunk = ((p.k + split - 1) / split + BK - 1) / BK * BK;
+    split = (p.k + p.kchunk - 1) / p.kchunk;
+  }
+  if (split > 1) {
+    const size_t bytes = (size_t)split * nz * p.m * p.n * sizeof(float);
+    scratch = wdh_alloc(bytes);
+    if (!scratch) return WDH_ENOMEM;
+    p.partial = (float *)wdh::resolve(scratch, nullptr);
+    p.ksplit = split;
+  }
+  dim3 grid((unsigned)tiles, (unsigned)nz, (unsigned)p.ksplit);
   if (vec)
-    hipLaunchKernelGGL((contraction_kernel<A_KC, BMODE, true>), grid,
+    hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, true>), grid,
                        dim3(NTHREADS), 0, wdh::stream(), p);
   else
-    hipLaunchKernelGGL((contraction_kernel<A_KC, BMODE, false>), grid,
+    hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, false>), grid,
                        dim3(NTHREADS), 0, wdh::stream(), p);
-  WDH_LAUNCH_CHECK();
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && p.ksplit > 1) {
+    const long long total = (long long)p.m * p.n * nz;
+    long long blocks = (total + 255) / 256;
+    const long long cap = 16LL * wdh::compute_units();
+    if (blocks > cap) blocks = cap;
+    if (BMODE == B_IM2COL || BMODE == B_IM2COL_BIG)
+      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
+                         wdh::stream(), p, nz);
+    else
+      hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
+                         wdh::stream(), p, nz);
+    e = hipGetLastError();
+  }
+  // The scratch block goes back to the pool right away: whoever gets it next
+  // touches it through the same stream, behind the two kernels above.
+  if (scratch) (void)wdh_free(scratch);
+  if (e != hipSuccess)
+    return wdh::fail(WDH_EHIP, "contraction launch failed: %s", hipGetErrorString(e));
   return WDH_OK;
+}
+
+template <bool A_KC, int BMODE>
+int launch(Params &p, int nz, bool vec) {
+  // Convs measured best on 64x64 tiles at every ResNet-50 layer shape (more
+  // wavefronts in flight to cover the gather's latency); Gemm/MatMul use the
+  // cost model.
+  const bool conv = BMODE == B_IM2COL || BMODE == B_IM2COL_BIG;
+  TileId t = g_forced_tile >= 0 ? (TileId)g_forced_tile
+                                : (conv ? T64x64 : pick_tile(p.m, p.n, nz));
+  switch (t) {
+    case T128x128: return launch_tile<128, 128, 2, 2, A_KC, BMODE>(p, nz, vec);
+    case T64x256: return launch_tile<64, 256, 1, 4, A_KC, BMODE>(p, nz, vec);
+    case T64x128: return launch_tile<64, 128, 1, 4, A_KC, BMODE>(p, nz, vec);
+    default: return launch_tile<64, 64, 2, 2, A_KC, BMODE>(p, nz, vec);
+  }
 }
 
 bool aligned16(const void *ptr) { return ((uintptr_t)ptr & 15) == 0; }
@@ -422,6 +650,24 @@ long long span(long long nb, long long sb, long long n0, long long s0,
 }  // namespace
 
 using wdh::fail;
+
+extern "C" int wdh_set_option(const char *name, int value) {
+  if (!name) return fail(WDH_EINVAL, "wdh_set_option: name is NULL");
+  if (strcmp(name, "contraction_tile") == 0) {
+    if (value < -1 || value > T64x64)
+      return fail(WDH_EINVAL, "wdh_set_option: contraction_tile %d outside -1..%d", value,
+                  (int)T64x64);
+    g_forced_tile = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "split_k") == 0) {
+    if (value < -1 || value == 0 || value > 64)
+      return fail(WDH_EINVAL, "wdh_set_option: split_k %d (use -1 or 1..64)", value);
+    g_forced_split = value;
+    return WDH_OK;
+  }
+  return fail(WDH_EINVAL, "wdh_set_option: unknown option \"%s\"", name);
+}
 
 extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
                         int batch, int m, int n, int k, int64_t sAb,
@@ -466,15 +712,13 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   p.sBb = sBb; p.sB0 = sB0; p.sB1 = sB1;
   p.sC0 = sC0; p.sC1 = sC1;
   p.alpha = alpha; p.beta = beta; p.epilogue = epilogue;
-  p.tiles_m = (m + BM - 1) / BM;
-  p.tiles_n = (n + BN - 1) / BN;
 
   // Which index of each operand is contiguous?  An extent of 1 makes the
   // stride along it irrelevant.
   const bool a_kc = (sA1 == 1 || k == 1), a_mc = (sA0 == 1 || m == 1);
   const bool b_kc = (sB0 == 1 || k == 1), b_mc = (sB1 == 1 || n == 1);
   if (!(a_kc || a_mc) || !(b_kc || b_mc) ||
-      (long long)p.tiles_m * p.tiles_n > 0x7fffffffLL) {
+      ((long long)(m + 63) / 64) * ((n + 63) / 64) > 0x7fffffffLL) {
     dim3 grid((unsigned)(((long long)m * n + 255) / 256), (unsigned)batch);
     hipLaunchKernelGGL(contraction_strided_kernel, grid, dim3(256), 0,
                        wdh::stream(), p);
@@ -506,24 +750,29 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
 
 namespace {
 
-// One lookup table per conv geometry, built on the host once and kept on the
-// device for the life of the library: entry k = (ci, ky, kx) holds the offset
-// of that tap relative to the (iy0, ix0) corner of the receptive field and
-// the tap's (dy, dx).
+// Tap tables per conv geometry, built on the host once and kept on the device
+// for the life of the library.
 struct KtabKey {
   int c_in_g, kh, kw, dh, dw, h, w;
   bool operator<(const KtabKey &o) const {
     return memcmp(this, &o, sizeof(*this)) < 0;
   }
 };
+struct KtabVal {
+  int2 *ktab;
+  int *taptab;
+};
 
-std::map<KtabKey, int2 *> g_ktabs;
+std::map<KtabKey, KtabVal> g_ktabs;
 
 }  // namespace
 
 namespace wdh {
 void release_conv_tables() {
-  for (auto &kv : g_ktabs) (void)hipFree(kv.second);
+  for (auto &kv : g_ktabs) {
+    (void)hipFree(kv.second.ktab);
+    (void)hipFree(kv.second.taptab);
+  }
   g_ktabs.clear();
 }
 }  // namespace wdh
@@ -580,42 +829,51 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   if (!wdh::operand(hY, out_bytes, "wdh_conv2d: Y", &ptr)) return WDH_EINVAL;
   p.Y = (float *)ptr;
 
+  const int ntaps = kh * kw;
+  const bool mask_mode = ntaps <= 64;
   KtabKey key;
   memset(&key, 0, sizeof(key));
   key.c_in_g = c_in_g; key.kh = kh; key.kw = kw; key.dh = dh; key.dw = dw;
   key.h = h; key.w = w;
   auto it = g_ktabs.find(key);
   if (it == g_ktabs.end()) {
-    std::vector<int2> tab((size_t)kdim);
+    std::vector<int2> tab((size_t)((kdim + BK - 1) / BK * BK), int2{0, 0});
+    std::vector<int> taps((size_t)ntaps);
     size_t idx = 0;
     for (int ci = 0; ci < c_in_g; ci++)
       for (int ky = 0; ky < kh; ky++)
         for (int kx = 0; kx < kw; kx++) {
-          tab[idx].x = ci * h * w;
-          tab[idx].y = ((ky * dh) << 16) | (kx * dw);
+          const int packed = ((ky * dh) << 16) | (kx * dw);
+          tab[idx].x = ci * h * w + ky * dh * w + kx * dw;
+          tab[idx].y = mask_mode ? ky * kw + kx : packed;
+          taps[ky * kw + kx] = packed;
           idx++;
         }
-    int2 *dev = nullptr;
-    if (hipMalloc(&dev, tab.size() * sizeof(int2)) != hipSuccess) {
+    KtabVal val = {nullptr, nullptr};
+    if (hipMalloc(&val.ktab, tab.size() * sizeof(int2)) != hipSuccess ||
+        hipMalloc(&val.taptab, taps.size() * sizeof(int)) != hipSuccess) {
       (void)hipGetLastError();
+      if (val.ktab) (void)hipFree(val.ktab);
       return fail(WDH_ENOMEM, "wdh_conv2d: tap table allocation failed");
     }
-    // synchronous copy: the host vector dies at the end of this scope
-    WDH_HIP_CHECK(hipMemcpy(dev, tab.data(), tab.size() * sizeof(int2),
+    // synchronous copies: the host vectors die at the end of this scope
+    WDH_HIP_CHECK(hipMemcpy(val.ktab, tab.data(), tab.size() * sizeof(int2),
                             hipMemcpyHostToDevice));
-    it = g_ktabs.emplace(key, dev).first;
+    WDH_HIP_CHECK(hipMemcpy(val.taptab, taps.data(), taps.size() * sizeof(int),
+                            hipMemcpyHostToDevice));
+    it = g_ktabs.emplace(key, val).first;
   }
 
   p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
   p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
   p.sBb = 0; p.sB0 = 0; p.sB1 = 0;
   p.alpha = 1.0f; p.beta = 1.0f; p.epilogue = epilogue;
-  p.tiles_m = (p.m + BM - 1) / BM;
-  p.tiles_n = (p.n + BN - 1) / BN;
   p.cv.c_in_g = c_in_g; p.cv.h = h; p.cv.w = w; p.cv.oh = oh; p.cv.ow = ow;
-  p.cv.kh = kh; p.cv.kw = kw; p.cv.pt = pt; p.cv.pl = pl; p.cv.sh = sh; p.cv.sw = sw;
+  p.cv.pt = pt; p.cv.pl = pl; p.cv.sh = sh; p.cv.sw = sw;
   p.cv.c_total = c; p.cv.cout_total = cout; p.cv.cout_g = cout_g;
-  p.cv.npix = npix; p.cv.ktab = it->second;
-  const bool vec = aligned16(p.A) && kdim % 4 == 0;
-  return launch<true, B_IM2COL>(p, group, vec);
+  p.cv.ntaps = ntaps;
+  p.cv.npix = npix; p.cv.ktab = it->second.ktab; p.cv.taptab = it->second.taptab;
+  const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
+  if (mask_mode) return launch<true, B_IM2COL>(p, group, vec);
+  return launch<true, B_IM2COL_BIG>(p, group, vec);
 }

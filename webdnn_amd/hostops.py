@@ -149,6 +149,9 @@ class HipContext:
         return {"name": name.value.decode(), "compute_units": cu.value, "clock_mhz": mhz.value,
                 "hbm_bytes": hbm.value}
 
+    def set_option(self, name, value):
+        call("wdh_set_option", name.encode(), int(value))
+
     def empty_tensor(self, dims, data_type="float32"):
         return HipTensor(self, dims, data_type)
 
