@@ -1,0 +1,104 @@
+"""The Node.js host on the hip backend: WebDNN.load() + runner.run() on a real MI355X, against the
+same graph on the cpu path (the JavaScript oracle) and against the C oracle.
+
+Every run is strict: the per-node CPU retry of the reference's runner is off, and the per-backend
+node counter must show every node on `hip`, so that a fallback cannot fake a pass."""
+import numpy as np
+import pytest
+
+import graph_ref
+import node_runner
+from util import assert_bit_exact, assert_close_max
+from webdnn_amd import modelgen
+
+pytestmark = pytest.mark.gpu
+
+
+def run_both(tmp_path, model_bytes, feeds, fuse=True):
+    (tmp_path / "model.onnx").write_bytes(model_bytes)
+    model = modelgen.parse_model(model_bytes)
+    ordered = [feeds[n] for n, _ in model["inputs"]]
+    hip, report = node_runner.run_model(str(tmp_path), ordered, "hip", strict=True, fuse=fuse)
+    assert report["backend"] == "hip"
+    assert list(report["stats"]["nodesByBackend"]) == ["hip"], report["stats"]
+    assert report["stats"]["retriedOnCpu"] == []
+    return model, hip, report
+
+
+def test_gemm_config1(tmp_path):
+    data, _ = modelgen.gemm_model()
+    A = np.random.default_rng(1).uniform(-1, 1, (256, 512)).astype(np.float32)
+    model, hip, _ = run_both(tmp_path, data, {"A": A})
+    want = graph_ref.run_graph(model, {"A": A})["Y"]
+    assert_close_max(hip[0], want, 1e-4, "config 1 through the runner")
+
+
+def test_ffn_config2_fused_and_unfused(tmp_path):
+    data, _ = modelgen.ffn_model()
+    X = np.random.default_rng(2).standard_normal((8, 512, 768)).astype(np.float32)
+    model, fused, rep_f = run_both(tmp_path, data, {"X": X}, fuse=True)
+    _, plain, rep_p = run_both(tmp_path, data, {"X": X}, fuse=False)
+    assert rep_p["nodes"] == 5 and rep_f["nodes"] == 2          # MatMul+Add+Relu, MatMul+Add
+    assert_bit_exact(fused[0], plain[0], "fusion does not change the result")
+    rows = np.sort(np.random.default_rng(3).choice(8 * 512, 48, replace=False))
+    sub = modelgen.parse_model(data)
+    want = graph_ref.run_graph(sub, {"X": X.reshape(-1, 768)[rows]})["out"]
+    assert_close_max(fused[0].reshape(-1, 768)[rows], want, 1e-4, "config 2 rows")
+
+
+def test_conv_config3(tmp_path):
+    data, _ = modelgen.conv_model()
+    X = np.random.default_rng(4).uniform(0, 1, (32, 64, 56, 56)).astype(np.float32)
+    model, hip, rep = run_both(tmp_path, data, {"X": X})
+    assert rep["nodes"] == 1                                        # Conv+Relu fused
+    want = graph_ref.run_graph(model, {"X": X})["Y"]
+    assert_close_max(hip[0], want, 1e-4, "config 3 through the runner")
+
+
+def test_resnet_tiny_matches_cpu_path(tmp_path):
+    data, _ = modelgen.resnet50_model(batch=2, image=64, classes=10, width=16, blocks=(2, 1, 1, 1))
+    X = np.random.default_rng(5).standard_normal((2, 3, 64, 64)).astype(np.float32)
+    model, hip, rep = run_both(tmp_path, data, {"input": X})
+    cpu, rep_cpu = node_runner.run_model(str(tmp_path), [X], "cpu", oracle_cpu=True)
+    assert rep_cpu["stats"]["nodesByBackend"] == {"cpu": rep_cpu["nodes"]}
+    assert np.abs(hip[0] - cpu[0]).max() <= 1e-3, "logits within 1e-3 of the cpu backend"
+    _, plain, _ = run_both(tmp_path, data, {"input": X}, fuse=False)
+    assert_bit_exact(hip[0], plain[0], "fusion does not change the logits")
+
+
+def test_resnet50_batch32_logits(tmp_path):
+    """Config 4 at full size: logits within 1e-3 (absolute) of the CPU oracle."""
+    data, g = modelgen.resnet50_model()
+    X = np.random.default_rng(6).standard_normal((32, 3, 224, 224)).astype(np.float32)
+    model, hip, rep = run_both(tmp_path, data, {"input": X})
+    assert hip[0].shape == (32, 1000) and np.isfinite(hip[0]).all()
+    # the oracle follows 4 of the 32 images (every op of the graph is per-image)
+    pick = [0, 7, 19, 31]
+    want = graph_ref.run_graph(model, {"input": X[pick]})["logits"]
+    err = np.abs(hip[0][pick] - want).max()
+    assert err <= 1e-3, "max |logit diff| %.3e" % err
+
+
+def test_non_strict_falls_back_per_node(tmp_path):
+    """An operator the hip backend rejects at run time is retried once on the cpu operators
+    (reference: core/runnerImpl.ts:511-520) when strict mode is off, and fails loudly when it is on."""
+    g = modelgen.GraphBuilder(0)
+    g.op("Softmax", ["X"], "s", axis=1)          # non-last axis: hip throws, and so does the cpu operator
+    data = g.finish([("X", [2, 3, 4])], [("s", [2, 3, 4])])
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.zeros((2, 3, 4), np.float32)
+    with pytest.raises(RuntimeError, match="only reducing final axis"):
+        node_runner.run_model(str(tmp_path), [X], "hip", strict=True)
+    with pytest.raises(RuntimeError, match="only reducing final axis"):
+        node_runner.run_model(str(tmp_path), [X], "hip", strict=False, oracle_cpu=True)
+    g = modelgen.GraphBuilder(0)
+    g.op("Relu", ["X"], "r")
+    g.op("ReduceMean", ["r"], "m", axes=[0], keepdims=1)   # hip supports only the last axis -> cpu retry
+    g.op("Relu", ["m"], "Y")
+    data = g.finish([("X", [4, 6])], [("Y", [1, 6])])
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(7).standard_normal((4, 6)).astype(np.float32)
+    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=False, oracle_cpu=True)
+    assert rep["stats"]["retriedOnCpu"] == ["ReduceMean_1"]
+    assert rep["stats"]["nodesByBackend"] == {"hip": 2, "cpu": 1}
+    np.testing.assert_allclose(outs[0], np.maximum(np.maximum(X, 0).mean(0, keepdims=True), 0), rtol=1e-6)

@@ -63,9 +63,10 @@ def build_addon(verbose=True):
         return None
     if verbose:
         print("[build] gcc addon.c")
-    _run(["gcc", "-O2", "-fPIC", "-shared", "-std=c11", "-Wall",
+    # links against the library next to it ($ORIGIN), so the pair can be moved together
+    _run(["gcc", "-O2", "-fPIC", "-shared", "-std=c11", "-Wall", "-DNODE_GYP_MODULE_NAME=webdnn_hip",
           "-I", "/usr/include/node", "-I", os.path.join(ROOT, "include"),
-          ADDON_SRC, "-o", ADDON, "-ldl"])
+          ADDON_SRC, "-o", ADDON, "-L", LIBDIR, "-lwebdnn_hip", "-Wl,-rpath,$ORIGIN"])
     return ADDON
 
 

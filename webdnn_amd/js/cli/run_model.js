@@ -1,0 +1,123 @@
+#!/usr/bin/env node
+"use strict";
+// Runs an ONNX model directory through the descriptor runner from the command line.
+//
+//   node run_model.js --model DIR [--onnx model.onnx] [--backend hip|cpu]
+//        --inputs a.bin[,b.bin...] --output out.bin
+//        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure]
+//        [--cpu-entries module.js]
+//
+// Inputs are raw little-endian files (float32, or int32 where the graph input says
+// so) in the order of the graph's non-initializer inputs; outputs are written the same
+// way, concatenated.  One JSON line on stdout reports output dims, per-run wall times,
+// the per-backend node counts of the last run and, with --measure, per-node device
+// times.  --cpu-entries registers extra cpu OperatorEntry objects exported by a module
+// (getOpEntries()); parity tests and the CPU baseline pass the CPU restatement of the
+// reference operators that way, the product itself ships hot-path operators for hip only.
+//
+// Methodology follows the reference's harness (example/benchmark/runner/bench.js:130-167):
+// warm-up runs, then timed runner.run() calls.
+const fs = require("fs");
+const path = require("path");
+const WebDNN = require("../index");
+const { registerOperators } = require("../core/operatorTable");
+
+function parseArgs(argv) {
+  const args = { backend: "hip", warmup: 0, runs: 1, onnx: "model.onnx" };
+  for (let i = 2; i < argv.length; i++) {
+    const a = argv[i];
+    const next = () => {
+      if (i + 1 >= argv.length) throw new Error(`${a} needs a value`);
+      return argv[++i];
+    };
+    if (a === "--model") args.model = next();
+    else if (a === "--onnx") args.onnx = next();
+    else if (a === "--backend") args.backend = next();
+    else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
+    else if (a === "--output") args.output = next();
+    else if (a === "--strict") args.strict = true;
+    else if (a === "--no-fuse") args.noFuse = true;
+    else if (a === "--warmup") args.warmup = parseInt(next(), 10);
+    else if (a === "--runs") args.runs = parseInt(next(), 10);
+    else if (a === "--measure") args.measure = true;
+    else if (a === "--cpu-entries") args.cpuEntries = next();
+    else if (a === "--tile") args.tile = parseInt(next(), 10);
+    else throw new Error(`unknown argument ${a}`);
+  }
+  if (!args.model) throw new Error("--model is required");
+  return args;
+}
+
+async function main() {
+  const args = parseArgs(process.argv);
+  if (args.cpuEntries) registerOperators(require(path.resolve(args.cpuEntries)).getOpEntries());
+  const hipOption = { strict: !!args.strict, fuse: !args.noFuse };
+  if (args.tile != null) hipOption.contractionTile = args.tile;
+  const runner = await WebDNN.load(args.model, {
+    backendOrder: args.backend === "cpu" ? ["cpu"] : ["hip", "cpu"],
+    backendOptions: { hip: hipOption },
+    onnxBaseName: args.onnx,
+  });
+  if (args.backend === "hip" && runner.backendName !== "hip") {
+    throw new Error("hip backend was requested but is not available");
+  }
+  const graphInputs = runner.inputsWithoutInitializer;
+  const files = args.inputs || [];
+  if (files.length !== graphInputs.length) {
+    throw new Error(`model has ${graphInputs.length} inputs, ${files.length} files given`);
+  }
+  const inputs = graphInputs.map((gi, idx) => {
+    const tt = gi.type.tensorType;
+    const dims = tt.shape.dim.map((d) => d.dimValue);
+    const dataType = tt.elemType === 1 ? "float32" : "int32";
+    const buf = fs.readFileSync(files[idx]);
+    const Ctor = dataType === "float32" ? Float32Array : Int32Array;
+    const copy = new Uint8Array(buf.byteLength);
+    copy.set(buf);
+    const data = new Ctor(copy.buffer, 0, copy.byteLength / 4);
+    const expect = dims.reduce((a, b) => a * b, 1);
+    if (data.length !== expect) throw new Error(`${files[idx]}: ${data.length} elements, graph input needs ${expect}`);
+    return new WebDNN.CPUTensor(dims, dataType, data);
+  });
+
+  for (let i = 0; i < args.warmup; i++) await runner.run(inputs);
+  const times = [];
+  let outputs = null;
+  for (let i = 0; i < args.runs; i++) {
+    const t0 = process.hrtime.bigint();
+    outputs = await runner.run(inputs, { measurePerformance: !!args.measure && i === args.runs - 1 });
+    times.push(Number(process.hrtime.bigint() - t0) / 1e6);
+  }
+  if (args.output) {
+    const fd = fs.openSync(args.output, "w");
+    for (const t of outputs) {
+      const d = t.data;
+      fs.writeSync(fd, Buffer.from(d.buffer, d.byteOffset, d.byteLength));
+    }
+    fs.closeSync(fd);
+  }
+  const report = {
+    backend: runner.backendName,
+    outputs: outputs.map((t, i) => ({ name: runner.getOutputNames()[i], dims: t.dims, dataType: t.dataType })),
+    msPerRun: times,
+    stats: runner.lastRunStats,
+    nodes: runner.model.graph.node.length,
+    node: process.version,
+  };
+  if (args.measure && runner.lastPerformance) {
+    report.performance = runner.lastPerformance.map((p) => ({
+      name: p.name, opType: p.opType, backend: p.backend, outputDims: p.outputDims,
+      elapsed: p.elapsed, deviceElapsed: p.deviceElapsed,
+    }));
+  }
+  if (runner.backendContexts.hip && runner.backendContexts.hip.initialized) {
+    report.device = runner.backendContexts.hip.deviceInfo();
+    report.memory = runner.backendContexts.hip.memStats();
+  }
+  process.stdout.write(JSON.stringify(report) + "\n");
+}
+
+main().catch((e) => {
+  process.stderr.write(`run_model: ${e && e.stack ? e.stack : e}\n`);
+  process.exit(1);
+});

@@ -1,0 +1,300 @@
+"use strict";
+// The descriptor runner: loads an ONNX model and interprets it node by node.
+// Reference: src/descriptor_runner/core/runnerImpl.ts:42-597, with a `hip` slot in
+// every place where the reference hard-codes its closed backend set
+// (BackendContexts :35-40, tensorsForBackends :323-328, the context switch :470-486,
+// end-of-run disposal :574-582).
+//
+// Additions for the hip backend (none changes what a model computes):
+//   * strict mode (backendOptions.hip.strict): the one-time retry of a failed node on
+//     the cpu operators (:511-520) is switched off, so a benchmark or parity run cannot
+//     silently pass on the fallback;
+//   * lastRunStats: how many nodes ran on which backend, and which were retried;
+//   * measurePerformance uses HIP events on the library's stream for hip nodes
+//     (Date.now() only sees enqueue time there).
+const fs = require("fs");
+const path = require("path");
+const { backends, backendsWithoutCPU } = require("../interface/constants");
+const { nonnull, clipToInt32 } = require("../util");
+const { findTensorReleaseTiming, modelTransform } = require("./modelTransform");
+const { instantiateOperator } = require("./operatorTable");
+const { decodeModel, DataType } = require("./onnxProto");
+const { tensorProtoToArray } = require("../operators/operatorUtil");
+const { getLogger } = require("../logging");
+
+const logger = getLogger("WebDNN.runner");
+
+class RunnerImpl {
+  // backendContexts: { cpu, hip? };  options: { strict?, fuse? }
+  constructor(backendOrder, backendContexts, options) {
+    this.backendOrder = backendOrder;
+    this.backendContexts = backendContexts;
+    this.backendName = backendOrder[0];
+    this.options = options || {};
+    this.loaded = false;
+    this.model = null;
+    this.tensorMoveOptions = {};
+    this.forceOperatorBackendOrder = {};
+    this.lastRunStats = null;
+    this.lastPerformance = null;
+  }
+
+  async loadModel(directory, onnxBasename) {
+    const bytes = fs.readFileSync(path.join(directory, onnxBasename));
+    this.loadModelFromBytes(bytes, directory);
+  }
+
+  // `bytes`: the serialized ModelProto; `directory`: where external weight files live
+  loadModelFromBytes(bytes, directory) {
+    this.model = decodeModel(new Uint8Array(bytes.buffer, bytes.byteOffset, bytes.byteLength));
+    modelTransform(this.model, this.backendOrder, { fuse: this.options.fuse });
+    if (this.model.opsetImport.length !== 1) {
+      logger.warn("Specifying multiple opset_import is not supported. Using first one.");
+    }
+    if (this.model.opsetImport.length === 0) throw new Error("model has no opset_import");
+    this.opset = clipToInt32(this.model.opsetImport[0].version);
+    this.initializerTensors = new Map();
+    for (const [name, tensor] of this.extractInitializerTensor().entries()) {
+      this.initializerTensors.set(name, tensor);
+    }
+    for (const [name, tensor] of this.loadExternalInitializerTensor(directory).entries()) {
+      this.initializerTensors.set(name, tensor);
+    }
+    this.copiedInitializerTensors = new Map();
+    for (const backend of this.backendOrder) {
+      if (backend !== "cpu") this.copiedInitializerTensors.set(backend, new Map());
+    }
+    this.inputsWithoutInitializer = this.model.graph.input.filter(
+      (v) => v.name && !this.initializerTensors.has(v.name)
+    );
+    for (const md of this.model.metadataProps) {
+      if (md.key === "WebDNN2.TensorMoveOptions") this.tensorMoveOptions = JSON.parse(md.value);
+      if (md.key === "WebDNN2.ForceOperatorBackendOrder") this.forceOperatorBackendOrder = JSON.parse(md.value);
+    }
+    this.loaded = true;
+  }
+
+  // FLOAT / INT64 (clipped to int32) / INT32 initializers become CPU tensors; anything
+  // else throws (runnerImpl.ts:136-233).
+  extractInitializerTensor() {
+    const tensors = new Map();
+    for (const initializer of this.model.graph.initializer) {
+      if (![DataType.FLOAT, DataType.INT64, DataType.INT32].includes(initializer.dataType)) {
+        throw new Error(`Unsupported initializer dataType ${initializer.dataType}`);
+      }
+      const { dims, dataType, data } = tensorProtoToArray(initializer);
+      tensors.set(initializer.name, this.backendContexts.cpu.emptyTensor(dims, dataType, data));
+    }
+    return tensors;
+  }
+
+  // Optimized models keep their weights in WDN2 tensor files named by metadata
+  // (runnerImpl.ts:235-268).
+  loadExternalInitializerTensor(directory) {
+    for (const md of this.model.metadataProps) {
+      if (md.key === "WebDNN2.WeightPaths") {
+        const { TensorLoaderImpl } = require("./tensorLoaderImpl");
+        const paths = md.value.split(":").map((bn) => path.join(directory || ".", bn));
+        return new TensorLoaderImpl(paths, this.backendContexts.cpu).loadAllSync();
+      }
+    }
+    return new Map();
+  }
+
+  getInputNames() {
+    return this.inputsWithoutInitializer.map((gi) => gi.name);
+  }
+
+  getOutputNames() {
+    return nonnull(this.model).graph.output.map((gi) => gi.name);
+  }
+
+  contextFor(backend) {
+    const context = this.backendContexts[backend];
+    if (!context) throw new Error(`No context for backend ${backend}`);
+    return context;
+  }
+
+  async run(inputs, options) {
+    const opts = options || {};
+    if (!this.model || !this.loaded) throw new Error("not initialized");
+    if (!inputs) throw new Error("inputs are required");
+    const graph = this.model.graph;
+    const tensorsForBackends = {};
+    for (const backend of backends) tensorsForBackends[backend] = new Map();
+
+    for (const [name, tensor] of this.initializerTensors.entries()) tensorsForBackends.cpu.set(name, tensor);
+    for (const [backend, kv] of this.copiedInitializerTensors.entries()) {
+      for (const [name, tensor] of kv.entries()) tensorsForBackends[backend].set(name, tensor);
+    }
+
+    if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
+    for (let i = 0; i < inputs.length; i++) {
+      tensorsForBackends.cpu.set(this.inputsWithoutInitializer[i].name, inputs[i]);
+    }
+
+    const tensorReleaseTiming = findTensorReleaseTiming(this.model, new Set(this.initializerTensors.keys()));
+    const nodePerformances = [];
+    const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length };
+    const strict = !!this.options.strict;
+    const hip = this.backendContexts.hip;
+    const useEvents = !!opts.measurePerformance && hip && hip.initialized && graph.node.length * 2 <= 4096;
+
+    try {
+      for (let i = 0; i < graph.node.length; i++) {
+        const nodeStartTime = Date.now(),
+          node = graph.node[i],
+          opType = nonnull(node.opType);
+        let actualBackend, actualInputDims, actualOutputDims;
+        let backendOrderForNode = this.forceOperatorBackendOrder[node.name] || this.backendOrder;
+        let firstTry = true;
+
+        // eslint-disable-next-line no-constant-condition
+        while (true) {
+          try {
+            // where does each input live?
+            const currentTensorsBackends = [];
+            for (const inputName of node.input) {
+              const bs = [];
+              for (const backend of backendOrderForNode) {
+                if (tensorsForBackends[backend].has(inputName)) bs.push(backend);
+              }
+              if (bs.length === 0) {
+                // a forced order such as ["hip"] must still find tensors that sit on the cpu
+                for (const backend of backends) {
+                  if (tensorsForBackends[backend].has(inputName)) bs.push(backend);
+                }
+              }
+              currentTensorsBackends.push(bs);
+            }
+            const operator = instantiateOperator(opType, this.opset, backendOrderForNode, currentTensorsBackends);
+            if (!operator) {
+              throw new Error(`Operator implementation for ${opType}, opset=${this.opset} does not exist.`);
+            }
+            operator.initialize(nonnull(node.attribute));
+            const requirement = operator.getTensorBackendRequirement(node.input.length, node.output.length);
+            const operatorInputs = [];
+            for (let j = 0; j < node.input.length; j++) {
+              const inputName = node.input[j],
+                reqBackend = requirement[j];
+              if (!reqBackend) {
+                // anywhere will do
+                const where = currentTensorsBackends[j][0];
+                const t = where && tensorsForBackends[where].get(inputName);
+                if (!t) throw new Error(`Input ${inputName} not found`);
+                operatorInputs.push(t);
+                continue;
+              }
+              const t = tensorsForBackends[reqBackend].get(inputName);
+              if (t) {
+                operatorInputs.push(t);
+                continue;
+              }
+              let found = false;
+              for (const otherBackend of this.backendOrder) {
+                const otherT = tensorsForBackends[otherBackend].get(inputName);
+                if (otherT) {
+                  const movedT = await this.contextFor(reqBackend).moveTensor(
+                    otherT,
+                    this.tensorMoveOptions[inputName] || {}
+                  );
+                  tensorsForBackends[reqBackend].set(inputName, movedT);
+                  operatorInputs.push(movedT);
+                  found = true;
+                  break;
+                }
+              }
+              if (!found) throw new Error(`Input ${inputName} not found`);
+            }
+
+            const context = this.contextFor(operator.backend);
+            logger.debug(`Running ${node.name}(${opType}) on ${operator.backend}`);
+            if (useEvents) hip.native.eventRecord(2 * i);
+            const operatorOutputs = await operator.run(context, operatorInputs, node.output.length);
+            if (useEvents) hip.native.eventRecord(2 * i + 1);
+            actualInputDims = operatorInputs.map((t) => t.dims);
+            actualOutputDims = operatorOutputs.map((t) => t.dims);
+            for (let j = 0; j < node.output.length; j++) {
+              tensorsForBackends[operatorOutputs[j].backend].set(node.output[j], operatorOutputs[j]);
+            }
+            actualBackend = operator.backend;
+            break;
+          } catch (error) {
+            if (firstTry && !strict && !(backendOrderForNode.length === 1 && backendOrderForNode[0] === "cpu")) {
+              logger.warn(`Failed to run ${node.name}. Retrying on cpu.`, error);
+              firstTry = false;
+              backendOrderForNode = ["cpu"];
+              stats.retriedOnCpu.push(node.name);
+              continue;
+            }
+            throw error;
+          }
+        }
+
+        stats.nodesByBackend[actualBackend] = (stats.nodesByBackend[actualBackend] || 0) + 1;
+        for (const name of tensorReleaseTiming.get(node.name) || []) {
+          for (const backend of backends) {
+            const t = tensorsForBackends[backend].get(name);
+            if (t) {
+              t.dispose();
+              tensorsForBackends[backend].delete(name);
+            }
+          }
+        }
+        nodePerformances.push({
+          opType: node.opType,
+          name: node.name,
+          backend: actualBackend,
+          inputDims: actualInputDims,
+          outputDims: actualOutputDims,
+          elapsed: Date.now() - nodeStartTime,
+        });
+      }
+
+      const outputs = [];
+      for (const outputInfo of graph.output) {
+        let outputTensor = tensorsForBackends.cpu.get(outputInfo.name);
+        if (!outputTensor) {
+          for (const otherBackend of this.backendOrder) {
+            const otherT = tensorsForBackends[otherBackend].get(outputInfo.name);
+            if (otherT) {
+              // device -> host: the only point where the run waits for the GPU
+              outputTensor = await this.backendContexts.cpu.moveTensor(otherT, {});
+              tensorsForBackends.cpu.set(outputInfo.name, outputTensor);
+              break;
+            }
+          }
+        }
+        if (!outputTensor) throw new Error(`Output ${outputInfo.name} not found`);
+        outputs.push(outputTensor);
+      }
+
+      if (opts.measurePerformance) {
+        if (useEvents) {
+          for (let i = 0; i < nodePerformances.length; i++) {
+            if (nodePerformances[i].backend === "hip") {
+              nodePerformances[i].deviceElapsed = hip.native.eventElapsedMs(2 * i, 2 * i + 1);
+            }
+          }
+        }
+        this.lastPerformance = nodePerformances;
+        logger.debug("Performance", nodePerformances);
+      }
+      this.lastRunStats = stats;
+      return outputs;
+    } finally {
+      // device copies of initializers stay for the next run; every other device tensor goes
+      for (const backend of backendsWithoutCPU) {
+        for (const [name, t] of tensorsForBackends[backend].entries()) {
+          if (this.initializerTensors.has(name) && this.copiedInitializerTensors.has(backend)) {
+            this.copiedInitializerTensors.get(backend).set(name, t);
+          } else {
+            t.dispose();
+          }
+        }
+      }
+    }
+  }
+}
+
+module.exports = { RunnerImpl };

@@ -1,0 +1,359 @@
+"""Seeded writers for the ONNX graphs of the benchmark configurations.
+
+No `onnx` package is needed: a small protobuf encoder/decoder for the handful of ONNX
+messages the descriptor runner reads (field numbers of the reference's scripts/onnx.proto:
+ModelProto:357-400, GraphProto:456-477, NodeProto:208-224, AttributeProto:122-185,
+TensorProto:499-618).  Weights are random-initialised from numpy's default_rng with a seed
+per tensor, so the same bytes are produced on every machine.
+
+Graphs (the shapes follow example/benchmark/make_models.py:142-162 of the reference and the
+five benchmark configurations):
+    gemm_model      Gemm A[M,K] . B[N,K]^T + C[N]
+    ffn_model       MatMul -> Add -> Relu -> MatMul -> Add(residual)
+    conv_model      Conv 3x3 -> Relu
+    resnet50_model  ResNet-50 v1 with BatchNorm folded into the conv bias
+"""
+import struct
+
+import numpy as np
+
+FLOAT, INT32, INT64 = 1, 6, 7
+ATTR_FLOAT, ATTR_INT, ATTR_STRING, ATTR_TENSOR, ATTR_FLOATS, ATTR_INTS = 1, 2, 3, 4, 6, 7
+
+
+# ------------------------------------------------------------------ protobuf wire format
+def _varint(v):
+    if v < 0:
+        v += 1 << 64
+    out = bytearray()
+    while v > 0x7F:
+        out.append((v & 0x7F) | 0x80)
+        v >>= 7
+    out.append(v)
+    return bytes(out)
+
+
+def _tag(field, wire):
+    return _varint(field << 3 | wire)
+
+
+def _len(field, payload):
+    return _tag(field, 2) + _varint(len(payload)) + payload
+
+
+def _int(field, v):
+    return _tag(field, 0) + _varint(int(v))
+
+
+def _str(field, s):
+    return _len(field, s.encode("utf-8"))
+
+
+def _packed_ints(field, values):
+    return _len(field, b"".join(_varint(int(v)) for v in values)) if len(values) else b""
+
+
+def tensor_proto(name, array):
+    array = np.asarray(array)
+    if array.dtype == np.float32:
+        dt = FLOAT
+    elif array.dtype == np.int64:
+        dt = INT64
+    elif array.dtype == np.int32:
+        dt = INT32
+    else:
+        raise TypeError("unsupported initializer dtype %s" % array.dtype)
+    return (_packed_ints(1, array.shape) + _int(2, dt) + _str(8, name)
+            + _len(9, np.ascontiguousarray(array).tobytes()))
+
+
+def attribute(name, value):
+    out = _str(1, name)
+    if isinstance(value, float):
+        return out + _tag(2, 5) + struct.pack("<f", value) + _int(20, ATTR_FLOAT)
+    if isinstance(value, (int, np.integer)):
+        return out + _int(3, value) + _int(20, ATTR_INT)
+    if isinstance(value, str):
+        return out + _len(4, value.encode("utf-8")) + _int(20, ATTR_STRING)
+    if isinstance(value, (list, tuple)):
+        return out + _packed_ints(8, value) + _int(20, ATTR_INTS)
+    raise TypeError("unsupported attribute %r" % (value,))
+
+
+def node(op_type, inputs, outputs, name, **attrs):
+    out = b"".join(_str(1, i) for i in inputs) + b"".join(_str(2, o) for o in outputs)
+    out += _str(3, name) + _str(4, op_type)
+    out += b"".join(_len(5, attribute(k, v)) for k, v in attrs.items())
+    return out
+
+
+def value_info(name, shape, elem_type=FLOAT):
+    dims = b"".join(_len(1, _int(1, d)) for d in shape)
+    tensor_type = _int(1, elem_type) + _len(2, dims)
+    return _str(1, name) + _len(2, _len(1, tensor_type))
+
+
+def model_proto(nodes, initializers, inputs, outputs, opset=13, graph_name="graph", metadata=None):
+    graph = b"".join(_len(1, n) for n in nodes) + _str(2, graph_name)
+    graph += b"".join(_len(5, t) for t in initializers)
+    graph += b"".join(_len(11, v) for v in inputs) + b"".join(_len(12, v) for v in outputs)
+    out = _int(1, 7) + _str(2, "webdnn_amd.modelgen") + _len(7, graph)
+    out += _len(8, _str(1, "") + _int(2, opset))
+    for key, value in (metadata or {}).items():
+        out += _len(14, _str(1, key) + _str(2, value))
+    return out
+
+
+# ------------------------------------------------------------------ reader (for the Python graph checker)
+def _read_varint(buf, pos):
+    result, shift = 0, 0
+    while True:
+        b = buf[pos]
+        pos += 1
+        result |= (b & 0x7F) << shift
+        if not b & 0x80:
+            return result, pos
+        shift += 7
+
+
+def _fields(buf):
+    pos, end = 0, len(buf)
+    while pos < end:
+        key, pos = _read_varint(buf, pos)
+        field, wire = key >> 3, key & 7
+        if wire == 0:
+            v, pos = _read_varint(buf, pos)
+        elif wire == 2:
+            n, pos = _read_varint(buf, pos)
+            v = buf[pos:pos + n]
+            pos += n
+        elif wire == 5:
+            v = buf[pos:pos + 4]
+            pos += 4
+        elif wire == 1:
+            v = buf[pos:pos + 8]
+            pos += 8
+        else:
+            raise ValueError("wire type %d" % wire)
+        yield field, wire, v
+
+
+def _signed(v):
+    return v - (1 << 64) if v >= 1 << 63 else v
+
+
+def _ints(wire, v):
+    if wire == 0:
+        return [_signed(v)]
+    out, pos = [], 0
+    while pos < len(v):
+        x, pos = _read_varint(v, pos)
+        out.append(_signed(x))
+    return out
+
+
+def parse_model(data):
+    """-> dict(opset, nodes=[dict(op_type, name, inputs, outputs, attrs)], initializers={name: array},
+    inputs=[(name, shape)], outputs=[(name, shape)])."""
+    data = memoryview(data)
+    model = {"opset": None, "nodes": [], "initializers": {}, "inputs": [], "outputs": [], "metadata": {}}
+
+    def parse_tensor(buf):
+        dims, dt, name, raw = [], None, "", b""
+        for f, w, v in _fields(buf):
+            if f == 1:
+                dims += _ints(w, v)
+            elif f == 2:
+                dt = v
+            elif f == 8:
+                name = bytes(v).decode()
+            elif f == 9:
+                raw = bytes(v)
+        np_dt = {FLOAT: np.float32, INT64: np.int64, INT32: np.int32}[dt]
+        return name, np.frombuffer(raw, dtype=np_dt).reshape(dims).copy()
+
+    def parse_attr(buf):
+        name, value = "", None
+        for f, w, v in _fields(buf):
+            if f == 1:
+                name = bytes(v).decode()
+            elif f == 2:
+                value = struct.unpack("<f", bytes(v))[0]
+            elif f == 3:
+                value = _signed(v)
+            elif f == 4:
+                value = bytes(v).decode()
+            elif f == 8:
+                value = (value or []) + _ints(w, v)
+        return name, value
+
+    def parse_node(buf):
+        n = {"op_type": "", "name": "", "inputs": [], "outputs": [], "attrs": {}}
+        for f, w, v in _fields(buf):
+            if f == 1:
+                n["inputs"].append(bytes(v).decode())
+            elif f == 2:
+                n["outputs"].append(bytes(v).decode())
+            elif f == 3:
+                n["name"] = bytes(v).decode()
+            elif f == 4:
+                n["op_type"] = bytes(v).decode()
+            elif f == 5:
+                k, val = parse_attr(v)
+                n["attrs"][k] = val
+        return n
+
+    def parse_value_info(buf):
+        name, shape = "", []
+        for f, w, v in _fields(buf):
+            if f == 1:
+                name = bytes(v).decode()
+            elif f == 2:
+                for f2, _, v2 in _fields(v):            # TypeProto.tensor_type
+                    if f2 == 1:
+                        for f3, _, v3 in _fields(v2):    # Tensor: elem_type, shape
+                            if f3 == 2:
+                                for f4, _, v4 in _fields(v3):      # dim
+                                    for f5, _, v5 in _fields(v4):  # dim_value
+                                        if f5 == 1:
+                                            shape.append(v5)
+        return name, shape
+
+    for f, w, v in _fields(data):
+        if f == 7:
+            for gf, gw, gv in _fields(v):
+                if gf == 1:
+                    model["nodes"].append(parse_node(gv))
+                elif gf == 5:
+                    name, arr = parse_tensor(gv)
+                    model["initializers"][name] = arr
+                elif gf == 11:
+                    model["inputs"].append(parse_value_info(gv))
+                elif gf == 12:
+                    model["outputs"].append(parse_value_info(gv))
+        elif f == 8 and model["opset"] is None:
+            for of, ow, ov in _fields(v):
+                if of == 2:
+                    model["opset"] = ov
+        elif f == 14:
+            kv = {}
+            for mf, mw, mv in _fields(v):
+                kv[mf] = bytes(mv).decode()
+            model["metadata"][kv.get(1, "")] = kv.get(2, "")
+    model["inputs"] = [(n, s) for n, s in model["inputs"] if n not in model["initializers"]]
+    return model
+
+
+# ------------------------------------------------------------------ graph builders
+class GraphBuilder:
+    def __init__(self, seed=0):
+        self.nodes, self.initializers, self.counter = [], [], 0
+        self.seed = seed
+        self.flops = 0          # 2*M*N*K of every Gemm / MatMul / Conv
+        self.conv_gemm_nodes = 0
+
+    def rng(self):
+        self.counter += 1
+        return np.random.default_rng([self.seed, self.counter])
+
+    def const(self, name, array):
+        self.initializers.append(tensor_proto(name, array))
+        return name
+
+    def op(self, op_type, inputs, output, **attrs):
+        self.nodes.append(node(op_type, inputs, [output], "%s_%d" % (op_type, len(self.nodes)), **attrs))
+        return output
+
+    def finish(self, inputs, outputs, opset=13):
+        return model_proto(self.nodes, self.initializers, [value_info(n, s) for n, s in inputs],
+                           [value_info(n, s) for n, s in outputs], opset)
+
+
+def gemm_model(m=256, k=512, n=1024, seed=0):
+    """Config 1: A[m,k] (input), B[n,k] transB=1, C[n]; uniform[-1,1]."""
+    g = GraphBuilder(seed)
+    g.const("B", g.rng().uniform(-1, 1, (n, k)).astype(np.float32))
+    g.const("C", g.rng().uniform(-1, 1, (n,)).astype(np.float32))
+    g.op("Gemm", ["A", "B", "C"], "Y", alpha=1.0, beta=1.0, transB=1)
+    g.flops = 2 * m * n * k
+    return g.finish([("A", [m, k])], [("Y", [m, n])]), g
+
+
+def ffn_model(batch=8, seq=512, d=768, hidden=3072, seed=0):
+    """Config 2: X -> MatMul W1 -> Add b1 -> Relu -> MatMul W2 -> Add X."""
+    g = GraphBuilder(seed)
+    g.const("W1", (g.rng().standard_normal((d, hidden)) * 0.02).astype(np.float32))
+    g.const("b1", np.zeros(hidden, np.float32))
+    g.const("W2", (g.rng().standard_normal((hidden, d)) * 0.02).astype(np.float32))
+    g.op("MatMul", ["X", "W1"], "h")
+    g.op("Add", ["h", "b1"], "hb")
+    g.op("Relu", ["hb"], "hr")
+    g.op("MatMul", ["hr", "W2"], "y")
+    g.op("Add", ["y", "X"], "out")
+    g.flops = 2 * 2 * batch * seq * d * hidden
+    return g.finish([("X", [batch, seq, d])], [("out", [batch, seq, d])]), g
+
+
+def conv_model(batch=32, cin=64, hw=56, cout=64, k=3, seed=0):
+    """Config 3: Conv 3x3 pad 1 (He-normal weights, zero bias) -> Relu."""
+    g = GraphBuilder(seed)
+    g.const("W", (g.rng().standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / (cin * k * k))).astype(np.float32))
+    g.const("B", np.zeros(cout, np.float32))
+    p = k // 2
+    g.op("Conv", ["X", "W", "B"], "c", kernel_shape=[k, k], pads=[p, p, p, p], strides=[1, 1], dilations=[1, 1], group=1)
+    g.op("Relu", ["c"], "Y")
+    g.flops = 2 * batch * hw * hw * cout * cin * k * k
+    return g.finish([("X", [batch, cin, hw, hw])], [("Y", [batch, cout, hw, hw])]), g
+
+
+def resnet50_model(batch=32, image=224, classes=1000, seed=0, width=64, blocks=(3, 4, 6, 3)):
+    """Config 4: ResNet-50 v1 (stride on the first 1x1 of a stage's first block, as in the original
+    architecture), He-normal conv weights, BatchNorm folded into the conv bias with gamma=1, beta=0,
+    mean=0, var=1 and eps dropped (scale exactly 1, bias exactly 0), FC weights N(0, 0.01).
+    Nodes: Conv, Relu, Add, MaxPool, GlobalAveragePool, Flatten, Gemm."""
+    g = GraphBuilder(seed)
+    size = {"hw": image}
+
+    def conv(x, cin, cout, k, stride, pad, relu, name):
+        w = (g.rng().standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / (cin * k * k))).astype(np.float32)
+        g.const(name + "_w", w)
+        g.const(name + "_b", np.zeros(cout, np.float32))
+        out_hw = (size["hw"] + 2 * pad - k) // stride + 1
+        g.flops += 2 * batch * out_hw * out_hw * cout * cin * k * k
+        g.conv_gemm_nodes += 1
+        y = g.op("Conv", [x, name + "_w", name + "_b"], name, kernel_shape=[k, k], pads=[pad] * 4,
+                 strides=[stride, stride], dilations=[1, 1], group=1)
+        size["hw"] = out_hw
+        return g.op("Relu", [y], name + "_relu") if relu else y
+
+    x = conv("input", 3, width, 7, 2, 3, True, "stem")
+    x = g.op("MaxPool", [x], "pool", kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
+    size["hw"] = (size["hw"] + 2 - 3) // 2 + 1
+    cin = width
+    for stage, nblocks in enumerate(blocks):
+        mid, cout = width * 2 ** stage, width * 4 * 2 ** stage
+        for b in range(nblocks):
+            stride = 2 if (stage > 0 and b == 0) else 1
+            name = "s%db%d" % (stage + 1, b)
+            hw_in = size["hw"]
+            y = conv(x, cin, mid, 1, stride, 0, True, name + "_c1")
+            y = conv(y, mid, mid, 3, 1, 1, True, name + "_c2")
+            y = conv(y, mid, cout, 1, 1, 0, False, name + "_c3")
+            hw_out = size["hw"]
+            if b == 0:
+                size["hw"] = hw_in
+                shortcut = conv(x, cin, cout, 1, stride, 0, False, name + "_ds")
+                size["hw"] = hw_out
+            else:
+                shortcut = x
+            s = g.op("Add", [y, shortcut], name + "_add")
+            x = g.op("Relu", [s], name + "_out")
+            cin = cout
+    x = g.op("GlobalAveragePool", [x], "gap")
+    x = g.op("Flatten", [x], "flat", axis=1)
+    g.const("fc_w", (g.rng().standard_normal((classes, cin)) * 0.01).astype(np.float32))
+    g.const("fc_b", np.zeros(classes, np.float32))
+    g.op("Gemm", [x, "fc_w", "fc_b"], "logits", alpha=1.0, beta=1.0, transB=1)
+    g.flops += 2 * batch * classes * cin
+    g.conv_gemm_nodes += 1
+    return g.finish([("input", [batch, 3, image, image])], [("logits", [batch, classes])]), g
