@@ -1,16 +1,28 @@
 """Benchmark of the hip backend hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-Prints one JSON line.  A step is one pass of the workload over synthetic, seeded inputs that are
-already resident in HBM when the timed region starts.  `roofline` is measured live with HIP events
-on the library's own stream around the same launches; `cpu_baseline` times the CPU oracle (a
-restatement of the reference's CPU operators) on one host core over a bounded sample.
+Prints one JSON line.
+
+Workload of `value` (BASELINE config 4): ResNet-50 v1, batch 32, fp32, random-initialised weights
+(seeded), BatchNorm folded, run through the Node.js descriptor runner on the `hip` backend
+(WebDNN.load + runner.run) in strict mode — no CPU fallback.  A step is one runner.run() over one
+batch whose input tensor is already resident in HBM; the step ends when the logits are back on the
+host (the run's only synchronisation).  `value` = 32 * steps / total time.
+
+`roofline` is for the dominant kernel of that workload, the implicit-GEMM contraction kernel: its
+algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over its device time,
+measured with HIP events recorded on the library's stream around every node of one run.
+`extra` carries the two single-kernel figures the metric names: Gemm 4096^3 and the config-3 Conv.
+`cpu_baseline` times the JavaScript restatement of the reference's CPU operators (oracle/js) through
+the same runner with backendOrder ["cpu"] in Node.js on one host core, on ONE image of the batch.
 """
 import argparse
 import json
 import os
+import subprocess
 import sys
+import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -21,64 +33,109 @@ import numpy as np  # noqa: E402
 
 METRIC = "fp32 Gemm/Conv GFLOP/s (% MFMA peak) + ResNet-50 b32 images/sec, 1 MI355X"
 PEAK_FP32_MFMA_TFLOPS = 157.3
-PEAK_HBM_GBS = 8000.0
+CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
+ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
+
+
+def node_run(model_dir, input_path, backend, runs, warmup, extra):
+    cmd = ["node", CLI, "--model", model_dir, "--backend", backend, "--inputs", input_path,
+           "--runs", str(runs), "--warmup", str(warmup)] + extra
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("node runner failed: %s" % proc.stderr[-2000:])
+    return json.loads(proc.stdout.strip().splitlines()[-1])
+
+
+def bench_resnet(steps, warmup, workdir):
+    from webdnn_amd import modelgen
+
+    batch = 32
+    data, g = modelgen.resnet50_model(batch=batch)
+    with open(os.path.join(workdir, "model.onnx"), "wb") as f:
+        f.write(data)
+    x = np.random.default_rng(6).standard_normal((batch, 3, 224, 224)).astype(np.float32)
+    inp = os.path.join(workdir, "input.bin")
+    x.tofile(inp)
+    timed = node_run(workdir, inp, "hip", steps, warmup, ["--strict", "--resident-inputs"])
+    assert timed["backend"] == "hip" and list(timed["stats"]["nodesByBackend"]) == ["hip"], timed["stats"]
+    total_ms = sum(timed["msPerRun"])
+    # one more run with per-node HIP events for the kernel-level figure
+    prof = node_run(workdir, inp, "hip", 1, 2, ["--strict", "--resident-inputs", "--measure"])
+    contraction_ms = sum(p["deviceElapsed"] for p in prof["performance"]
+                         if p["opType"] in ("Conv", "WebDNNHipFusedConv", "Gemm"))
+    launches = sum(1 for p in prof["performance"] if p["opType"] in ("Conv", "WebDNNHipFusedConv", "Gemm"))
+    all_ms = sum(p["deviceElapsed"] or 0.0 for p in prof["performance"])
+    # PCIe-inclusive: the input is a host tensor, uploaded by the run
+    host_in = node_run(workdir, inp, "hip", max(3, steps // 4), 2, ["--strict"])
+    return {
+        "batch": batch, "flops": g.flops, "nodes": timed["nodes"], "ms_per_step": total_ms / steps,
+        "images_per_s": batch * steps / total_ms * 1e3, "contraction_ms": contraction_ms,
+        "contraction_launches": launches, "device_ms": all_ms,
+        "images_per_s_host_input": batch / (sum(host_in["msPerRun"]) / len(host_in["msPerRun"])) * 1e3,
+        "device": timed.get("device"), "node_version": timed["node"],
+    }
+
+
+def cpu_baseline_resnet(workdir):
+    """ResNet-50 on one image through the runner's cpu path with the JS oracle operators."""
+    from webdnn_amd import modelgen
+
+    d = os.path.join(workdir, "cpu1")
+    os.makedirs(d, exist_ok=True)
+    data, g = modelgen.resnet50_model(batch=1)
+    with open(os.path.join(d, "model.onnx"), "wb") as f:
+        f.write(data)
+    x = np.random.default_rng(6).standard_normal((1, 3, 224, 224)).astype(np.float32)
+    inp = os.path.join(d, "input.bin")
+    x.tofile(inp)
+    rep = node_run(d, inp, "cpu", 1, 0, ["--cpu-entries", ORACLE_JS])
+    sec = rep["msPerRun"][0] / 1e3
+    return {"value": round(1.0 / sec, 4), "unit": "images/s", "cores": 1, "kind": "port",
+            "sample": "1 image of the 32 (ResNet-50, %.1f GFLOP) through runner.run with backendOrder [\"cpu\"] "
+                      "and the JavaScript restatement of the reference CPU operators, Node %s, %.1f s"
+                      % (g.flops / 1e9, rep["node"], sec),
+            "gflops": round(g.flops / sec / 1e9, 3)}
 
 
 def timed_steps(ctx, step, steps, warmup):
-    """Wall clock over exactly `steps` calls bracketed by stream syncs, plus the HIP-event time of
-    the same region on the library's stream."""
     for _ in range(warmup):
         step()
     ctx.sync()
-    t0 = time.perf_counter()
     ctx.event_record(0)
     for _ in range(steps):
         step()
     ctx.event_record(1)
     ctx.sync()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    dev_ms = ctx.event_elapsed_ms(0, 1) / steps
-    return wall_ms, dev_ms
+    return ctx.event_elapsed_ms(0, 1) / steps
 
 
-def bench_gemm(ctx, H, n, steps, warmup, rng):
+def bench_kernels(steps, warmup):
+    """The two single-kernel figures the metric names, through the C ABI (ctypes)."""
+    from webdnn_amd import hostops as H
+
+    ctx = H.HipContext(0).initialize()
+    rng = np.random.default_rng(0)
+    n = 4096
     A = ctx.move_tensor(rng.uniform(-1, 1, (n, n)).astype(np.float32))
     B = ctx.move_tensor(rng.uniform(-1, 1, (n, n)).astype(np.float32))
     C = ctx.move_tensor(rng.uniform(-1, 1, (n,)).astype(np.float32))
-
-    def step():
-        H.gemm(ctx, A, B, C).dispose()
-
-    wall_ms, dev_ms = timed_steps(ctx, step, steps, warmup)
-    flops = 2.0 * n * n * n
-    return {"wall_ms": wall_ms, "dev_ms": dev_ms, "flops": flops, "gflops": flops / dev_ms / 1e6}
-
-
-def bench_conv3(ctx, H, steps, warmup, rng):
+    gemm_ms = timed_steps(ctx, lambda: H.gemm(ctx, A, B, C).dispose(), steps, warmup)
     X = ctx.move_tensor(rng.uniform(0, 1, (32, 64, 56, 56)).astype(np.float32))
     W = ctx.move_tensor((rng.standard_normal((64, 64, 3, 3)) * np.sqrt(2 / 576)).astype(np.float32))
     Bv = ctx.move_tensor(np.zeros(64, np.float32))
+    conv_ms = timed_steps(ctx, lambda: H.conv(ctx, X, W, Bv, pads=[1, 1, 1, 1], epilogue="relu").dispose(),
+                          steps, warmup)
+    gemm_flops, conv_flops = 2.0 * n ** 3, 2.0 * 100352 * 64 * 576
 
-    def step():
-        H.conv(ctx, X, W, Bv, pads=[1, 1, 1, 1], epilogue="relu").dispose()
+    def entry(workload, flops, ms):
+        tf = flops / ms / 1e9
+        return {"workload": workload, "ms": round(ms, 4), "gflops": round(tf * 1e3, 1),
+                "frac_mfma_peak": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)}
 
-    wall_ms, dev_ms = timed_steps(ctx, step, steps, warmup)
-    flops = 2.0 * 100352 * 64 * 576
-    return {"wall_ms": wall_ms, "dev_ms": dev_ms, "flops": flops, "gflops": flops / dev_ms / 1e6}
-
-
-def cpu_baseline_gemm(n, rows, rng):
-    """The oracle's Gemm (double accumulation, one thread) on `rows` rows of the n x n problem."""
-    from oracle import ref
-
-    ref.set_threads(1)
-    A = rng.uniform(-1, 1, (rows, n)).astype(np.float32)
-    B = rng.uniform(-1, 1, (n, n)).astype(np.float32)
-    C = rng.uniform(-1, 1, (n,)).astype(np.float32)
-    t0 = time.perf_counter()
-    ref.gemm(A, B, C)
-    dt = time.perf_counter() - t0
-    return 2.0 * rows * n * n / dt / 1e9, dt
+    return {
+        "gemm_4096": entry("Gemm M=N=K=4096 + bias[4096], alpha=beta=1, U[-1,1] (north_star NS-4096)", gemm_flops, gemm_ms),
+        "conv_c3": entry("Conv 3x3 X[32,64,56,56] W[64,64,3,3] pad 1 + bias + Relu fused (config 3)", conv_flops, conv_ms),
+    }
 
 
 def main():
@@ -92,56 +149,50 @@ def main():
         sys.exit("bench.py: this build runs on exactly one GPU (the path shards by batch with no "
                  "exchange; multi-GPU runs are not part of it). Use --gpus 1.")
 
-    from webdnn_amd import hostops as H
+    with tempfile.TemporaryDirectory(prefix="webdnn_bench_") as workdir:
+        resnet = bench_resnet(args.steps, args.warmup, workdir)
+        baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
+    kernels = bench_kernels(args.steps, args.warmup)
 
-    ctx = H.HipContext(0).initialize()
-    rng = np.random.default_rng(0)
-    n = 4096
-    gemm = bench_gemm(ctx, H, n, args.steps, args.warmup, rng)
-    conv = bench_conv3(ctx, H, args.steps, args.warmup, rng)
-
+    achieved = resnet["flops"] / resnet["contraction_ms"] / 1e9
     line = {
         "metric": METRIC,
-        "value": round(gemm["flops"] / gemm["wall_ms"] / 1e6, 1),
-        "unit": "GFLOP/s",
+        "value": round(resnet["images_per_s"], 1),
+        "unit": "images/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(gemm["wall_ms"], 4),
+        "ms_per_step": round(resnet["ms_per_step"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "Gemm M=N=K=4096, A,B U[-1,1] seed 0, C[4096] bias, alpha=beta=1 (north_star NS-4096)"},
+        "config": {"workload": "ResNet-50 v1 batch 32 [32,3,224,224] fp32, random init (seeded), BN folded, "
+                               "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict "
+                               "(BASELINE config 4)" % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
-            "kernel": "contraction_kernel<A k-contiguous, B n-contiguous, 16-byte loads>",
-            "achieved": round(gemm["gflops"] / 1e3, 2),
+            "kernel": "contraction_kernel (implicit-GEMM Conv + Gemm head), %d launches per step"
+                      % resnet["contraction_launches"],
+            "achieved": round(achieved, 2),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(gemm["gflops"] / 1e3 / PEAK_FP32_MFMA_TFLOPS, 4),
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "traffic": None,
+            "flops_per_step": resnet["flops"],
+            "avg_launch_ms": round(resnet["contraction_ms"] / resnet["contraction_launches"], 5),
         },
         "extra": {
-            "conv_c3": {
-                "workload": "Conv 3x3 X[32,64,56,56] W[64,64,3,3] pad 1 + bias + Relu fused (config 3)",
-                "gflops": round(conv["gflops"], 1),
-                "ms": round(conv["dev_ms"], 4),
-                "frac_mfma_peak": round(conv["gflops"] / 1e3 / PEAK_FP32_MFMA_TFLOPS, 4),
-            },
+            "gemm_4096": kernels["gemm_4096"],
+            "conv_c3": kernels["conv_c3"],
+            "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
+            "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),
+            "device": resnet["device"],
         },
     }
-    if not args.no_cpu_baseline:
-        rows = 128
-        gf, dt = cpu_baseline_gemm(n, rows, rng)
-        line["cpu_baseline"] = {
-            "value": round(gf, 3),
-            "unit": "GFLOP/s",
-            "cores": 1,
-            "kind": "port",
-            "sample": "oracle Gemm on %d of the %d rows of A against the full B (%.1f s)" % (rows, n, dt),
-        }
+    if baseline is not None:
+        line["cpu_baseline"] = baseline
     print(json.dumps(line))
 
 

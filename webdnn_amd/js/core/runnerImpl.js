@@ -129,8 +129,15 @@ class RunnerImpl {
     }
 
     if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
+    // Inputs are CPU tensors in the reference; a tensor that already lives on another
+    // backend (uploaded once by the caller, e.g. through context.moveTensor) is taken
+    // where it is.  Caller-owned tensors are never disposed by the run.
+    const callerOwned = new Set();
     for (let i = 0; i < inputs.length; i++) {
-      tensorsForBackends.cpu.set(this.inputsWithoutInitializer[i].name, inputs[i]);
+      const name = this.inputsWithoutInitializer[i].name;
+      if (!(inputs[i].backend in tensorsForBackends)) throw new Error(`input ${name}: unknown backend ${inputs[i].backend}`);
+      tensorsForBackends[inputs[i].backend].set(name, inputs[i]);
+      callerOwned.add(inputs[i]);
     }
 
     const tensorReleaseTiming = findTensorReleaseTiming(this.model, new Set(this.initializerTensors.keys()));
@@ -288,7 +295,7 @@ class RunnerImpl {
         for (const [name, t] of tensorsForBackends[backend].entries()) {
           if (this.initializerTensors.has(name) && this.copiedInitializerTensors.has(backend)) {
             this.copiedInitializerTensors.get(backend).set(name, t);
-          } else {
+          } else if (!callerOwned.has(t)) {
             t.dispose();
           }
         }
