@@ -1,0 +1,257 @@
+"use strict";
+/*
+ * TEST INFRASTRUCTURE — a JavaScript stand-in for the N-API addon (webdnn_hip.node) so
+ * that the host side of the hip backend (contexts, tensors, operators, fusion, runner)
+ * can be exercised on a machine without a GPU.  It implements the entry points of
+ * include/webdnn_hip.h over typed arrays, accumulating in double and rounding where the
+ * reference CPU operators round, so a graph run on "hip" through this module must equal
+ * the same graph on the cpu path bit for bit.  Never loaded by the product.
+ */
+const buffers = new Map();
+let nextHandle = 1;
+let inUse = 0, peak = 0;
+const calls = {};
+const options = {};
+
+function count(name) {
+  calls[name] = (calls[name] || 0) + 1;
+}
+function buf(h, what) {
+  const b = buffers.get(h);
+  if (!b) throw new Error(`${what}: unknown buffer handle ${h}`);
+  return b;
+}
+const f32 = (h, what) => new Float32Array(buf(h, what).buffer);
+const i32 = (h, what) => new Int32Array(buf(h, what).buffer);
+function need(h, bytes, what) {
+  if (buf(h, what).byteLength < bytes) throw new Error(`${what}: buffer holds ${buf(h, what).byteLength} bytes, operation needs ${bytes}`);
+}
+function reluJs(v) {
+  return Math.max(v, 0);
+}
+function toInt32(d) {
+  return d | 0; // ToInt32, like a store into an Int32Array
+}
+
+const native = {
+  init(device) {
+    count("init");
+    if (device !== 0) throw new Error("wdh_init failed (-1): device out of range");
+  },
+  shutdown() {},
+  deviceInfo() {
+    return { name: "fake-gfx950", computeUnits: 256, clockMHz: 2400, hbmBytes: 1 << 30 };
+  },
+  setOption(name, value) {
+    if (name !== "contraction_tile" && name !== "split_k") throw new Error(`wdh_set_option failed (-2): unknown option "${name}"`);
+    options[name] = value;
+  },
+  alloc(bytes) {
+    count("alloc");
+    const h = nextHandle++;
+    buffers.set(h, new Uint8Array(Math.max(bytes, 0)));
+    inUse += bytes;
+    if (inUse > peak) peak = inUse;
+    return h;
+  },
+  free(h) {
+    count("free");
+    inUse -= buf(h, "wdh_free").byteLength;
+    buffers.delete(h);
+  },
+  write(h, off, data) {
+    count("write");
+    const src = new Uint8Array(data.buffer, data.byteOffset, data.byteLength);
+    if (off + src.length > buf(h, "wdh_write").byteLength) throw new Error("wdh_write failed (-2): exceeds buffer");
+    buf(h).set(src, off);
+  },
+  read(h, off, data) {
+    count("read");
+    const dst = new Uint8Array(data.buffer, data.byteOffset, data.byteLength);
+    if (off + dst.length > buf(h, "wdh_read").byteLength) throw new Error("wdh_read failed (-2): exceeds buffer");
+    dst.set(buf(h).subarray(off, off + dst.length));
+  },
+  copy(dst, doff, src, soff, bytes) {
+    buf(dst).set(buf(src).subarray(soff, soff + bytes), doff);
+  },
+  sync() {},
+  memStats() {
+    return { inUse, cached: 0, peak };
+  },
+  trim() {},
+  eventRecord() {},
+  eventElapsedMs() {
+    return 0;
+  },
+
+  gemm(A, B, C, Y, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1, alpha, beta, epi, R) {
+    count("gemm");
+    need(Y, batch * m * n * 4, "wdh_gemm: Y");
+    const a = f32(A, "A"), b = f32(B, "B"), y = f32(Y, "Y");
+    const c = C ? f32(C, "C") : null, r = R ? f32(R, "R") : null;
+    const out = new Float32Array(1);
+    for (let z = 0; z < batch; z++) for (let i = 0; i < m; i++) for (let j = 0; j < n; j++) {
+      let sum = 0;
+      for (let x = 0; x < k; x++) sum += a[z * sAb + i * sA0 + x * sA1] * b[z * sBb + x * sB0 + j * sB1];
+      out[0] = sum * alpha;
+      if (c) out[0] += c[i * sC0 + j * sC1] * beta;
+      const off = (z * m + i) * n + j;
+      if (r) out[0] += r[off];
+      y[off] = epi === 1 ? reluJs(out[0]) : out[0];
+    }
+  },
+
+  conv2d(X, W, Bias, Y, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epi, R) {
+    count("conv2d");
+    if (c % group || cout % group) throw new Error("wdh_conv2d failed (-2): channels not divisible by group");
+    const oh = Math.floor((h + pt + pb - dh * (kh - 1) - 1) / sh) + 1;
+    const ow = Math.floor((w + pl + pr - dw * (kw - 1) - 1) / sw) + 1;
+    need(Y, n * cout * oh * ow * 4, "wdh_conv2d: Y");
+    const x = f32(X), wt = f32(W), y = f32(Y), bias = Bias ? f32(Bias) : null, r = R ? f32(R) : null;
+    const cg = c / group, og = cout / group, out = new Float32Array(1);
+    for (let b = 0; b < n; b++) for (let co = 0; co < cout; co++) {
+      const g = Math.floor(co / og);
+      for (let oy = 0; oy < oh; oy++) for (let ox = 0; ox < ow; ox++) {
+        let s = 0;
+        for (let ci = 0; ci < cg; ci++) for (let ky = 0; ky < kh; ky++) for (let kx = 0; kx < kw; kx++) {
+          const iy = oy * sh - pt + ky * dh, ix = ox * sw - pl + kx * dw;
+          const v = iy >= 0 && iy < h && ix >= 0 && ix < w ? x[((b * c + g * cg + ci) * h + iy) * w + ix] : 0;
+          s += v * wt[((co * cg + ci) * kh + ky) * kw + kx];
+        }
+        out[0] = s;
+        if (bias) out[0] += bias[co];
+        const off = ((b * cout + co) * oh + oy) * ow + ox;
+        if (r) out[0] += r[off];
+        y[off] = epi === 1 ? reluJs(out[0]) : out[0];
+      }
+    }
+  },
+
+  binary(op, dtype, L, R, Y, shape, sl, sr) {
+    count("binary");
+    const total = shape.reduce((a, b) => a * b, 1);
+    need(Y, total * 4, "wdh_binary: Y");
+    const view = dtype === 0 ? f32 : i32;
+    const l = view(L), r = view(R), y = view(Y);
+    const fn = [(a, b) => a + b, (a, b) => a - b, (a, b) => a * b, (a, b) => a / b, (a, b) => a ** b][op];
+    if (!fn) throw new Error(`wdh_binary failed (-2): unknown op ${op}`);
+    const nd = shape.length, idx = new Array(nd).fill(0);
+    let ol = 0, or = 0;
+    for (let i = 0; i < total; i++) {
+      y[i] = dtype === 0 ? fn(l[ol], r[or]) : toInt32(fn(l[ol], r[or]));
+      for (let d = nd - 1; d >= 0; d--) {
+        idx[d]++; ol += sl[d]; or += sr[d];
+        if (idx[d] < shape[d]) break;
+        ol -= sl[d] * shape[d]; or -= sr[d] * shape[d]; idx[d] = 0;
+      }
+    }
+  },
+
+  unary(op, dtype, X, Y, length) {
+    count("unary");
+    need(Y, length * 4, "wdh_unary: Y");
+    const view = dtype === 0 ? f32 : i32, x = view(X), y = view(Y);
+    const fn = [reluJs, (v) => (Math.tanh(v / 2) + 1) / 2, Math.sqrt, Math.exp, Math.tanh, Math.abs, (v) => -v, (v) => 1 / v][op];
+    if (!fn) throw new Error(`wdh_unary failed (-2): unknown op ${op}`);
+    for (let i = 0; i < length; i++) y[i] = fn(x[i]);
+  },
+
+  softmax(X, Y, outer, len) {
+    count("softmax");
+    const x = f32(X), y = f32(Y);
+    for (let o = 0; o < outer; o++) {
+      let max = -Infinity;
+      for (let r = 0; r < len; r++) if (x[o * len + r] > max) max = x[o * len + r];
+      let sum = 0;
+      for (let r = 0; r < len; r++) { const e = Math.exp(x[o * len + r] - max); y[o * len + r] = e; sum += e; }
+      for (let r = 0; r < len; r++) y[o * len + r] /= sum;
+    }
+  },
+
+  layernorm(X, G, B, Y, outer, len, eps) {
+    count("layernorm");
+    const x = f32(X), y = f32(Y), g = G ? f32(G) : null, b = B ? f32(B) : null, t = new Float32Array(4);
+    for (let o = 0; o < outer; o++) {
+      let s = 0;
+      for (let r = 0; r < len; r++) s += x[o * len + r];
+      t[0] = s / len; // mean
+      let q = 0;
+      for (let r = 0; r < len; r++) { t[1] = x[o * len + r] - t[0]; t[2] = t[1] * t[1]; q += t[2]; }
+      t[2] = q / len; t[2] = t[2] + Math.fround(eps); t[3] = Math.sqrt(t[2]);
+      for (let r = 0; r < len; r++) {
+        t[1] = x[o * len + r] - t[0]; t[1] = t[1] / t[3];
+        if (g) t[1] = t[1] * g[r];
+        if (b) t[1] = t[1] + b[r];
+        y[o * len + r] = t[1];
+      }
+    }
+  },
+
+  reduceMean(X, Y, outer, len) {
+    count("reduceMean");
+    const x = f32(X), y = f32(Y);
+    for (let o = 0; o < outer; o++) {
+      let s = 0;
+      for (let r = 0; r < len; r++) s += x[o * len + r];
+      y[o] = s / len;
+    }
+  },
+
+  maxpool2d(X, Y, n, c, h, w, oh, ow, kh, kw, pt, pl, sh, sw, dh, dw) {
+    count("maxpool2d");
+    const x = f32(X), y = f32(Y);
+    let idx = 0;
+    for (let p = 0; p < n * c; p++) for (let oy = 0; oy < oh; oy++) for (let ox = 0; ox < ow; ox++) {
+      let mv = -Infinity;
+      for (let ky = 0; ky < kh; ky++) for (let kx = 0; kx < kw; kx++) {
+        const iy = oy * sh - pt + ky * dh, ix = ox * sw - pl + kx * dw;
+        if (iy >= 0 && iy < h && ix >= 0 && ix < w) { const v = x[(p * h + iy) * w + ix]; if (v > mv) mv = v; }
+      }
+      y[idx++] = mv;
+    }
+  },
+
+  globalAvgpool(X, Y, nc, hw) {
+    count("globalAvgpool");
+    native.reduceMean(X, Y, nc, hw);
+  },
+
+  transpose(X, Y, shape, strides) {
+    count("transpose");
+    const x = new Uint32Array(buf(X).buffer), y = new Uint32Array(buf(Y).buffer);
+    const total = shape.reduce((a, b) => a * b, 1), nd = shape.length, idx = new Array(nd).fill(0);
+    let off = 0;
+    for (let i = 0; i < total; i++) {
+      y[i] = x[off];
+      for (let d = nd - 1; d >= 0; d--) {
+        idx[d]++; off += strides[d];
+        if (idx[d] < shape[d]) break;
+        off -= strides[d] * shape[d]; idx[d] = 0;
+      }
+    }
+  },
+
+  gather(D, I, Y, outer, axisLen, inner, nIdx) {
+    count("gather");
+    const d = new Uint32Array(buf(D).buffer), ix = i32(I), y = new Uint32Array(buf(Y).buffer);
+    let p = 0;
+    for (let o = 0; o < outer; o++) for (let j = 0; j < nIdx; j++) {
+      let k = ix[j];
+      if (k < 0) k += axisLen;
+      for (let n = 0; n < inner; n++) y[p++] = d[(o * axisLen + k) * inner + n];
+    }
+  },
+
+  // ---- test introspection ----
+  __liveBuffers() {
+    return buffers.size;
+  },
+  __calls() {
+    return Object.assign({}, calls);
+  },
+  __options() {
+    return Object.assign({}, options);
+  },
+};
+
+module.exports = native;

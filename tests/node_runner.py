@@ -8,10 +8,11 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_ENTRIES = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
+FAKE_NATIVE = os.path.join(ROOT, "tests", "js", "fake_native.js")
 
 
 def run_model(model_dir, inputs, backend, strict=True, fuse=True, oracle_cpu=False, runs=1, warmup=0,
-              measure=False, extra=(), timeout=600):
+              measure=False, extra=(), timeout=600, fake_native=False):
     """inputs: list of numpy arrays in graph-input order.  Returns (outputs, report)."""
     files = []
     for i, a in enumerate(inputs):
@@ -19,6 +20,8 @@ def run_model(model_dir, inputs, backend, strict=True, fuse=True, oracle_cpu=Fal
         np.ascontiguousarray(a).tofile(p)
         files.append(p)
     out_path = os.path.join(model_dir, "output_%s.bin" % backend)
+    if fake_native:
+        extra = list(extra) + ["--native", FAKE_NATIVE]
     cmd = ["node", CLI, "--model", model_dir, "--backend", backend, "--inputs", ",".join(files),
            "--output", out_path, "--runs", str(runs), "--warmup", str(warmup)]
     if strict:

@@ -1,0 +1,145 @@
+"""Host side of the hip backend without a GPU: the real contexts, tensors, operators, fusion pass and
+runner, with the N-API addon replaced by tests/js/fake_native.js (same entry points over typed arrays,
+reference rounding).  Whatever the hip host code gets wrong — a stride, a shape, an argument order, a
+fused chain, a tensor freed too early — shows up as a difference from the cpu path, which must be
+bit-exact here."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import graph_ref
+import node_runner
+from util import assert_bit_exact
+from webdnn_amd import modelgen
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def both_paths(tmp_path, data, feeds, fuse=True, strict=True):
+    (tmp_path / "model.onnx").write_bytes(data)
+    model = modelgen.parse_model(data)
+    ordered = [feeds[n] for n, _ in model["inputs"]]
+    hip, rep = node_runner.run_model(str(tmp_path), ordered, "hip", strict=strict, fuse=fuse, fake_native=True,
+                                     oracle_cpu=not strict, runs=2)
+    cpu, _ = node_runner.run_model(str(tmp_path), ordered, "cpu", oracle_cpu=True)
+    return model, hip, cpu, rep
+
+
+def test_every_config_graph_on_the_hip_host_path(tmp_path):
+    cases = [
+        (modelgen.gemm_model(m=9, k=20, n=13)[0], {"A": (9, 20)}),
+        (modelgen.ffn_model(batch=2, seq=5, d=12, hidden=20)[0], {"X": (2, 5, 12)}),
+        (modelgen.conv_model(batch=2, cin=4, hw=7, cout=6)[0], {"X": (2, 4, 7, 7)}),
+        (modelgen.resnet50_model(batch=1, image=32, classes=7, width=4, blocks=(2, 1, 1, 1))[0], {"input": (1, 3, 32, 32)}),
+    ]
+    rng = np.random.default_rng(0)
+    for i, (data, shapes) in enumerate(cases):
+        d = tmp_path / str(i)
+        d.mkdir()
+        feeds = {k: rng.standard_normal(s).astype(np.float32) for k, s in shapes.items()}
+        for fuse in (True, False):
+            model, hip, cpu, rep = both_paths(d, data, feeds, fuse=fuse)
+            assert list(rep["stats"]["nodesByBackend"]) == ["hip"]
+            for got, want, (name, _) in zip(hip, cpu, model["outputs"]):
+                assert_bit_exact(got, want, "case %d fuse=%s %s" % (i, fuse, name))
+            # nothing but the device copies of the initializers survives a run
+            assert rep["liveBuffers"] == rep["initializerCopies"], rep
+
+
+def test_fusion_rewrites_the_expected_chains(tmp_path):
+    data, _ = modelgen.resnet50_model(batch=1, image=32, classes=7, width=4, blocks=(2, 1, 1, 1))
+    feeds = {"input": np.random.default_rng(1).standard_normal((1, 3, 32, 32)).astype(np.float32)}
+    _, _, _, fused = both_paths(tmp_path, data, feeds, fuse=True)
+    _, _, _, plain = both_paths(tmp_path, data, feeds, fuse=False)
+    n_conv = plain["nativeCalls"]["conv2d"]
+    assert fused["nativeCalls"]["conv2d"] == n_conv
+    assert "binary" not in fused["nativeCalls"] and "unary" not in fused["nativeCalls"]   # all Add/Relu absorbed
+    assert plain["nativeCalls"]["binary"] == 2 * 5 and plain["nativeCalls"]["unary"] == 2 * (1 + 3 * 5)
+    assert fused["nodes"] == plain["nodes"] - 5 - 16
+
+
+def test_a_tensor_with_two_readers_is_not_fused_away(tmp_path):
+    g = modelgen.GraphBuilder(0)
+    g.const("W", g.rng().standard_normal((4, 3, 1, 1)).astype(np.float32))
+    g.op("Conv", ["X", "W"], "c")          # read by Relu AND by the final Add -> must stay a tensor
+    g.op("Relu", ["c"], "r")
+    g.op("Add", ["r", "c"], "Y")
+    data = g.finish([("X", [1, 3, 5, 5])], [("Y", [1, 4, 5, 5])])
+    feeds = {"X": np.random.default_rng(2).standard_normal((1, 3, 5, 5)).astype(np.float32)}
+    model, hip, cpu, rep = both_paths(tmp_path, data, feeds)
+    assert rep["nodes"] == 3
+    assert_bit_exact(hip[0], cpu[0], "shared tensor")
+
+
+def test_broadcasting_add_after_conv_falls_back_to_separate_kernels(tmp_path):
+    g = modelgen.GraphBuilder(0)
+    g.const("W", g.rng().standard_normal((4, 3, 3, 3)).astype(np.float32))
+    g.op("Conv", ["X", "W"], "c", pads=[1, 1, 1, 1])
+    g.op("Add", ["c", "S"], "a")           # S is [1,4,1,1]: not a same-shape residual
+    g.op("Relu", ["a"], "Y")
+    data = g.finish([("X", [2, 3, 5, 5]), ("S", [1, 4, 1, 1])], [("Y", [2, 4, 5, 5])])
+    rng = np.random.default_rng(3)
+    feeds = {"X": rng.standard_normal((2, 3, 5, 5)).astype(np.float32), "S": rng.standard_normal((1, 4, 1, 1)).astype(np.float32)}
+    model, hip, cpu, rep = both_paths(tmp_path, data, feeds)
+    assert rep["nodes"] == 1 and rep["nativeCalls"]["binary"] == 2 and rep["nativeCalls"]["unary"] == 2
+    assert_bit_exact(hip[0], cpu[0], "broadcast residual")
+
+
+def test_layout_ops_alias_and_attention_shapes(tmp_path):
+    """Reshape / Transpose / MatMul / Softmax / LayerNormalization / Gemm as a transformer block uses them."""
+    g = modelgen.GraphBuilder(0)
+    t, d, h = 10, 16, 4
+    g.const("Wq", (g.rng().standard_normal((d, d)) * 0.3).astype(np.float32))
+    g.const("split", np.array([t, h, d // h], np.int64))
+    g.const("merge", np.array([t, d], np.int64))
+    g.const("scale", np.array(0.5, np.float32))
+    g.const("gamma", g.rng().standard_normal(d).astype(np.float32))
+    g.const("beta", g.rng().standard_normal(d).astype(np.float32))
+    g.op("MatMul", ["X", "Wq"], "q")
+    g.op("Reshape", ["q", "split"], "q3")
+    g.op("Transpose", ["q3"], "qh", perm=[1, 0, 2])       # [h, t, d/h]
+    g.op("Transpose", ["q3"], "kt", perm=[1, 2, 0])       # [h, d/h, t]
+    g.op("MatMul", ["qh", "kt"], "scores")
+    g.op("Mul", ["scores", "scale"], "scaled")
+    g.op("Softmax", ["scaled"], "attn", axis=-1)
+    g.op("MatMul", ["attn", "qh"], "ctx")
+    g.op("Transpose", ["ctx"], "ctx_t", perm=[1, 0, 2])
+    g.op("Reshape", ["ctx_t", "merge"], "merged")
+    g.op("Add", ["merged", "X"], "res")
+    g.op("LayerNormalization", ["res", "gamma", "beta"], "Y", axis=-1, epsilon=1e-5)
+    data = g.finish([("X", [t, d])], [("Y", [t, d])], opset=17)
+    feeds = {"X": np.random.default_rng(4).standard_normal((t, d)).astype(np.float32)}
+    (tmp_path / "model.onnx").write_bytes(data)
+    hip, rep = node_runner.run_model(str(tmp_path), [feeds["X"]], "hip", strict=True, fake_native=True)
+    assert list(rep["stats"]["nodesByBackend"]) == ["hip"] and rep["liveBuffers"] == rep["initializerCopies"]
+    want = graph_ref.run_graph(modelgen.parse_model(data), feeds)["Y"]
+    np.testing.assert_allclose(hip[0], want, rtol=0, atol=2e-6)
+
+
+def test_strict_and_retry(tmp_path):
+    g = modelgen.GraphBuilder(0)
+    g.op("Relu", ["X"], "r")
+    g.op("ReduceMean", ["r"], "m", axes=[0], keepdims=1)   # hip: last axis only -> throws
+    g.op("Relu", ["m"], "Y")
+    data = g.finish([("X", [4, 6])], [("Y", [1, 6])])
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(5).standard_normal((4, 6)).astype(np.float32)
+    with pytest.raises(RuntimeError, match="only a reduction over the last axis"):
+        node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fake_native=True, oracle_cpu=True)
+    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=False, fake_native=True, oracle_cpu=True)
+    assert rep["stats"]["retriedOnCpu"] == ["ReduceMean_1"] and rep["stats"]["nodesByBackend"] == {"hip": 2, "cpu": 1}
+    # without a cpu implementation the retry fails too, and the error surfaces
+    with pytest.raises(RuntimeError, match="does not exist"):
+        node_runner.run_model(str(tmp_path), [X], "hip", strict=False, fake_native=True, oracle_cpu=False)
+
+
+def test_unit_level_js(tmp_path):
+    """tests/js/unit.js: registry rules, CPUTensor, ONNX reader, fusion pass, load() fallbacks."""
+    proc = subprocess.run(["node", os.path.join(ROOT, "tests", "js", "unit.js")], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
+    summary = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert summary["failed"] == 0 and summary["passed"] >= 14, summary

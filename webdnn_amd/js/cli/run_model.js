@@ -5,7 +5,7 @@
 //   node run_model.js --model DIR [--onnx model.onnx] [--backend hip|cpu]
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure]
-//        [--resident-inputs] [--cpu-entries module.js]
+//        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
 //
 // Inputs are raw little-endian files (float32, or int32 where the graph input says
 // so) in the order of the graph's non-initializer inputs; outputs are written the same
@@ -43,6 +43,7 @@ function parseArgs(argv) {
     else if (a === "--cpu-entries") args.cpuEntries = next();
     else if (a === "--tile") args.tile = parseInt(next(), 10);
     else if (a === "--resident-inputs") args.residentInputs = true;
+    else if (a === "--native") args.native = next();
     else throw new Error(`unknown argument ${a}`);
   }
   if (!args.model) throw new Error("--model is required");
@@ -54,6 +55,8 @@ async function main() {
   if (args.cpuEntries) registerOperators(require(path.resolve(args.cpuEntries)).getOpEntries());
   const hipOption = { strict: !!args.strict, fuse: !args.noFuse };
   if (args.tile != null) hipOption.contractionTile = args.tile;
+  // --native: another implementation of the addon's interface (host tests without a GPU)
+  if (args.native) hipOption.native = require(path.resolve(args.native));
   const runner = await WebDNN.load(args.model, {
     backendOrder: args.backend === "cpu" ? ["cpu"] : ["hip", "cpu"],
     backendOptions: { hip: hipOption },
@@ -119,8 +122,14 @@ async function main() {
     }));
   }
   if (runner.backendContexts.hip && runner.backendContexts.hip.initialized) {
-    report.device = runner.backendContexts.hip.deviceInfo();
-    report.memory = runner.backendContexts.hip.memStats();
+    const hip = runner.backendContexts.hip;
+    report.device = hip.deviceInfo();
+    report.memory = hip.memStats();
+    if (hip.native.__liveBuffers) {
+      report.liveBuffers = hip.native.__liveBuffers();
+      report.nativeCalls = hip.native.__calls();
+      report.initializerCopies = Array.from(runner.copiedInitializerTensors.get("hip").keys()).length;
+    }
   }
   process.stdout.write(JSON.stringify(report) + "\n");
 }
