@@ -33,6 +33,10 @@ import numpy as np  # noqa: E402
 
 METRIC = "fp32 Gemm/Conv GFLOP/s (% MFMA peak) + ResNet-50 b32 images/sec, 1 MI355X"
 PEAK_FP32_MFMA_TFLOPS = 157.3
+# HBM-side bytes per contraction-kernel launch of the ResNet-50 step, averaged over its 54 launches:
+# rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB device copy;
+# recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read counters itself).
+TRAFFIC_BYTES_PER_LAUNCH = 82.6e6
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 
@@ -109,12 +113,20 @@ def timed_steps(ctx, step, steps, warmup):
     return ctx.event_elapsed_ms(0, 1) / steps
 
 
-def bench_kernels(steps, warmup):
+def bench_kernels(steps, warmup, calibrate_copy=False):
     """The two single-kernel figures the metric names, through the C ABI (ctypes)."""
+    from webdnn_amd import capi
     from webdnn_amd import hostops as H
 
     ctx = H.HipContext(0).initialize()
     rng = np.random.default_rng(0)
+    if calibrate_copy:
+        # a plain copy of known size: reads 256 MiB, writes 256 MiB
+        nbytes = 256 << 20
+        src, dst = ctx.empty_tensor([nbytes // 4]), ctx.empty_tensor([nbytes // 4])
+        for _ in range(3):
+            capi.call("wdh_copy", dst.handle, 0, src.handle, 0, nbytes)
+        ctx.sync()
     n = 4096
     A = ctx.move_tensor(rng.uniform(-1, 1, (n, n)).astype(np.float32))
     B = ctx.move_tensor(rng.uniform(-1, 1, (n, n)).astype(np.float32))
@@ -144,10 +156,17 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "kernels"], default="all",
+                    help="kernels: only the in-process Gemm 4096 / Conv C3 launches plus one device-to-device "
+                         "copy of known size (the unit for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the path shards by batch with no "
                  "exchange; multi-GPU runs are not part of it). Use --gpus 1.")
+
+    if args.only == "kernels":
+        print(json.dumps({"kernels": bench_kernels(args.steps, args.warmup, calibrate_copy=True)}))
+        return
 
     with tempfile.TemporaryDirectory(prefix="webdnn_bench_") as workdir:
         resnet = bench_resnet(args.steps, args.warmup, workdir)
@@ -179,7 +198,8 @@ def main():
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": None,
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic_note": "bytes/launch from rocprofv3 FETCH_SIZE+WRITE_SIZE, see profiles/; algorithmic 64.1e6",
             "flops_per_step": resnet["flops"],
             "avg_launch_ms": round(resnet["contraction_ms"] / resnet["contraction_launches"], 5),
         },
