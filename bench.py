@@ -80,6 +80,32 @@ def bench_resnet(steps, warmup, workdir):
     }
 
 
+def bench_report_only(workdir, steps, warmup):
+    """Configs 2 and 5, reported but not part of `value`: the FFN MatMul chain and the DETR-R50-style graph."""
+    from webdnn_amd import modelgen
+
+    out = {}
+    for key, (data, g), shape, label in (
+        ("ffn_c2", modelgen.ffn_model(), (8, 512, 768),
+         "MatMul chain X[8,512,768] -> 3072 -> 768 + residual, fused to 2 nodes (config 2)"),
+        ("detr_r50_b1", modelgen.detr_model(), (1, 3, 800, 1088),
+         "DETR-R50-style graph, input [1,3,800,1088], 850 tokens, 6+6 layers (config 5)"),
+    ):
+        d = os.path.join(workdir, key)
+        os.makedirs(d, exist_ok=True)
+        with open(os.path.join(d, "model.onnx"), "wb") as f:
+            f.write(data)
+        inp = os.path.join(d, "input.bin")
+        np.random.default_rng(11).standard_normal(shape).astype(np.float32).tofile(inp)
+        rep = node_run(d, inp, "hip", steps, warmup, ["--strict", "--resident-inputs"])
+        assert list(rep["stats"]["nodesByBackend"]) == ["hip"], rep["stats"]
+        ms = sum(rep["msPerRun"]) / len(rep["msPerRun"])
+        out[key] = {"workload": label, "nodes": rep["nodes"], "ms_per_run": round(ms, 4),
+                    "gflops": round(g.flops / ms / 1e6, 1),
+                    "frac_mfma_peak": round(g.flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
+    return out
+
+
 def cpu_baseline_resnet(workdir):
     """ResNet-50 on one image through the runner's cpu path with the JS oracle operators."""
     from webdnn_amd import modelgen
@@ -170,6 +196,7 @@ def main():
 
     with tempfile.TemporaryDirectory(prefix="webdnn_bench_") as workdir:
         resnet = bench_resnet(args.steps, args.warmup, workdir)
+        report_only = bench_report_only(workdir, max(3, args.steps // 2), min(args.warmup, 3))
         baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
     kernels = bench_kernels(args.steps, args.warmup)
 
@@ -206,6 +233,8 @@ def main():
         "extra": {
             "gemm_4096": kernels["gemm_4096"],
             "conv_c3": kernels["conv_c3"],
+            "ffn_c2": report_only["ffn_c2"],
+            "detr_r50_b1": report_only["detr_r50_b1"],
             "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
             "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),
             "device": resnet["device"],

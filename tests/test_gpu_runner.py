@@ -102,3 +102,23 @@ def test_non_strict_falls_back_per_node(tmp_path):
     assert rep["stats"]["retriedOnCpu"] == ["ReduceMean_1"]
     assert rep["stats"]["nodesByBackend"] == {"hip": 2, "cpu": 1}
     np.testing.assert_allclose(outs[0], np.maximum(np.maximum(X, 0).mean(0, keepdims=True), 0), rtol=1e-6)
+
+
+def test_detr_style_small(tmp_path):
+    data, g = modelgen.detr_model(image=(128, 160), d=64, heads=8, ffn=128, enc_layers=2, dec_layers=2, queries=20,
+                                  classes=11, width=16, blocks=(1, 1, 1, 1))
+    X = np.random.default_rng(9).standard_normal((1, 3, 128, 160)).astype(np.float32)
+    model, hip, rep = run_both(tmp_path, data, {"input": X})
+    want = graph_ref.run_graph(model, {"input": X})
+    assert np.abs(hip[0] - want["logits"]).max() <= 1e-3 and np.abs(hip[1] - want["boxes"]).max() <= 1e-3
+
+
+def test_detr_r50_config5(tmp_path):
+    """Config 5 at full size (input [1,3,800,1088], 850 tokens, 6+6 layers): outputs within 1e-3 of the oracle."""
+    data, g = modelgen.detr_model()
+    X = np.random.default_rng(10).standard_normal((1, 3, 800, 1088)).astype(np.float32)
+    model, hip, rep = run_both(tmp_path, data, {"input": X})
+    assert hip[0].shape == (100, 92) and hip[1].shape == (100, 4)
+    want = graph_ref.run_graph(model, {"input": X})
+    assert np.abs(hip[0] - want["logits"]).max() <= 1e-3, np.abs(hip[0] - want["logits"]).max()
+    assert np.abs(hip[1] - want["boxes"]).max() <= 1e-3

@@ -143,3 +143,21 @@ def test_unit_level_js(tmp_path):
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
     summary = json.loads(proc.stdout.strip().splitlines()[-1])
     assert summary["failed"] == 0 and summary["passed"] >= 14, summary
+
+
+def test_detr_style_graph_on_the_hip_host_path(tmp_path):
+    """The config-5 graph at toy size: every operator and shape trick it uses (head split by
+    Reshape+Transpose, K^T by Transpose, scalar Mul, Softmax, LayerNormalization, fused MatMul+bias,
+    Sigmoid) through the hip host code."""
+    data, g = modelgen.detr_model(image=(64, 96), d=32, heads=4, ffn=64, enc_layers=2, dec_layers=2, queries=10,
+                                  classes=7, width=8, blocks=(1, 1, 1, 1))
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(8).standard_normal((1, 3, 64, 96)).astype(np.float32)
+    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fake_native=True)
+    assert list(rep["stats"]["nodesByBackend"]) == ["hip"] and rep["liveBuffers"] == rep["initializerCopies"]
+    want = graph_ref.run_graph(modelgen.parse_model(data), {"input": X})
+    np.testing.assert_allclose(outs[0], want["logits"], rtol=0, atol=1e-5)
+    np.testing.assert_allclose(outs[1], want["boxes"], rtol=0, atol=1e-5)
+    plain, rep_p = node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fuse=False, fake_native=True)
+    assert rep_p["nodes"] > rep["nodes"]
+    assert_bit_exact(plain[0], outs[0], "fusion keeps the logits")

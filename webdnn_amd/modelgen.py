@@ -12,6 +12,7 @@ five benchmark configurations):
     ffn_model       MatMul -> Add -> Relu -> MatMul -> Add(residual)
     conv_model      Conv 3x3 -> Relu
     resnet50_model  ResNet-50 v1 with BatchNorm folded into the conv bias
+    detr_model      DETR-R50-style detector: ResNet-50 trunk, 1x1 projection, 6+6 transformer layers
 """
 import struct
 
@@ -312,43 +313,7 @@ def resnet50_model(batch=32, image=224, classes=1000, seed=0, width=64, blocks=(
     mean=0, var=1 and eps dropped (scale exactly 1, bias exactly 0), FC weights N(0, 0.01).
     Nodes: Conv, Relu, Add, MaxPool, GlobalAveragePool, Flatten, Gemm."""
     g = GraphBuilder(seed)
-    size = {"hw": image}
-
-    def conv(x, cin, cout, k, stride, pad, relu, name):
-        w = (g.rng().standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / (cin * k * k))).astype(np.float32)
-        g.const(name + "_w", w)
-        g.const(name + "_b", np.zeros(cout, np.float32))
-        out_hw = (size["hw"] + 2 * pad - k) // stride + 1
-        g.flops += 2 * batch * out_hw * out_hw * cout * cin * k * k
-        g.conv_gemm_nodes += 1
-        y = g.op("Conv", [x, name + "_w", name + "_b"], name, kernel_shape=[k, k], pads=[pad] * 4,
-                 strides=[stride, stride], dilations=[1, 1], group=1)
-        size["hw"] = out_hw
-        return g.op("Relu", [y], name + "_relu") if relu else y
-
-    x = conv("input", 3, width, 7, 2, 3, True, "stem")
-    x = g.op("MaxPool", [x], "pool", kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
-    size["hw"] = (size["hw"] + 2 - 3) // 2 + 1
-    cin = width
-    for stage, nblocks in enumerate(blocks):
-        mid, cout = width * 2 ** stage, width * 4 * 2 ** stage
-        for b in range(nblocks):
-            stride = 2 if (stage > 0 and b == 0) else 1
-            name = "s%db%d" % (stage + 1, b)
-            hw_in = size["hw"]
-            y = conv(x, cin, mid, 1, stride, 0, True, name + "_c1")
-            y = conv(y, mid, mid, 3, 1, 1, True, name + "_c2")
-            y = conv(y, mid, cout, 1, 1, 0, False, name + "_c3")
-            hw_out = size["hw"]
-            if b == 0:
-                size["hw"] = hw_in
-                shortcut = conv(x, cin, cout, 1, stride, 0, False, name + "_ds")
-                size["hw"] = hw_out
-            else:
-                shortcut = x
-            s = g.op("Add", [y, shortcut], name + "_add")
-            x = g.op("Relu", [s], name + "_out")
-            cin = cout
+    x, cin = _resnet_trunk(g, "input", batch, [image, image], width, blocks, init="he")
     x = g.op("GlobalAveragePool", [x], "gap")
     x = g.op("Flatten", [x], "flat", axis=1)
     g.const("fc_w", (g.rng().standard_normal((classes, cin)) * 0.01).astype(np.float32))
@@ -357,3 +322,164 @@ def resnet50_model(batch=32, image=224, classes=1000, seed=0, width=64, blocks=(
     g.flops += 2 * batch * classes * cin
     g.conv_gemm_nodes += 1
     return g.finish([("input", [batch, 3, image, image])], [("logits", [batch, classes])]), g
+
+
+def _resnet_trunk(g, x, batch, size, width=64, blocks=(3, 4, 6, 3), init="he"):
+    """ResNet-50 v1 trunk up to the last stage (no pooling head).  `size` = [h, w], updated in place.
+    Returns (tensor name, channels)."""
+
+    def conv(x, cin, cout, k, stride, pad, relu, name):
+        fan_in, fan_out = cin * k * k, cout * k * k
+        if init == "he":
+            w = g.rng().standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / fan_in)
+        else:  # Xavier-uniform
+            a = np.sqrt(6.0 / (fan_in + fan_out))
+            w = g.rng().uniform(-a, a, (cout, cin, k, k))
+        g.const(name + "_w", w.astype(np.float32))
+        g.const(name + "_b", np.zeros(cout, np.float32))
+        oh = (size[0] + 2 * pad - k) // stride + 1
+        ow = (size[1] + 2 * pad - k) // stride + 1
+        g.flops += 2 * batch * oh * ow * cout * cin * k * k
+        g.conv_gemm_nodes += 1
+        y = g.op("Conv", [x, name + "_w", name + "_b"], name, kernel_shape=[k, k], pads=[pad] * 4,
+                 strides=[stride, stride], dilations=[1, 1], group=1)
+        size[0], size[1] = oh, ow
+        return g.op("Relu", [y], name + "_relu") if relu else y
+
+    x = conv(x, 3, width, 7, 2, 3, True, "stem")
+    x = g.op("MaxPool", [x], "pool", kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
+    size[0], size[1] = (size[0] + 2 - 3) // 2 + 1, (size[1] + 2 - 3) // 2 + 1
+    cin = width
+    for stage, nblocks in enumerate(blocks):
+        mid, cout = width * 2 ** stage, width * 4 * 2 ** stage
+        for b in range(nblocks):
+            stride = 2 if (stage > 0 and b == 0) else 1
+            name = "s%db%d" % (stage + 1, b)
+            size_in = list(size)
+            y = conv(x, cin, mid, 1, stride, 0, True, name + "_c1")
+            y = conv(y, mid, mid, 3, 1, 1, True, name + "_c2")
+            y = conv(y, mid, cout, 1, 1, 0, False, name + "_c3")
+            size_out = list(size)
+            if b == 0:
+                size[0], size[1] = size_in
+                shortcut = conv(x, cin, cout, 1, stride, 0, False, name + "_ds")
+                size[0], size[1] = size_out
+            else:
+                shortcut = x
+            x = g.op("Relu", [g.op("Add", [y, shortcut], name + "_add")], name + "_out")
+            cin = cout
+    return x, cin
+
+
+def detr_model(image=(800, 1088), d=256, heads=8, ffn=2048, enc_layers=6, dec_layers=6, queries=100,
+               classes=92, seed=0, width=64, blocks=(3, 4, 6, 3)):
+    """Config 5: DETR-R50-style graph, batch 1.  ResNet-50 trunk -> 1x1 Conv to d -> tokens [T, d] with a
+    sinusoidal position encoding -> post-norm transformer (8-head attention as MatMul/Softmax,
+    LayerNormalization, FFN) -> class head Gemm [d, classes] and box MLP [d, d, 4] with Sigmoid.
+    Xavier-uniform weights, zero biases, learned queries ~N(0,1).  Every MatMul is rank <= 3 (the batch of
+    one is dropped), heads are split with Reshape + Transpose, opset 17 (LayerNormalization)."""
+    g = GraphBuilder(seed)
+    size = [image[0], image[1]]
+    x, cin = _resnet_trunk(g, "input", 1, size, width, blocks, init="xavier")
+    h, w = size
+    tokens = h * w
+    hd = d // heads
+
+    def xavier(name, shape):
+        a = np.sqrt(6.0 / (shape[0] + shape[1]))
+        return g.const(name, g.rng().uniform(-a, a, shape).astype(np.float32))
+
+    def zeros(name, n):
+        return g.const(name, np.zeros(n, np.float32))
+
+    def shape(name, dims):
+        return g.const(name, np.array(dims, np.int64))
+
+    def linear(xn, rows, din, dout, name, relu=False):
+        xavier(name + "_w", (din, dout))
+        zeros(name + "_b", dout)
+        g.flops += 2 * rows * din * dout
+        g.conv_gemm_nodes += 1
+        y = g.op("Add", [g.op("MatMul", [xn, name + "_w"], name + "_mm"), name + "_b"], name + "_lin")
+        return g.op("Relu", [y], name + "_relu") if relu else y
+
+    def layernorm(xn, name):
+        g.const(name + "_g", np.ones(d, np.float32))
+        zeros(name + "_beta", d)
+        return g.op("LayerNormalization", [xn, name + "_g", name + "_beta"], name, axis=-1, epsilon=1e-5)
+
+    def attention(q_in, k_in, v_in, tq, tk, name):
+        q = linear(q_in, tq, d, d, name + "_q")
+        k = linear(k_in, tk, d, d, name + "_k")
+        v = linear(v_in, tk, d, d, name + "_v")
+        shape(name + "_sq", [tq, heads, hd])
+        shape(name + "_sk", [tk, heads, hd])
+        shape(name + "_so", [tq, d])
+        qh = g.op("Transpose", [g.op("Reshape", [q, name + "_sq"], name + "_q3")], name + "_qh", perm=[1, 0, 2])
+        kt = g.op("Transpose", [g.op("Reshape", [k, name + "_sk"], name + "_k3")], name + "_kt", perm=[1, 2, 0])
+        vh = g.op("Transpose", [g.op("Reshape", [v, name + "_sk"], name + "_v3")], name + "_vh", perm=[1, 0, 2])
+        g.const(name + "_scale", np.array(1.0 / np.sqrt(hd), np.float32))
+        scores = g.op("MatMul", [qh, kt], name + "_scores")
+        attn = g.op("Softmax", [g.op("Mul", [scores, name + "_scale"], name + "_scaled")], name + "_attn", axis=-1)
+        ctx = g.op("MatMul", [attn, vh], name + "_ctx")
+        g.flops += 2 * 2 * heads * tq * tk * hd
+        g.conv_gemm_nodes += 2
+        merged = g.op("Reshape", [g.op("Transpose", [ctx], name + "_ctx_t", perm=[1, 0, 2]), name + "_so"], name + "_merged")
+        return linear(merged, tq, d, d, name + "_o")
+
+    # 1x1 projection and flattening to tokens
+    a = np.sqrt(6.0 / (cin + d))
+    g.const("proj_w", g.rng().uniform(-a, a, (d, cin, 1, 1)).astype(np.float32))
+    zeros("proj_b", d)
+    g.flops += 2 * tokens * d * cin
+    g.conv_gemm_nodes += 1
+    p = g.op("Conv", [x, "proj_w", "proj_b"], "proj", kernel_shape=[1, 1], pads=[0, 0, 0, 0], strides=[1, 1],
+             dilations=[1, 1], group=1)
+    shape("tok_shape", [d, tokens])
+    src = g.op("Transpose", [g.op("Reshape", [p, "tok_shape"], "proj_flat")], "src0", perm=[1, 0])
+    # sinusoidal position encoding over (y, x), d/2 channels each
+    half = d // 2
+    dim_t = 10000.0 ** (2 * (np.arange(half) // 2) / half)
+    ys, xs = np.meshgrid(np.arange(1, h + 1), np.arange(1, w + 1), indexing="ij")
+    scale = 2 * np.pi
+    py = (ys / (h + 1e-6) * scale)[..., None] / dim_t
+    px = (xs / (w + 1e-6) * scale)[..., None] / dim_t
+    enc = lambda t: np.stack([np.sin(t[..., 0::2]), np.cos(t[..., 1::2])], axis=-1).reshape(h, w, half)
+    g.const("pos", np.concatenate([enc(py), enc(px)], axis=-1).reshape(tokens, d).astype(np.float32))
+
+    for i in range(enc_layers):
+        n = "enc%d" % i
+        qk = g.op("Add", [src, "pos"], n + "_qk")
+        sa = attention(qk, qk, src, tokens, tokens, n + "_sa")
+        src = layernorm(g.op("Add", [src, sa], n + "_res1"), n + "_ln1")
+        f = linear(linear(src, tokens, d, ffn, n + "_f1", relu=True), tokens, ffn, d, n + "_f2")
+        src = layernorm(g.op("Add", [src, f], n + "_res2"), n + "_ln2")
+    memory = src
+    mem_k = g.op("Add", [memory, "pos"], "mem_k")
+
+    g.const("query_pos", g.rng().standard_normal((queries, d)).astype(np.float32))
+    tgt = g.const("tgt0", np.zeros((queries, d), np.float32))
+    for i in range(dec_layers):
+        n = "dec%d" % i
+        qk = g.op("Add", [tgt, "query_pos"], n + "_qk")
+        sa = attention(qk, qk, tgt, queries, queries, n + "_sa")
+        tgt = layernorm(g.op("Add", [tgt, sa], n + "_res1"), n + "_ln1")
+        q = g.op("Add", [tgt, "query_pos"], n + "_q")
+        ca = attention(q, mem_k, memory, queries, tokens, n + "_ca")
+        tgt = layernorm(g.op("Add", [tgt, ca], n + "_res2"), n + "_ln2")
+        f = linear(linear(tgt, queries, d, ffn, n + "_f1", relu=True), queries, ffn, d, n + "_f2")
+        tgt = layernorm(g.op("Add", [tgt, f], n + "_res3"), n + "_ln3")
+    hs = layernorm(tgt, "dec_norm")
+
+    xavier("class_w", (d, classes))
+    zeros("class_b", classes)
+    g.flops += 2 * queries * d * classes
+    g.op("Gemm", [hs, "class_w", "class_b"], "logits", alpha=1.0, beta=1.0)
+    b1 = linear(hs, queries, d, d, "box1", relu=True)
+    b2 = linear(b1, queries, d, d, "box2", relu=True)
+    b3 = linear(b2, queries, d, 4, "box3")
+    g.op("Sigmoid", [b3], "boxes")
+    g.conv_gemm_nodes += 1
+    data = g.finish([("input", [1, 3, image[0], image[1]])], [("logits", [queries, classes]), ("boxes", [queries, 4])],
+                    opset=17)
+    return data, g
