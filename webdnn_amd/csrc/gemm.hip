@@ -47,13 +47,35 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+// Buffer descriptors: untyped 32-bit data, a window of 2^31-1 bytes above the
+// base.  A byte offset with bit 31 set lies outside every such window and the
+// hardware returns 0 for it without touching memory, which is how padding
+// taps of a convolution are read.
+constexpr int BUF_WORD3 = 0x00020000;
+constexpr int BUF_RANGE = 0x7fffffff;
+constexpr int BUF_OOB = (int)0x80000000u;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, BUF_RANGE, BUF_WORD3);
+}
+__device__ __forceinline__ float buf_load(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ f32x4 buf_load4(rsrc_t r, int voff, int soff) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
 
 constexpr int BK = 16;
 constexpr int NTHREADS = 256;
 constexpr int LDK = BK + 4;  // KC tile row stride (floats)
 constexpr int MC_PAD = 8;    // MC tile row stride = extent + 8 (floats)
 
-enum BMode { B_KC = 0, B_MC = 1, B_IM2COL = 2, B_IM2COL_BIG = 3 };  // BIG: more than 64 taps
+// B_IM2COL32 / B_IM2COL64: at most 31 / 63 taps and X below 2 GiB, read through
+// a buffer descriptor; B_IM2COL_BIG: anything else, read with flat loads.
+enum BMode { B_KC = 0, B_MC = 1, B_IM2COL32 = 2, B_IM2COL64 = 3, B_IM2COL_BIG = 4 };
 
 struct ConvGeom {
   int c_in_g;        // input channels per group
@@ -66,9 +88,11 @@ struct ConvGeom {
   int cout_g;        // output channels per group
   int ntaps;         // kh*kw
   long long npix;    // batch * oh * ow
-  // per k = (ci, ky, kx): x = ci*h*w + ky*dh*w + kx*dw (offset from the
-  // receptive field's corner), y = tap index ky*kw+kx (at most 64 taps) or
-  // (ky*dh)<<16 | kx*dw (otherwise); padded with zeros to a multiple of 16
+  // per k = (ci, ky, kx), padded to a multiple of 16 entries.
+  // Descriptor modes: x = 4*(ci*h*w + ky*dh*w + kx*dw), the byte offset from
+  // the receptive field's corner, y = tap index ky*kw+kx; padding entries
+  // carry tap 31 (B_IM2COL32) or 63 (B_IM2COL64), which no pixel has.
+  // B_IM2COL_BIG: x = the same offset in elements, y = (ky*dh)<<16 | kx*dw.
   const int2 *ktab;
   // per tap: (ky*dh)<<16 | kx*dw, used to build the per-pixel mask
   const int *taptab;
@@ -90,6 +114,7 @@ struct Params {
   int ksplit;       // > 1: K is cut into ksplit chunks (blockIdx.z), partial sums go to `partial`
   int kchunk;       // chunk length, a multiple of 16
   float *partial;   // [ksplit][gridDim.y][m][n] raw sums
+  int fast;         // every operand spans less than 2 GiB: descriptor loads allowed
   ConvGeom cv;
 };
 
@@ -187,10 +212,10 @@ struct PixelCtx {
   const float *xbase;       // X + (image*c_total + group*c_in_g)*h*w (image 0 past the edge)
   int pbase;                // iy0*w + ix0
   int iy0, ix0;             // corner of the receptive field (may be negative)
-  unsigned long long mask;  // bit t set: tap t falls inside the input (0 past the edge)
+  unsigned long long mask;  // 1 for a pixel of the output, 0 past the edge
 };
 
-template <int EXT, bool MASK>
+template <int EXT>
 __device__ __forceinline__ unsigned fetch_im2col(const ConvGeom &cv,
                                                  const PixelCtx &px, int k0,
                                                  int kdim, int tid,
@@ -206,20 +231,56 @@ __device__ __forceinline__ unsigned fetch_im2col(const ConvGeom &cv,
   unsigned okbits = 0;
 #pragma unroll
   for (int i = 0; i < L; i++) {
-    bool ok;
-    if (MASK) {
-      ok = (px.mask >> e[i].y) & 1ull;
-    } else {
-      const int iy = px.iy0 + (e[i].y >> 16), ix = px.ix0 + (e[i].y & 0xffff);
-      ok = px.mask && (unsigned)iy < (unsigned)cv.h && (unsigned)ix < (unsigned)cv.w;
-    }
-    ok = ok && kfirst + i < kdim;
+    const int iy = px.iy0 + (e[i].y >> 16), ix = px.ix0 + (e[i].y & 0xffff);
+    const bool ok = px.mask && (unsigned)iy < (unsigned)cv.h &&
+                    (unsigned)ix < (unsigned)cv.w && kfirst + i < kdim;
     // Unconditional load from a safe address; the value is zeroed when it is
     // stored to LDS (stash_im2col), so nothing here waits for the load.
     reg[i >> 2][i & 3] = px.xbase[ok ? px.pbase + e[i].x : 0];
     okbits |= (ok ? 1u : 0u) << i;
   }
   return okbits;
+}
+
+// ---- the same fetches through a buffer descriptor --------------------------
+// Everything a thread needs to know about its rows is folded into one byte
+// offset per 16-byte piece before the K loop starts; advancing along K is a
+// scalar offset, so a slab costs no vector ALU work beyond the loads.
+template <int EXT, bool VEC>
+__device__ __forceinline__ void fetch_rows_fast(rsrc_t r, const int (&voff)[EXT / 64],
+                                                int soff, f32x4 (&reg)[EXT / 64]) {
+#pragma unroll
+  for (int i = 0; i < EXT / 64; i++) {
+    if (VEC)
+      reg[i] = buf_load4(r, voff[i], soff);
+    else
+      reg[i] = f32x4{buf_load(r, voff[i], soff), buf_load(r, voff[i] + 4, soff),
+                     buf_load(r, voff[i] + 8, soff), buf_load(r, voff[i] + 12, soff)};
+  }
+}
+
+// Per-thread constants of the descriptor im2col fetch.
+struct PixelFast {
+  int valid;            // byte offset of the receptive field's corner, biased to be >= 0
+  unsigned pad_lo;      // bit t set: tap t of this pixel falls in the padding (taps 0..31)
+  unsigned pad_hi;      // taps 32..63
+};
+
+template <int EXT, bool TAPS64>
+__device__ __forceinline__ void fetch_im2col_fast(rsrc_t r, const int2 *__restrict__ ktab,
+                                                  const PixelFast &px, int kfirst,
+                                                  f32x4 (&reg)[EXT / 64]) {
+  constexpr int G = NTHREADS / EXT, L = BK / G;
+  int2 e[L];
+#pragma unroll
+  for (int i = 0; i < L; i++) e[i] = ktab[kfirst + i];
+#pragma unroll
+  for (int i = 0; i < L; i++) {
+    const unsigned word = (TAPS64 && (e[i].y & 32)) ? px.pad_hi : px.pad_lo;
+    // -1 when the tap is padding, 0 otherwise
+    const int pad = __builtin_amdgcn_sbfe((int)word, (unsigned)e[i].y & 31u, 1u);
+    reg[i >> 2][i & 3] = buf_load(r, (pad & BUF_OOB) | px.valid, e[i].x);
+  }
 }
 
 // ---- register -> LDS -------------------------------------------------------
@@ -249,6 +310,15 @@ __device__ __forceinline__ void stash_im2col(float *tile, int tid,
     tile[(kgroup * L + i) * LD + pix] = ((okbits >> i) & 1u) ? reg[i >> 2][i & 3] : 0.0f;
 }
 
+template <int EXT>
+__device__ __forceinline__ void stash_im2col_fast(float *tile, int tid,
+                                                  const f32x4 (&reg)[EXT / 64]) {
+  constexpr int G = NTHREADS / EXT, L = BK / G, LD = EXT + MC_PAD;
+  const int kgroup = tid / EXT, pix = tid % EXT;
+#pragma unroll
+  for (int i = 0; i < L; i++) tile[(kgroup * L + i) * LD + pix] = reg[i >> 2][i & 3];
+}
+
 constexpr int tile_floats(bool kc, int ext) { return kc ? ext * LDK : BK * (ext + MC_PAD); }
 
 // ---- the kernel -------------------------------------------------------------
@@ -261,13 +331,14 @@ constexpr int min_blocks(int bm, int bn) {
 
 template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE_, bool VEC>
 __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kernel(Params p) {
-  constexpr bool MASK = BMODE_ == B_IM2COL;
-  constexpr int BMODE = BMODE_ == B_IM2COL_BIG ? (int)B_IM2COL : BMODE_;
+  constexpr bool IM2COL_FAST = BMODE_ == B_IM2COL32 || BMODE_ == B_IM2COL64;
+  constexpr bool IM2COL = IM2COL_FAST || BMODE_ == B_IM2COL_BIG;
+  constexpr bool B_IS_KC = BMODE_ == B_KC;
   static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
   constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
   static_assert(MT >= 1 && NT >= 1, "tile too small for the wavefront grid");
   constexpr int A_FLOATS = tile_floats(A_KC, BM);
-  constexpr int B_FLOATS = tile_floats(BMODE == B_KC, BN);
+  constexpr int B_FLOATS = tile_floats(B_IS_KC, BN);
   constexpr int LDA = BM + MC_PAD, LDB = BN + MC_PAD;
   __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
   __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
@@ -287,36 +358,86 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   const float *A = p.A + (long long)bz * p.sAb;
   const float *B = p.B + (long long)bz * p.sBb;
   const long long lda = A_KC ? p.sA0 : p.sA1;
-  const long long ldb = (BMODE == B_KC) ? p.sB1 : p.sB0;
+  const long long ldb = B_IS_KC ? p.sB1 : p.sB0;
 
+  // this workgroup's share of K
+  const int kbeg = p.ksplit > 1 ? (int)blockIdx.z * p.kchunk : 0;
+  const int kend = p.ksplit > 1 ? (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k) : p.k;
+
+  // ---- descriptor fetch plans: one byte offset per 16-byte piece -------------
+  // A row-major-in-K operand may always take this path (rows past the edge are
+  // clamped, their products are never stored); an operand that is contiguous
+  // along M or N takes it on tiles that lie fully inside the matrix.
+  const bool a_fast = p.fast && (A_KC || (VEC && row0 + BM <= p.m));
+  const bool b_fast = p.fast && (B_IS_KC || IM2COL_FAST || (VEC && col0 + BN <= p.n));
+  int voff_a[BM / 64], voff_b[BN / 64];
+  if (A_KC) {
+#pragma unroll
+    for (int i = 0; i < BM / 64; i++) {
+      int r = row0 + (tid >> 2) + i * 64;
+      r = r < p.m ? r : p.m - 1;
+      voff_a[i] = (int)(((long long)r * lda + (tid & 3) * 4) * 4);
+    }
+  } else {
+    constexpr int TPR = BM / 4, RPP = NTHREADS / TPR;
+#pragma unroll
+    for (int i = 0; i < BM / 64; i++)
+      voff_a[i] = (int)(((long long)(tid / TPR + i * RPP) * lda + row0 + (tid % TPR) * 4) * 4);
+  }
+  if (B_IS_KC) {
+#pragma unroll
+    for (int i = 0; i < BN / 64; i++) {
+      int c = col0 + (tid >> 2) + i * 64;
+      c = c < p.n ? c : p.n - 1;
+      voff_b[i] = (int)(((long long)c * ldb + (tid & 3) * 4) * 4);
+    }
+  } else if (!IM2COL) {
+    constexpr int TPR = BN / 4, RPP = NTHREADS / TPR;
+#pragma unroll
+    for (int i = 0; i < BN / 64; i++)
+      voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + col0 + (tid % TPR) * 4) * 4);
+  }
+  const rsrc_t rsrc_a = make_rsrc(A);
+
+  // ---- im2col: what this thread's pixel looks like ----------------------------
   PixelCtx px = {p.B, 0, 0, 0, 0ull};
-  if (BMODE == B_IM2COL) {
+  PixelFast pf = {0, 0xffffffffu, 0xffffffffu};
+  const float *bbase = B;  // base of the B descriptor
+  if (IM2COL) {
     const long long P = (long long)col0 + (tid % BN);
     const long long plane = (long long)p.cv.h * p.cv.w;
+    const int bias = p.cv.pt * p.cv.w + p.cv.pl;  // makes every corner offset >= 0
     px.xbase = p.B + (long long)bz * p.cv.c_in_g * plane;
+    bbase = px.xbase - bias;
     if (P < p.cv.npix) {
       const int ohw = p.cv.oh * p.cv.ow;
       const int img = (int)(P / ohw);
       const int q = (int)(P - (long long)img * ohw);
       const int oy = q / p.cv.ow, ox = q - oy * p.cv.ow;
-      px.xbase += (long long)img * p.cv.c_total * plane;
+      const long long img_off = (long long)img * p.cv.c_total * plane;
       px.iy0 = oy * p.cv.sh - p.cv.pt;
       px.ix0 = ox * p.cv.sw - p.cv.pl;
       px.pbase = px.iy0 * p.cv.w + px.ix0;
-      if (MASK) {
-        unsigned long long m = 0;
+      if (IM2COL_FAST) {
+        pf.valid = (int)((img_off + px.pbase + bias) * 4);
+        unsigned long long inside = 0;
         for (int t = 0; t < p.cv.ntaps; t++) {
           const int d = p.cv.taptab[t];
           const int iy = px.iy0 + (d >> 16), ix = px.ix0 + (d & 0xffff);
           if ((unsigned)iy < (unsigned)p.cv.h && (unsigned)ix < (unsigned)p.cv.w)
-            m |= 1ull << t;
+            inside |= 1ull << t;
         }
-        px.mask = m;
+        pf.pad_lo = ~(unsigned)inside;
+        pf.pad_hi = ~(unsigned)(inside >> 32);
       } else {
+        px.xbase += img_off;
         px.mask = 1ull;
       }
     }
   }
+  const rsrc_t rsrc_b = make_rsrc(bbase);
+  // first of the L consecutive k rows this wavefront gathers in each slab
+  const int kgroup0 = IM2COL ? __builtin_amdgcn_readfirstlane(tid / BN) * (BK / (NTHREADS / BN)) : 0;
 
   f32x16 acc[MT][NT];
 #pragma unroll
@@ -326,38 +447,56 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
 
-  // this workgroup's share of K
-  const int kbeg = p.ksplit > 1 ? (int)blockIdx.z * p.kchunk : 0;
-  const int kend = p.ksplit > 1 ? (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k) : p.k;
-
   // Registers that carry one fetched K slab from global memory to LDS.
   struct Staged {
     f32x4 a[BM / 64], b[BN / 64];
-    unsigned ok;  // im2col only: which fetched taps lie inside the input
+    unsigned ok;  // flat im2col only: which fetched taps lie inside the input
   };
-  auto fetch = [&](int k0, Staged &st) {
-    if (A_KC)
+  // Descriptor-only fetch: legal for a slab that lies fully inside K when
+  // both operands qualify (all_fast).
+  auto fetch_fast = [&](int k0, Staged &st) {
+    fetch_rows_fast<BM, VEC>(rsrc_a, voff_a, A_KC ? k0 * 4 : (int)(k0 * lda * 4), st.a);
+    if (IM2COL_FAST)
+      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(rsrc_b, p.cv.ktab, pf, k0 + kgroup0, st.b);
+    else if (!IM2COL)
+      fetch_rows_fast<BN, VEC>(rsrc_b, voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * ldb * 4), st.b);
+  };
+  // Fetch that copes with everything: ragged last slab, edge tiles, huge operands.
+  auto fetch_any = [&](int k0, Staged &st) {
+    const bool full = k0 + BK <= kend;
+    if (a_fast && full) {
+      fetch_rows_fast<BM, VEC>(rsrc_a, voff_a, A_KC ? k0 * 4 : (int)(k0 * lda * 4), st.a);
+    } else if (A_KC) {
       fetch_kc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
-    else
+    } else {
       fetch_mc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
-    if (BMODE == B_KC)
+    }
+    if (IM2COL_FAST) {
+      // padding entries of the tap table read as 0, so a ragged K needs no care
+      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(rsrc_b, p.cv.ktab, pf, k0 + kgroup0, st.b);
+    } else if (IM2COL) {
+      st.ok = fetch_im2col<BN>(p.cv, px, k0, kend, tid, st.b);
+    } else if (b_fast && full) {
+      fetch_rows_fast<BN, VEC>(rsrc_b, voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * ldb * 4), st.b);
+    } else if (B_IS_KC) {
       fetch_kc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
-    else if (BMODE == B_MC)
+    } else {
       fetch_mc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
-    else
-      st.ok = fetch_im2col<BN, MASK>(p.cv, px, k0, kend, tid, st.b);
+    }
   };
   auto stash = [&](int buf, const Staged &st) {
     if (A_KC)
       stash_kc<BM>(lds_a[buf], tid, st.a);
     else
       stash_mc<BM>(lds_a[buf], tid, st.a);
-    if (BMODE == B_KC)
+    if (B_IS_KC)
       stash_kc<BN>(lds_b[buf], tid, st.b);
-    else if (BMODE == B_MC)
-      stash_mc<BN>(lds_b[buf], tid, st.b);
-    else
+    else if (IM2COL_FAST)
+      stash_im2col_fast<BN>(lds_b[buf], tid, st.b);
+    else if (IM2COL)
       stash_im2col<BN>(lds_b[buf], tid, st.b, st.ok);
+    else
+      stash_mc<BN>(lds_b[buf], tid, st.b);
   };
   // One K slab from LDS buffer `cur` through the matrix cores.
   auto compute = [&](int cur) {
@@ -372,7 +511,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
           av[mt][j] = *reinterpret_cast<const f32x4 *>(
               ta + (wrow + mt * 32 + li) * LDK + 8 * j + 4 * half);
     }
-    if (BMODE == B_KC) {
+    if (B_IS_KC) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
 #pragma unroll
@@ -389,8 +528,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
         a_el[mt] = A_KC ? av[mt][st >> 2][st & 3] : ta[kk * LDA + wrow + mt * 32 + li];
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
-        b_el[nt] = (BMODE == B_KC) ? bv[nt][st >> 2][st & 3]
-                                   : tb[kk * LDB + wcol + nt * 32 + li];
+        b_el[nt] = B_IS_KC ? bv[nt][st >> 2][st & 3] : tb[kk * LDB + wcol + nt * 32 + li];
 #pragma unroll
       for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -400,16 +538,34 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     }
   };
 
+  // Slab s+1 travels global -> registers while slab s runs through the matrix
+  // cores, then goes to the other LDS buffer.  (A second slab in flight was
+  // measured and bought nothing.)  The main loop takes two slabs per trip, so
+  // that LDS buffer indices are compile-time constants, and contains
+  // descriptor fetches only; the few slabs it leaves over (and every slab of a
+  // workgroup that cannot use descriptors) run in the general loop below it.
   const int nslabs = (kend - kbeg + BK - 1) / BK;
+  const int nfull = (kend - kbeg) / BK;
+  const bool all_fast = a_fast && b_fast && !(IM2COL && !IM2COL_FAST);
+  const int nfast = all_fast ? nfull - 1 : 0;  // steps whose next slab is a full one
   Staged st0;
-  fetch(kbeg, st0);
+  fetch_any(kbeg, st0);
   stash(0, st0);
   __syncthreads();
-  // fetch slab s+1 while slab s computes (a second slab in flight was measured
-  // and bought nothing: the loop is not waiting on these loads)
-  for (int s = 0; s < nslabs; s++) {
+  int s = 0;
+  for (; s + 2 <= nfast; s += 2) {
+    fetch_fast(kbeg + (s + 1) * BK, st0);
+    compute(0);
+    stash(1, st0);
+    __syncthreads();
+    fetch_fast(kbeg + (s + 2) * BK, st0);
+    compute(1);
+    stash(0, st0);
+    __syncthreads();
+  }
+  for (; s < nslabs; s++) {
     const int cur = s & 1;
-    if (s + 1 < nslabs) fetch(kbeg + (s + 1) * BK, st0);
+    if (s + 1 < nslabs) fetch_any(kbeg + (s + 1) * BK, st0);
     compute(cur);
     if (s + 1 < nslabs) stash(cur ^ 1, st0);
     __syncthreads();
@@ -441,7 +597,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     if (col >= p.n) continue;
     long long ybase;     // offset of (row 0, this column) in Y
     long long ystride;   // distance between consecutive rows in Y
-    if (BMODE == B_IM2COL) {
+    if (IM2COL) {
       const int ohw = p.cv.oh * p.cv.ow;
       const int img = col / ohw;
       const int q = col - img * ohw;
@@ -459,7 +615,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
         if (row >= p.m) continue;
         float y = p.alpha * acc[mt][nt][r];
         if (p.C) {
-          float c = (BMODE == B_IM2COL)
+          float c = IM2COL
                         ? p.C[bz * p.cv.cout_g + row]
                         : p.C[(long long)row * p.sC0 + (long long)col * p.sC1];
           y = __builtin_fmaf(c, p.beta, y);
@@ -607,7 +763,7 @@ int launch_tile(Params &p, int nz, bool vec) {
     long long blocks = (total + 255) / 256;
     const long long cap = 16LL * wdh::compute_units();
     if (blocks > cap) blocks = cap;
-    if (BMODE == B_IM2COL || BMODE == B_IM2COL_BIG)
+    if (BMODE >= B_IM2COL32)
       hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
                          wdh::stream(), p, nz);
     else
@@ -628,7 +784,7 @@ int launch(Params &p, int nz, bool vec) {
   // Convs measured best on 64x64 tiles at every ResNet-50 layer shape (more
   // wavefronts in flight to cover the gather's latency); Gemm/MatMul use the
   // cost model.
-  const bool conv = BMODE == B_IM2COL || BMODE == B_IM2COL_BIG;
+  const bool conv = BMODE >= B_IM2COL32;
   TileId t = g_forced_tile >= 0 ? (TileId)g_forced_tile
                                 : (conv ? T64x64 : pick_tile(p.m, p.n, nz));
   switch (t) {
@@ -740,6 +896,10 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   if (useB_kc) p.sB0 = 1; else p.sB1 = 1;
   const bool vec = vec_ok(p.A, useA_kc ? p.sA0 : p.sA1, sAb) &&
                    vec_ok(p.B, useB_kc ? p.sB1 : p.sB0, sBb);
+  // Descriptor loads address one batch entry with 32-bit byte offsets (a
+  // clamped edge row plus a 16-byte piece may reach 12 bytes past the span).
+  p.fast = (span(1, 0, m, p.sA0, k, p.sA1) + 4) * 4 < 0x7fffffffLL &&
+           (span(1, 0, k, p.sB0, n, p.sB1) + 4) * 4 < 0x7fffffffLL;
   if (useA_kc && useB_kc) return launch<true, B_KC>(p, batch, vec);
   if (useA_kc && !useB_kc) return launch<true, B_MC>(p, batch, vec);
   if (!useA_kc && useB_kc) return launch<false, B_KC>(p, batch, vec);
@@ -753,7 +913,7 @@ namespace {
 // Tap tables per conv geometry, built on the host once and kept on the device
 // for the life of the library.
 struct KtabKey {
-  int c_in_g, kh, kw, dh, dw, h, w;
+  int c_in_g, kh, kw, dh, dw, h, w, mode;
   bool operator<(const KtabKey &o) const {
     return memcmp(this, &o, sizeof(*this)) < 0;
   }
@@ -830,22 +990,35 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.Y = (float *)ptr;
 
   const int ntaps = kh * kw;
-  const bool mask_mode = ntaps <= 64;
+  // Descriptor loads need every byte offset formed in the kernel (X, shifted up
+  // by the top-left padding, and one group's weights) to stay below 2^31.
+  const long long x_bytes = ((long long)n * c * h * w + (long long)pt * w + pl) * 4;
+  const long long w_bytes = (long long)cout_g * kdim * 4;
+  const bool small = x_bytes < 0x7fffffffLL && w_bytes < 0x7fffffffLL;
+  const int mode = !small || ntaps > 63 ? B_IM2COL_BIG : (ntaps > 31 ? B_IM2COL64 : B_IM2COL32);
   KtabKey key;
   memset(&key, 0, sizeof(key));
   key.c_in_g = c_in_g; key.kh = kh; key.kw = kw; key.dh = dh; key.dw = dw;
-  key.h = h; key.w = w;
+  key.h = h; key.w = w; key.mode = mode;
   auto it = g_ktabs.find(key);
   if (it == g_ktabs.end()) {
-    std::vector<int2> tab((size_t)((kdim + BK - 1) / BK * BK), int2{0, 0});
+    const int pad_tap = mode == B_IM2COL32 ? 31 : 63;
+    std::vector<int2> tab((size_t)((kdim + BK - 1) / BK * BK),
+                          mode == B_IM2COL_BIG ? int2{0, 0} : int2{0, pad_tap});
     std::vector<int> taps((size_t)ntaps);
     size_t idx = 0;
     for (int ci = 0; ci < c_in_g; ci++)
       for (int ky = 0; ky < kh; ky++)
         for (int kx = 0; kx < kw; kx++) {
           const int packed = ((ky * dh) << 16) | (kx * dw);
-          tab[idx].x = ci * h * w + ky * dh * w + kx * dw;
-          tab[idx].y = mask_mode ? ky * kw + kx : packed;
+          const int off = ci * h * w + ky * dh * w + kx * dw;
+          if (mode == B_IM2COL_BIG) {
+            tab[idx].x = off;
+            tab[idx].y = packed;
+          } else {
+            tab[idx].x = off * 4;
+            tab[idx].y = ky * kw + kx;
+          }
           taps[ky * kw + kx] = packed;
           idx++;
         }
@@ -874,6 +1047,8 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.ntaps = ntaps;
   p.cv.npix = npix; p.cv.ktab = it->second.ktab; p.cv.taptab = it->second.taptab;
   const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
-  if (mask_mode) return launch<true, B_IM2COL>(p, group, vec);
+  p.fast = small ? 1 : 0;
+  if (mode == B_IM2COL32) return launch<true, B_IM2COL32>(p, group, vec);
+  if (mode == B_IM2COL64) return launch<true, B_IM2COL64>(p, group, vec);
   return launch<true, B_IM2COL_BIG>(p, group, vec);
 }
