@@ -36,6 +36,22 @@
 // and gathers its taps straight from X (NCHW), consecutive lanes reading
 // consecutive addresses; the epilogue scatters rows back to NCHW and fuses
 // bias, residual and Relu.
+//
+// Global loads go through buffer descriptors wherever an operand spans less
+// than 2 GiB: every per-thread address term is folded into one byte offset
+// before the K loop, K advances through the instruction's scalar offset, and a
+// conv tap that falls in the padding is given an offset outside the
+// descriptor's window so that the hardware returns 0 for it.  The main loop
+// then holds no vector-ALU address arithmetic at all (vector-ALU instructions
+// issue in the same slot as the matrix-core ones and were measured to cost
+// about 2.5 cycles of matrix-core time each).  Ragged K ends, edge tiles of
+// an operand contiguous along M/N and operands of 2 GiB or more take a slower
+// flat-load path in a separate general loop.
+//
+// Work decomposition (plan_work): whole tiles fill complete rounds over the
+// CUs; the tiles left over, or every tile when there are too few to occupy
+// the chip, are cut along K into chunks whose partial sums a second kernel
+// adds in a fixed order.
 #include <string.h>
 
 #include <map>
@@ -50,16 +66,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-// Buffer descriptors: untyped 32-bit data, a window of 2^31-1 bytes above the
-// base.  A byte offset with bit 31 set lies outside every such window and the
-// hardware returns 0 for it without touching memory, which is how padding
-// taps of a convolution are read.
+// Buffer descriptors: untyped 32-bit data, a window of `bytes` (< 2^31) above
+// the base that covers exactly the operand.  A byte offset outside the window
+// makes the hardware return 0 without touching memory; an offset with bit 31
+// set is outside every window, which is how padding taps of a convolution are
+// read.
 constexpr int BUF_WORD3 = 0x00020000;
-constexpr int BUF_RANGE = 0x7fffffff;
 constexpr int BUF_OOB = (int)0x80000000u;
 
-__device__ __forceinline__ rsrc_t make_rsrc(const void *base) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, BUF_RANGE, BUF_WORD3);
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, BUF_WORD3);
 }
 __device__ __forceinline__ float buf_load(rsrc_t r, int voff, int soff) {
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
@@ -83,6 +99,8 @@ struct ConvGeom {
   int oh, ow;        // output spatial size
   int pt, pl;        // top / left padding
   int sh, sw;        // strides
+  int kh, kw;        // kernel size
+  int dh, dw;        // dilations
   int c_total;       // input channels (all groups)
   int cout_total;    // output channels (all groups)
   int cout_g;        // output channels per group
@@ -94,8 +112,6 @@ struct ConvGeom {
   // carry tap 31 (B_IM2COL32) or 63 (B_IM2COL64), which no pixel has.
   // B_IM2COL_BIG: x = the same offset in elements, y = (ky*dh)<<16 | kx*dw.
   const int2 *ktab;
-  // per tap: (ky*dh)<<16 | kx*dw, used to build the per-pixel mask
-  const int *taptab;
 };
 
 struct Params {
@@ -111,10 +127,19 @@ struct Params {
   float alpha, beta;
   int epilogue;
   int tiles_m, tiles_n;
-  int ksplit;       // > 1: K is cut into ksplit chunks (blockIdx.z), partial sums go to `partial`
-  int kchunk;       // chunk length, a multiple of 16
-  float *partial;   // [ksplit][gridDim.y][m][n] raw sums
+  // Work decomposition.  Tiles are numbered tile + z * tiles_m * tiles_n (z =
+  // batch entry or conv group).  The first full_tiles of them are computed by
+  // one workgroup each; every remaining ("tail") tile is cut along K into
+  // tail_split chunks of kchunk elements, one workgroup per chunk, whose raw
+  // sums go to `partial` and are added up by splitk_reduce_kernel.
+  int nz;
+  int full_tiles;
+  int tail_split;   // 1: no tile is split
+  int kchunk;       // a multiple of 16
+  float *partial;   // [tail tile][chunk][BM][BN]
   int fast;         // every operand spans less than 2 GiB: descriptor loads allowed
+  int a_bytes;      // fast: bytes of one z of A / of B (conv: of X from the first byte
+  int b_bytes;      //       of a group to the end of the tensor, plus the padding shift)
   ConvGeom cv;
 };
 
@@ -123,24 +148,26 @@ __device__ __forceinline__ float relu_js(float v) {
   return v > 0.0f ? v : (v != v ? v : 0.0f);
 }
 
-// Maps the linear workgroup id to a tile so that (1) each XCD (ids are dealt
-// round-robin over the 8 XCDs) works on a contiguous range of tiles and
-// (2) within that range tiles are visited in groups of 8 tile-rows, which
-// keeps the A and B panels a group touches resident in that XCD's L2.
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
-                                              int *tm, int *tn) {
-  const int total = tiles_m * tiles_n;
+// Whole-tile workgroups: ids are dealt round-robin over the 8 XCDs by the
+// hardware; this gives each XCD a contiguous range of tile numbers, so that
+// tiles sharing A and B panels meet in one L2.
+__device__ __forceinline__ int xcd_contiguous(int pid, int total) {
   constexpr int XCDS = 8;
-  int xcd = pid % XCDS, local = pid / XCDS;
-  int base = total / XCDS, rem = total % XCDS;
-  int start = xcd * base + (xcd < rem ? xcd : rem);
-  int id = start + local;
+  const int xcd = pid % XCDS, local = pid / XCDS;
+  const int base = total / XCDS, rem = total % XCDS;
+  return xcd * base + (xcd < rem ? xcd : rem) + local;
+}
+
+// Tile number within one z -> tile coordinates, visiting tiles in groups of 8
+// tile-rows so that the panels a group touches stay resident in L2.
+__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n,
+                                            int *tm, int *tn) {
   constexpr int GROUP = 8;
-  int per_group = GROUP * tiles_n;
-  int group = id / per_group;
-  int first_m = group * GROUP;
-  int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
-  int in_group = id % per_group;
+  const int per_group = GROUP * tiles_n;
+  const int group = id / per_group;
+  const int first_m = group * GROUP;
+  const int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
+  const int in_group = id % per_group;
   *tm = first_m + in_group % rows;
   *tn = in_group / rows;
 }
@@ -350,10 +377,22 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   const int li = lane & 31, half = lane >> 5;
   const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
 
+  // which tile, and which part of K
+  const int pid = blockIdx.x;
+  const bool whole = pid < p.full_tiles;
+  int lin, chunk = 0;
+  if (whole) {
+    lin = xcd_contiguous(pid, p.full_tiles);
+  } else {
+    const int c = pid - p.full_tiles;
+    lin = p.full_tiles + c / p.tail_split;
+    chunk = c % p.tail_split;
+  }
+  const int tiles_per_z = p.tiles_m * p.tiles_n;
+  const int bz = lin / tiles_per_z;  // batch entry (gemm) or group (conv)
   int tm, tn;
-  tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, &tm, &tn);
+  tile_coords(lin - bz * tiles_per_z, p.tiles_m, p.tiles_n, &tm, &tn);
   const int row0 = tm * BM, col0 = tn * BN;
-  const int bz = blockIdx.y;  // batch (gemm) or group (conv)
 
   const float *A = p.A + (long long)bz * p.sAb;
   const float *B = p.B + (long long)bz * p.sBb;
@@ -361,8 +400,8 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   const long long ldb = B_IS_KC ? p.sB1 : p.sB0;
 
   // this workgroup's share of K
-  const int kbeg = p.ksplit > 1 ? (int)blockIdx.z * p.kchunk : 0;
-  const int kend = p.ksplit > 1 ? (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k) : p.k;
+  const int kbeg = whole ? 0 : chunk * p.kchunk;
+  const int kend = whole ? p.k : (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k);
 
   // ---- descriptor fetch plans: one byte offset per 16-byte piece -------------
   // A row-major-in-K operand may always take this path (rows past the edge are
@@ -397,35 +436,37 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     for (int i = 0; i < BN / 64; i++)
       voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + col0 + (tid % TPR) * 4) * 4);
   }
-  const rsrc_t rsrc_a = make_rsrc(A);
+  const rsrc_t rsrc_a = make_rsrc(A, p.a_bytes);
 
   // ---- im2col: what this thread's pixel looks like ----------------------------
   PixelCtx px = {p.B, 0, 0, 0, 0ull};
   PixelFast pf = {0, 0xffffffffu, 0xffffffffu};
   const float *bbase = B;  // base of the B descriptor
   if (IM2COL) {
-    const long long P = (long long)col0 + (tid % BN);
+    const unsigned P = (unsigned)col0 + (unsigned)(tid % BN);  // npix < 2^31
     const long long plane = (long long)p.cv.h * p.cv.w;
     const int bias = p.cv.pt * p.cv.w + p.cv.pl;  // makes every corner offset >= 0
     px.xbase = p.B + (long long)bz * p.cv.c_in_g * plane;
     bbase = px.xbase - bias;
-    if (P < p.cv.npix) {
-      const int ohw = p.cv.oh * p.cv.ow;
-      const int img = (int)(P / ohw);
-      const int q = (int)(P - (long long)img * ohw);
-      const int oy = q / p.cv.ow, ox = q - oy * p.cv.ow;
+    if (P < (unsigned)p.cv.npix) {
+      const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+      const unsigned img = P / ohw;
+      const unsigned q = P - img * ohw;
+      const int oy = (int)(q / (unsigned)p.cv.ow), ox = (int)q - oy * p.cv.ow;
       const long long img_off = (long long)img * p.cv.c_total * plane;
       px.iy0 = oy * p.cv.sh - p.cv.pt;
       px.ix0 = ox * p.cv.sw - p.cv.pl;
       px.pbase = px.iy0 * p.cv.w + px.ix0;
       if (IM2COL_FAST) {
         pf.valid = (int)((img_off + px.pbase + bias) * 4);
+        // which taps of this pixel fall inside the input: rows first, then columns
         unsigned long long inside = 0;
-        for (int t = 0; t < p.cv.ntaps; t++) {
-          const int d = p.cv.taptab[t];
-          const int iy = px.iy0 + (d >> 16), ix = px.ix0 + (d & 0xffff);
-          if ((unsigned)iy < (unsigned)p.cv.h && (unsigned)ix < (unsigned)p.cv.w)
-            inside |= 1ull << t;
+        int t = 0;
+        for (int ky = 0; ky < p.cv.kh; ky++) {
+          const bool row_in = (unsigned)(px.iy0 + ky * p.cv.dh) < (unsigned)p.cv.h;
+          for (int kx = 0; kx < p.cv.kw; kx++, t++)
+            if (row_in && (unsigned)(px.ix0 + kx * p.cv.dw) < (unsigned)p.cv.w)
+              inside |= 1ull << t;
         }
         pf.pad_lo = ~(unsigned)inside;
         pf.pad_hi = ~(unsigned)(inside >> 32);
@@ -435,7 +476,10 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
       }
     }
   }
-  const rsrc_t rsrc_b = make_rsrc(bbase);
+  // conv: p.b_bytes is group 0's window, later groups start further into X
+  const int b_window =
+      IM2COL ? p.b_bytes - (int)((long long)bz * p.cv.c_in_g * p.cv.h * p.cv.w * 4) : p.b_bytes;
+  const rsrc_t rsrc_b = make_rsrc(bbase, b_window);
   // first of the L consecutive k rows this wavefront gathers in each slab
   const int kgroup0 = IM2COL ? __builtin_amdgcn_readfirstlane(tid / BN) * (BK / (NTHREADS / BN)) : 0;
 
@@ -553,12 +597,16 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   stash(0, st0);
   __syncthreads();
   int s = 0;
+  // The scheduling fences keep the compiler from sinking the loads below the
+  // matrix-core work they are meant to overlap.
   for (; s + 2 <= nfast; s += 2) {
     fetch_fast(kbeg + (s + 1) * BK, st0);
+    __builtin_amdgcn_sched_barrier(0);
     compute(0);
     stash(1, st0);
     __syncthreads();
     fetch_fast(kbeg + (s + 2) * BK, st0);
+    __builtin_amdgcn_sched_barrier(0);
     compute(1);
     stash(0, st0);
     __syncthreads();
@@ -573,57 +621,75 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
 
   // ---- epilogue: lane holds column (li) of each 32x32 tile, rows
   // 8*(r/4) + 4*half + r%4 for accumulator register r.
-  if (p.ksplit > 1) {
-    // raw partial sums in plain [z][y][m][n] order; splitk_reduce_kernel adds
-    // the chunks in index order and applies the epilogue
-    float *part = p.partial + ((long long)blockIdx.z * gridDim.y + bz) * p.m * p.n;
+  if (!whole) {
+    // raw sums of the whole tile (edge rows and columns included), tile-local
+    float *part = p.partial +
+                  ((long long)(lin - p.full_tiles) * p.tail_split + chunk) * (BM * BN);
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const int col = col0 + wcol + nt * 32 + li;
-      if (col >= p.n) continue;
+    for (int nt = 0; nt < NT; nt++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const int row = row0 + wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          if (row < p.m) part[(long long)row * p.n + col] = acc[mt][nt][r];
+          const int lr = wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          part[lr * BN + wcol + nt * 32 + li] = acc[mt][nt][r];
         }
-    }
     return;
   }
+  // Bias and residual values of a 32x32 block are all requested before the
+  // first is used, so the block pays one memory round trip, not thirty-two.
+  // Loads use clamped indices (always inside the tensors); only the store is
+  // conditional.
 #pragma unroll
   for (int nt = 0; nt < NT; nt++) {
     const int col = col0 + wcol + nt * 32 + li;
-    if (col >= p.n) continue;
+    const bool col_ok = col < p.n;
+    const int colc = col_ok ? col : p.n - 1;
     long long ybase;     // offset of (row 0, this column) in Y
     long long ystride;   // distance between consecutive rows in Y
     if (IM2COL) {
-      const int ohw = p.cv.oh * p.cv.ow;
-      const int img = col / ohw;
-      const int q = col - img * ohw;
+      const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+      const unsigned img = (unsigned)colc / ohw;
+      const unsigned q = (unsigned)colc - img * ohw;
       ybase = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g) * ohw + q;
       ystride = ohw;
     } else {
-      ybase = (long long)bz * p.m * p.n + col;
+      ybase = (long long)bz * p.m * p.n + colc;
       ystride = p.n;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
+      const int rfirst = row0 + wrow + mt * 32 + 4 * half;
+      // eight rows at a time keeps the 64-register tiles from spilling
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int row = row0 + wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (row >= p.m) continue;
-        float y = p.alpha * acc[mt][nt][r];
+      for (int hb = 0; hb < 2; hb++) {
+        float cv[8], rv[8];
         if (p.C) {
-          float c = IM2COL
-                        ? p.C[bz * p.cv.cout_g + row]
-                        : p.C[(long long)row * p.sC0 + (long long)col * p.sC1];
-          y = __builtin_fmaf(c, p.beta, y);
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+            row = row < p.m ? row : p.m - 1;
+            cv[j] = IM2COL ? p.C[bz * p.cv.cout_g + row]
+                           : p.C[(long long)row * p.sC0 + (long long)colc * p.sC1];
+          }
         }
-        const long long off = ybase + (long long)row * ystride;
-        if (p.R) y = y + p.R[off];
-        if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
-        p.Y[off] = y;
+        if (p.R) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+            row = row < p.m ? row : p.m - 1;
+            rv[j] = p.R[ybase + (long long)row * ystride];
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+          float y = p.alpha * acc[mt][nt][8 * hb + j];
+          if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+          if (p.R) y = y + rv[j];
+          if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+          if (col_ok && row < p.m) p.Y[ybase + (long long)row * ystride] = y;
+        }
       }
     }
   }
@@ -650,21 +716,30 @@ __global__ void contraction_strided_kernel(Params p) {
   p.Y[off] = y;
 }
 
-// Second pass of a split-K contraction: adds the ksplit partial sums of each
-// result element in chunk order (so the result does not depend on scheduling)
-// and applies the same epilogue as the single-pass kernel.
+// Second pass for the tail tiles: adds the chunks of each tile in index order
+// (so the result does not depend on scheduling) and applies the epilogue.
+// grid = (tail tiles, bm*bn/1024), 256 threads, 4 consecutive columns each.
 template <bool CONV>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int nz) {
-  const long long per_z = (long long)p.m * p.n;
-  const long long total = per_z * nz;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-    const int bz = (int)(i / per_z);
-    const long long rc = i - (long long)bz * per_z;
-    const int row = (int)(rc / p.n), col = (int)(rc - (long long)row * p.n);
-    float acc = 0.0f;
-    for (int s = 0; s < p.ksplit; s++) acc += p.partial[(long long)s * total + i];
-    float y = p.alpha * acc;
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int bm, int bn) {
+  const int j = blockIdx.x;
+  const int lin = p.full_tiles + j;
+  const int tiles_per_z = p.tiles_m * p.tiles_n;
+  const int bz = lin / tiles_per_z;
+  int tm, tn;
+  tile_coords(lin - bz * tiles_per_z, p.tiles_m, p.tiles_n, &tm, &tn);
+  const int e = ((int)blockIdx.y * 256 + (int)threadIdx.x) * 4;
+  const int lr = e / bn, lc = e - lr * bn;
+  const int row = tm * bm + lr;
+  if (row >= p.m) return;
+  const float *part = p.partial + (long long)j * p.tail_split * (bm * bn) + e;
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int c = 0; c < p.tail_split; c++)
+    acc += *reinterpret_cast<const f32x4 *>(part + (long long)c * (bm * bn));
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int col = tn * bn + lc + i;
+    if (col >= p.n) break;
+    float y = p.alpha * acc[i];
     long long off;
     if (CONV) {
       const int ohw = p.cv.oh * p.cv.ow;
@@ -672,7 +747,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int nz) {
       off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
       if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
     } else {
-      off = i;
+      off = ((long long)bz * p.m + row) * p.n + col;
       if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
     }
     if (p.R) y = y + p.R[off];
@@ -713,44 +788,103 @@ TileId pick_tile(int m, int n, int nz) {
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
 
-// When even the smallest tile leaves the chip short of work (few result
-// elements, long K: ResNet stage-3/4 convs at 14x14 and 7x7), K is cut into
-// chunks that run as separate workgroups.
-int pick_split(long long tiles, int k) {
+// How the tiles of one launch are spread over the chip.
+struct WorkPlan {
+  long long full;   // tiles computed by one workgroup each
+  long long tail;   // tiles cut along K
+  int split;        // chunks per tail tile
+  int kchunk;       // K elements per chunk (a multiple of 16)
+};
+
+// A launch keeps every CU busy for ceil(tiles / CUs) tile times, so a tile count
+// just above a multiple of the CU count wastes most of a round, and a CU that
+// holds only one or two workgroups cannot hide their latencies.  Candidate
+// plans -- nothing split, only the tiles beyond the last full round split, or
+// every tile split -- are compared with a small model in microseconds: a CU
+// works through its workgroups' K slabs at slab_us each, but never finishes
+// sooner than `solo` times the longest single workgroup (the slow-down of a
+// workgroup that runs alone on a CU); every workgroup adds a start-up/epilogue
+// cost and a split adds the reduce pass over the partial sums.
+WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
+  const long long cus = wdh::compute_units();
+  const int slabs = (k + BK - 1) / BK;
+  WorkPlan w = {tiles, 0, 1, 0};
+  auto with_split = [&](long long tail, int s) {
+    WorkPlan r;
+    r.kchunk = ((slabs + s - 1) / s) * BK;
+    r.split = (k + r.kchunk - 1) / r.kchunk;
+    if (r.split < 1) r.split = 1;
+    r.tail = r.split > 1 ? tail : 0;
+    r.full = tiles - r.tail;
+    return r;
+  };
   if (g_forced_split >= 1) {
-    int s = g_forced_split;
-    int max_s = (k + BK - 1) / BK;
-    return s < max_s ? s : (max_s > 0 ? max_s : 1);
+    // tuning / test hook: every tile is split this many ways
+    const int s = g_forced_split < slabs ? g_forced_split : (slabs > 0 ? slabs : 1);
+    return s > 1 ? with_split(tiles, s) : w;
   }
-  const long long target = 4LL * wdh::compute_units();
-  if (tiles * 2 >= target) return 1;
-  long long s = (target + tiles - 1) / tiles;
-  const long long max_s = k / (4 * BK);  // keep at least 4 slabs per chunk
-  if (s > max_s) s = max_s;
-  if (s > 32) s = 32;
-  return s < 2 ? 1 : (int)s;
+  if (slabs < 8) return w;
+  const double area = (double)bm * bn / (64.0 * 64.0);
+  const double slab_us = 0.30 * area;
+  const double start_us = 0.9 * (area > 1.0 ? 2.0 : 1.0);
+  const double solo = 2.5;
+  const double tile_bytes = (double)bm * bn * 4.0;
+  auto cost = [&](long long tail, int s) {
+    const long long full_rounds = (tiles - tail) / cus;  // tiles - tail is a multiple of cus or 0
+    const long long tail_rounds = (tail * s + cus - 1) / cus;
+    const double chunk_us = (double)slabs / s * slab_us + start_us;
+    const double whole_us = slabs * slab_us + start_us;
+    const double work = full_rounds * whole_us + tail_rounds * chunk_us;
+    const double longest = full_rounds > 0 ? whole_us : chunk_us;
+    double t = work > solo * longest ? work : solo * longest;
+    // reduce pass: a launch plus the partial sums written and read back (mostly
+    // through the last-level cache, ~8 TB/s)
+    if (s > 1) t += 3.0 + 2.0 * tail * s * tile_bytes / 8.0e6;
+    return t;
+  };
+  const long long rem = tiles % cus;
+  const int max_s = slabs / 4 < 32 ? slabs / 4 : 32;  // at least 4 slabs per chunk
+  double best;
+  // unsplit: the remainder tiles make one more (partial) round of whole tiles
+  {
+    const long long rounds = (tiles + cus - 1) / cus;
+    const double whole_us = slabs * slab_us + start_us;
+    const double work = rounds * whole_us;
+    best = work > solo * whole_us ? work : solo * whole_us;
+  }
+  long long best_tail = 0;
+  int best_s = 1;
+  for (int s = 2; s <= max_s; s++) {
+    if (rem) {
+      const double c = cost(rem, s);
+      if (c < best) { best = c; best_tail = rem; best_s = s; }
+    }
+    const double c = cost(tiles, s);
+    if (c < best) { best = c; best_tail = tiles; best_s = s; }
+  }
+  return best_s > 1 ? with_split(best_tail, best_s) : w;
 }
 
 template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE>
 int launch_tile(Params &p, int nz, bool vec) {
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
-  const long long tiles = (long long)p.tiles_m * p.tiles_n;
-  int split = pick_split(tiles * nz, p.k);
+  const long long tiles = (long long)p.tiles_m * p.tiles_n * nz;
+  const WorkPlan w = plan_work(tiles, p.k, BM, BN);
+  const long long blocks = w.full + w.tail * w.split;
+  if (blocks > 0x7fffffffLL)
+    return wdh::fail(WDH_EINVAL, "contraction: %lld workgroups exceed the grid limit", blocks);
+  p.nz = nz;
+  p.full_tiles = (int)w.full;
+  p.tail_split = w.split;
+  p.kchunk = w.kchunk;
   wdh_buf scratch = 0;
-  p.ksplit = 1;
-  if (split > 1) {
-    p.kchunk = ((p.k + split - 1) / split + BK - 1) / BK * BK;
-    split = (p.k + p.kchunk - 1) / p.kchunk;
-  }
-  if (split > 1) {
-    const size_t bytes = (size_t)split * nz * p.m * p.n * sizeof(float);
-    scratch = wdh_alloc(bytes);
+  if (w.tail > 0) {
+    scratch = wdh_alloc((size_t)w.tail * w.split * BM * BN * sizeof(float));
     if (!scratch) return WDH_ENOMEM;
     p.partial = (float *)wdh::resolve(scratch, nullptr);
-    p.ksplit = split;
   }
-  dim3 grid((unsigned)tiles, (unsigned)nz, (unsigned)p.ksplit);
+  dim3 grid((unsigned)blocks);
   if (vec)
     hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, true>), grid,
                        dim3(NTHREADS), 0, wdh::stream(), p);
@@ -758,17 +892,14 @@ int launch_tile(Params &p, int nz, bool vec) {
     hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, false>), grid,
                        dim3(NTHREADS), 0, wdh::stream(), p);
   hipError_t e = hipGetLastError();
-  if (e == hipSuccess && p.ksplit > 1) {
-    const long long total = (long long)p.m * p.n * nz;
-    long long blocks = (total + 255) / 256;
-    const long long cap = 16LL * wdh::compute_units();
-    if (blocks > cap) blocks = cap;
+  if (e == hipSuccess && w.tail > 0) {
+    dim3 rgrid((unsigned)w.tail, (unsigned)(BM * BN / 1024));
     if (BMODE >= B_IM2COL32)
-      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)blocks), dim3(256), 0,
-                         wdh::stream(), p, nz);
+      hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, wdh::stream(), p,
+                         BM, BN);
     else
-      hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)blocks), dim3(256), 0,
-                         wdh::stream(), p, nz);
+      hipLaunchKernelGGL(splitk_reduce_kernel<false>, rgrid, dim3(256), 0, wdh::stream(), p,
+                         BM, BN);
     e = hipGetLastError();
   }
   // The scratch block goes back to the pool right away: whoever gets it next
@@ -898,8 +1029,11 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
                    vec_ok(p.B, useB_kc ? p.sB1 : p.sB0, sBb);
   // Descriptor loads address one batch entry with 32-bit byte offsets (a
   // clamped edge row plus a 16-byte piece may reach 12 bytes past the span).
-  p.fast = (span(1, 0, m, p.sA0, k, p.sA1) + 4) * 4 < 0x7fffffffLL &&
-           (span(1, 0, k, p.sB0, n, p.sB1) + 4) * 4 < 0x7fffffffLL;
+  const long long a_bytes = k ? span(1, 0, m, p.sA0, k, p.sA1) * 4 : 0;
+  const long long b_bytes = k ? span(1, 0, k, p.sB0, n, p.sB1) * 4 : 0;
+  p.fast = a_bytes < 0x7fffffffLL && b_bytes < 0x7fffffffLL;
+  p.a_bytes = p.fast ? (int)a_bytes : 0;
+  p.b_bytes = p.fast ? (int)b_bytes : 0;
   if (useA_kc && useB_kc) return launch<true, B_KC>(p, batch, vec);
   if (useA_kc && !useB_kc) return launch<true, B_MC>(p, batch, vec);
   if (!useA_kc && useB_kc) return launch<false, B_KC>(p, batch, vec);
@@ -920,7 +1054,6 @@ struct KtabKey {
 };
 struct KtabVal {
   int2 *ktab;
-  int *taptab;
 };
 
 std::map<KtabKey, KtabVal> g_ktabs;
@@ -931,7 +1064,6 @@ namespace wdh {
 void release_conv_tables() {
   for (auto &kv : g_ktabs) {
     (void)hipFree(kv.second.ktab);
-    (void)hipFree(kv.second.taptab);
   }
   g_ktabs.clear();
 }
@@ -1005,7 +1137,6 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     const int pad_tap = mode == B_IM2COL32 ? 31 : 63;
     std::vector<int2> tab((size_t)((kdim + BK - 1) / BK * BK),
                           mode == B_IM2COL_BIG ? int2{0, 0} : int2{0, pad_tap});
-    std::vector<int> taps((size_t)ntaps);
     size_t idx = 0;
     for (int ci = 0; ci < c_in_g; ci++)
       for (int ky = 0; ky < kh; ky++)
@@ -1019,20 +1150,15 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
             tab[idx].x = off * 4;
             tab[idx].y = ky * kw + kx;
           }
-          taps[ky * kw + kx] = packed;
           idx++;
         }
-    KtabVal val = {nullptr, nullptr};
-    if (hipMalloc(&val.ktab, tab.size() * sizeof(int2)) != hipSuccess ||
-        hipMalloc(&val.taptab, taps.size() * sizeof(int)) != hipSuccess) {
+    KtabVal val = {nullptr};
+    if (hipMalloc(&val.ktab, tab.size() * sizeof(int2)) != hipSuccess) {
       (void)hipGetLastError();
-      if (val.ktab) (void)hipFree(val.ktab);
       return fail(WDH_ENOMEM, "wdh_conv2d: tap table allocation failed");
     }
-    // synchronous copies: the host vectors die at the end of this scope
+    // synchronous copy: the host vector dies at the end of this scope
     WDH_HIP_CHECK(hipMemcpy(val.ktab, tab.data(), tab.size() * sizeof(int2),
-                            hipMemcpyHostToDevice));
-    WDH_HIP_CHECK(hipMemcpy(val.taptab, taps.data(), taps.size() * sizeof(int),
                             hipMemcpyHostToDevice));
     it = g_ktabs.emplace(key, val).first;
   }
@@ -1045,9 +1171,13 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.pt = pt; p.cv.pl = pl; p.cv.sh = sh; p.cv.sw = sw;
   p.cv.c_total = c; p.cv.cout_total = cout; p.cv.cout_g = cout_g;
   p.cv.ntaps = ntaps;
-  p.cv.npix = npix; p.cv.ktab = it->second.ktab; p.cv.taptab = it->second.taptab;
+  p.cv.npix = npix; p.cv.ktab = it->second.ktab;
+  p.cv.kh = kh; p.cv.kw = kw; p.cv.dh = dh; p.cv.dw = dw;
   const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
   p.fast = small ? 1 : 0;
+  p.a_bytes = small ? (int)w_bytes : 0;
+  // a group's window runs from its first byte (shifted down by the padding) to the end of X
+  p.b_bytes = small ? (int)x_bytes : 0;  // window of group 0; the kernel shortens it per group
   if (mode == B_IM2COL32) return launch<true, B_IM2COL32>(p, group, vec);
   if (mode == B_IM2COL64) return launch<true, B_IM2COL64>(p, group, vec);
   return launch<true, B_IM2COL_BIG>(p, group, vec);
