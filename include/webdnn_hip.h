@@ -176,6 +176,11 @@ int wdh_binary(int op, int dtype, wdh_buf L, wdh_buf R, wdh_buf Y, int ndim,
 #define WDH_UN_NEG 6
 #define WDH_UN_RECIPROCAL 7
 int wdh_unary(int op, int dtype, wdh_buf X, wdh_buf Y, size_t length);
+/* Replaces Cast (operators/cpu/operators/standard/cast.ts:12-52): dtypes are
+ * 0 = float32, 1 = int32 (the runner's two; ONNX INT64/UINT8 arrive as int32).
+ * float32 -> int32 applies ToInt32 (what `Int32Array.set` does: truncate, wrap
+ * modulo 2^32, NaN and infinities give 0); int32 -> float32 rounds to nearest. */
+int wdh_cast(int from_dtype, int to_dtype, wdh_buf X, wdh_buf Y, size_t length);
 
 /* ---- row reductions ----------------------------------------------------
  * Softmax over the last axis: X viewed as [outer, len]; replaces
@@ -214,6 +219,16 @@ int wdh_transpose(wdh_buf X, wdh_buf Y, int ndim, const int32_t *out_shape,
  * indices[n_idx] (negative indices wrap once) -> Y [outer, n_idx, inner]. */
 int wdh_gather(wdh_buf Data, wdh_buf Indices, wdh_buf Y, int64_t outer,
                int axis_len, int64_t inner, int64_t n_idx);
+/* Replaces the copy loops of Slice10.copy1d..copy6d
+ * (operators/cpu/operators/standard/slice.ts:96-330), Concat.run
+ * (concat.ts:21-84) and CPUSplit2/13.run (split.ts:12-87), which are all
+ *   Y[y_offset + sum_i idx_i * y_strides[i]] = X[x_offset + sum_i idx_i * x_strides[i]]
+ * for idx over `shape` (ndim <= 6, 4-byte elements of either dtype, offsets and
+ * strides in elements).  x_strides may be negative (Slice with a negative
+ * step); the whole view must lie inside both buffers. */
+int wdh_strided_copy(wdh_buf X, int64_t x_offset, wdh_buf Y, int64_t y_offset,
+                     int ndim, const int32_t *shape, const int64_t *x_strides,
+                     const int64_t *y_strides);
 
 #ifdef __cplusplus
 }

@@ -1,7 +1,7 @@
 "use strict";
 /*
  * TEST INFRASTRUCTURE ONLY — JavaScript restatement of the WebDNN reference CPU
- * operators on the Gemm/MatMul/Conv hot path, behind the reference's own
+ * operators on the Gemm/MatMul/Conv hot path and the layout glue around it, behind the reference's own
  * Operator / OperatorEntry interface, so that a model can be run with
  * backendOrder ["cpu"] through the same runner and compared with ["hip"].
  *
@@ -517,6 +517,181 @@ class RefReduceMean extends OperatorImpl {
   }
 }
 
+// ---- Squeeze / Unsqueeze: operators/base/squeeze.ts:7-43, base/unsqueeze.ts:7-47; the cpu
+// operators share the input buffer (cpu/operators/standard/squeeze.ts:12-37, unsqueeze.ts)
+class RefSqueeze extends OperatorImpl {
+  constructor(axesFromInput) {
+    super("cpu");
+    this.axesFromInput = axesFromInput;
+  }
+  initialize(attribute) {
+    this.axes = this.axesFromInput ? null : getAttrInts(attribute, "axes", []);
+  }
+  async run(context, inputs) {
+    context.assertsCPUTensorArray(inputs);
+    const input = inputs[0];
+    const axes = this.axesFromInput ? (inputs[1] ? Array.from(inputs[1].data) : []) : this.axes;
+    let shape;
+    if (axes.length === 0) shape = input.dims.filter((s) => s !== 1);
+    else {
+      const nn = axes.map((a) => (a >= 0 ? a : a + input.dims.length));
+      shape = input.dims.filter((_, i) => !nn.includes(i));
+    }
+    return [context.emptyTensor(shape, input.dataType, input.data)];
+  }
+}
+
+class RefUnsqueeze extends OperatorImpl {
+  constructor(axesFromInput) {
+    super("cpu");
+    this.axesFromInput = axesFromInput;
+  }
+  initialize(attribute) {
+    this.axes = this.axesFromInput ? null : getAttrInts(attribute, "axes", []);
+  }
+  async run(context, inputs) {
+    context.assertsCPUTensorArray(inputs);
+    const input = inputs[0];
+    const axes = this.axesFromInput ? Array.from(inputs[1].data) : this.axes;
+    const nd = input.dims.length + axes.length, nn = axes.map((a) => (a >= 0 ? a : a + nd)), shape = [];
+    let src = 0;
+    for (let d = 0; d < nd; d++) shape.push(nn.includes(d) ? 1 : input.dims[src++]);
+    return [context.emptyTensor(shape, input.dataType, input.data)];
+  }
+}
+
+// ---- Concat: operators/cpu/operators/standard/concat.ts:9-84
+class RefConcat extends OperatorImpl {
+  constructor() {
+    super("cpu");
+  }
+  initialize(attribute) {
+    this.axis = getAttrInt(attribute, "axis", 0);
+  }
+  async run(context, inputs) {
+    context.assertsCPUTensorArray(inputs);
+    const axis = this.axis >= 0 ? this.axis : inputs[0].ndim + this.axis;
+    if (axis < 0 || axis >= inputs[0].ndim) throw new Error(`Concat: axis ${axis} out of range`);
+    let axisLength = 0;
+    const parts = [];
+    for (const it of inputs) {
+      const st = strides(it.dims);
+      parts.push([it, axisLength, it.dims[axis], st[Math.max(axis - 1, 0)], st[axis]]);
+      axisLength += it.dims[axis];
+    }
+    const outShape = inputs[0].dims.slice();
+    outShape[axis] = axisLength;
+    const outerLength = prod(inputs[0].dims.slice(0, axis)), innerLength = prod(inputs[0].dims.slice(axis + 1));
+    const output = context.emptyTensor(outShape, inputs[0].dataType), so = strides(outShape);
+    const outOuter = so[Math.max(axis - 1, 0)], outCat = so[axis];
+    for (const [it, off, dim, outerS, catS] of parts) {
+      for (let c = 0; c < dim; c++) for (let o = 0; o < outerLength; o++) for (let i = 0; i < innerLength; i++) {
+        output.data[(c + off) * outCat + o * outOuter + i] = it.data[c * catS + o * outerS + i];
+      }
+    }
+    return [output];
+  }
+}
+
+// ---- Split: operators/base/split.ts:7-102, operators/cpu/operators/standard/split.ts:7-87
+class RefSplit extends OperatorImpl {
+  constructor(splitFromInput) {
+    super("cpu");
+    this.splitFromInput = splitFromInput;
+  }
+  initialize(attribute) {
+    this.axis = getAttrInt(attribute, "axis", 0);
+    this.split = this.splitFromInput ? null : getAttrInts(attribute, "split", []);
+  }
+  async run(context, inputs, nOutputs) {
+    context.assertsCPUTensorArray(inputs);
+    const input = inputs[0];
+    const splitSrc = this.splitFromInput ? (inputs[1] ? Array.from(inputs[1].data) : []) : this.split;
+    let axis = this.axis;
+    if (axis < 0) axis += input.ndim;
+    if (axis < 0 || axis >= input.ndim) throw new Error(`Split: axis ${axis} out of range`);
+    const axisLength = input.dims[axis];
+    const split = splitSrc.length > 0 ? splitSrc : Array.from({ length: nOutputs }, () => Math.floor(axisLength / nOutputs));
+    const outerLength = prod(input.dims.slice(0, axis)), innerLength = prod(input.dims.slice(axis + 1));
+    const si = strides(input.dims), inOuter = si[Math.max(axis - 1, 0)], inCat = si[axis];
+    const outputs = [];
+    let offset = 0;
+    for (let n = 0; n < nOutputs; n++) {
+      const dim = split[n], outShape = input.dims.slice();
+      outShape[axis] = dim;
+      const outerS = prod(outShape.slice(Math.max(axis - 1, 0) + 1)), splitS = prod(outShape.slice(axis + 1));
+      const ot = context.emptyTensor(outShape, input.dataType);
+      for (let c = 0; c < dim; c++) for (let o = 0; o < outerLength; o++) for (let i = 0; i < innerLength; i++) {
+        ot.data[c * splitS + o * outerS + i] = input.data[(c + offset) * inCat + o * inOuter + i];
+      }
+      outputs.push(ot);
+      offset += dim;
+    }
+    return outputs;
+  }
+}
+
+// ---- Slice (opset >= 10): operators/cpu/operators/standard/slice.ts:12-330; copy1d..copy6d
+// are one loop nest here
+class RefSlice10 extends OperatorImpl {
+  constructor() {
+    super("cpu");
+  }
+  async run(context, inputs) {
+    context.assertsCPUTensorArray(inputs);
+    const [data, starts, ends, axesTensor, stepsTensor] = inputs;
+    if (data.ndim > 6) throw new Error(`Slice: input dimension ${data.ndim} > 6 is not yet supported`);
+    const axes = axesTensor ? Array.from(axesTensor.data).map((a) => (a < 0 ? a + data.ndim : a)) : data.dims.map((_, i) => i);
+    const steps = stepsTensor ? Array.from(stepsTensor.data) : axes.map(() => 1);
+    const ranges = data.dims.map((d) => [0, d, 1, d]);
+    for (let i = 0; i < axes.length; i++) ranges[axes[i]] = [starts.data[i], ends.data[i], steps[i], data.dims[axes[i]]];
+    const rws = ranges.map(([start, stop, step, srcsize]) => {
+      if (start < 0) start += srcsize;
+      start = Math.max(Math.min(start, srcsize - 1), 0);
+      if (stop < 0) stop += srcsize;
+      stop = Math.max(Math.min(stop, srcsize), -1);
+      return [start, stop, step, srcsize, Math.max(Math.ceil((stop - start) / step), 0)];
+    });
+    const outShape = rws.map((r) => r[4]), output = context.emptyTensor(outShape, data.dataType);
+    const ss = strides(data.dims), ds = strides(outShape), nd = data.ndim, idx = new Array(nd).fill(0);
+    const total = prod(outShape);
+    for (let n = 0; n < total; n++) {
+      let src = 0, dst = 0;
+      for (let d = 0; d < nd; d++) {
+        src += (rws[d][0] + idx[d] * rws[d][2]) * ss[d];
+        dst += idx[d] * ds[d];
+      }
+      output.data[dst] = data.data[src];
+      for (let d = nd - 1; d >= 0; d--) {
+        if (++idx[d] < outShape[d]) break;
+        idx[d] = 0;
+      }
+    }
+    return [output];
+  }
+}
+
+// ---- Cast: operators/cpu/operators/standard/cast.ts:12-52 (typed-array `set` does the conversion)
+class RefCast extends OperatorImpl {
+  constructor() {
+    super("cpu");
+  }
+  initialize(attribute) {
+    this.to = getAttrInt(attribute, "to", 1);
+  }
+  async run(context, inputs) {
+    context.assertsCPUTensorArray(inputs);
+    const input = inputs[0];
+    let dt;
+    if (this.to === 1) dt = "float32";
+    else if (this.to === 2 || this.to === 6 || this.to === 7) dt = "int32";
+    else throw new Error(`Cast: converting to DataType ${this.to} is not yet supported`);
+    const newData = dt === "float32" ? new Float32Array(input.data.length) : new Int32Array(input.data.length);
+    newData.set(input.data);
+    return [context.emptyTensor(input.dims, dt, newData)];
+  }
+}
+
 function getOpEntries() {
   const fi = ["float32", "int32"], f = ["float32"];
   const e = (opType, opsetMin, factory) => ({ opType, backend: "cpu", opsetMin, factory });
@@ -545,6 +720,15 @@ function getOpEntries() {
     e("Reshape", 5, () => new RefReshape5()),
     e("Gather", 1, () => new RefGather()),
     e("ReduceMean", 1, () => new RefReduceMean()),
+    { opType: "Squeeze", backend: "cpu", opsetMin: 13, factory: () => new RefSqueeze(true) },
+    { opType: "Squeeze", backend: "cpu", opsetMin: 1, opsetMax: 13, factory: () => new RefSqueeze(false) },
+    { opType: "Unsqueeze", backend: "cpu", opsetMin: 13, factory: () => new RefUnsqueeze(true) },
+    { opType: "Unsqueeze", backend: "cpu", opsetMin: 1, opsetMax: 13, factory: () => new RefUnsqueeze(false) },
+    e("Concat", 1, () => new RefConcat()),
+    { opType: "Split", backend: "cpu", opsetMin: 13, factory: () => new RefSplit(true) },
+    { opType: "Split", backend: "cpu", opsetMin: 1, opsetMax: 13, factory: () => new RefSplit(false) },
+    e("Slice", 10, () => new RefSlice10()),
+    e("Cast", 6, () => new RefCast()),
   ];
 }
 

@@ -280,3 +280,161 @@ def reshape(X, shape, allowzero=0):
         else:
             out.append(X.size // explicit)
     return X.reshape(out)
+
+
+# ---- layout glue: pure index arithmetic, restated in numpy/python ------------------
+
+def squeeze(X, axes=()):
+    """operators/base/squeeze.ts:8-22 (+ cpu squeeze.ts:12-37: shares the buffer)."""
+    X = np.asarray(X)
+    axes = [int(a) for a in axes]
+    if not axes:
+        shape = [s for s in X.shape if s != 1]
+    else:
+        nn = [a if a >= 0 else a + X.ndim for a in axes]
+        shape = [s for i, s in enumerate(X.shape) if i not in nn]
+    if int(np.prod(shape, dtype=np.int64)) != X.size:
+        raise RefThrows("Squeeze: removed axis is not of extent 1")  # emptyTensor(dims, type, data) length check
+    return X.reshape(shape)
+
+
+def unsqueeze(X, axes):
+    """operators/base/unsqueeze.ts:8-27 (+ cpu unsqueeze.ts: shares the buffer)."""
+    X = np.asarray(X)
+    axes = [int(a) for a in axes]
+    nd = X.ndim + len(axes)
+    nn = [a if a >= 0 else a + nd for a in axes]
+    shape, src = [], 0
+    for d in range(nd):
+        if d in nn:
+            shape.append(1)
+        else:
+            if src >= X.ndim:
+                raise RefThrows("Unsqueeze: axes out of range")
+            shape.append(X.shape[src])
+            src += 1
+    if src != X.ndim:
+        raise RefThrows("Unsqueeze: duplicate axes")
+    return X.reshape(shape)
+
+
+def concat(inputs, axis=0):
+    """cpu concat.ts:21-84: the flat-index loops, vectorised over (c, outer, inner)."""
+    inputs = [np.asarray(t, order="C") for t in inputs]
+    first = inputs[0]
+    ax = axis if axis >= 0 else first.ndim + axis
+    if ax < 0 or ax >= first.ndim:
+        raise RefThrows("Concat: axis %d out of range" % ax)
+    out_shape = list(first.shape)
+    out_shape[ax] = sum(t.shape[ax] for t in inputs)
+    outer_len = int(np.prod(first.shape[:ax], dtype=np.int64))
+    inner_len = int(np.prod(first.shape[ax + 1:], dtype=np.int64))
+
+    def strides(shape):
+        s, acc = [], 1
+        for d in reversed(shape):
+            s.insert(0, acc)
+            acc *= d
+        return s
+
+    out = np.zeros(int(np.prod(out_shape, dtype=np.int64)), dtype=first.dtype)
+    so = strides(out_shape)
+    out_outer, out_cat = so[max(ax - 1, 0)], so[ax]
+    offset = 0
+    for t in inputs:
+        st = strides(t.shape)
+        dim, outer_s, cat_s = t.shape[ax], st[max(ax - 1, 0)], st[ax]
+        c, o, i = np.meshgrid(np.arange(dim), np.arange(outer_len), np.arange(inner_len),
+                              indexing="ij")
+        out[((c + offset) * out_cat + o * out_outer + i).reshape(-1)] = \
+            t.reshape(-1)[(c * cat_s + o * outer_s + i).reshape(-1)]
+        offset += dim
+    return out.reshape(out_shape)
+
+
+def split(X, n_outputs, axis=0, split=()):
+    """operators/base/split.ts:10-70 + cpu split.ts:12-45."""
+    X = np.asarray(X, order="C")
+    ax = axis if axis >= 0 else axis + X.ndim
+    if ax < 0 or ax >= X.ndim:
+        raise RefThrows("Split: axis %d out of range" % ax)
+    axis_len = X.shape[ax]
+    parts = [int(s) for s in split] if len(split) else [axis_len // n_outputs] * n_outputs
+    outer_len = int(np.prod(X.shape[:ax], dtype=np.int64))
+    inner_len = int(np.prod(X.shape[ax + 1:], dtype=np.int64))
+    in_cat = inner_len
+    # input.strides[max(axis-1, 0)]
+    st, acc = [], 1
+    for d in reversed(X.shape):
+        st.insert(0, acc)
+        acc *= d
+    in_outer = st[max(ax - 1, 0)]
+    flat = X.reshape(-1)
+    outs, offset = [], 0
+    for n in range(n_outputs):
+        dim = parts[n]
+        out_shape = list(X.shape)
+        out_shape[ax] = dim
+        outer_s = int(np.prod(out_shape[max(ax - 1, 0) + 1:], dtype=np.int64))
+        split_s = int(np.prod(out_shape[ax + 1:], dtype=np.int64))
+        ot = np.zeros(int(np.prod(out_shape, dtype=np.int64)), dtype=X.dtype)
+        c, o, i = np.meshgrid(np.arange(dim), np.arange(outer_len), np.arange(inner_len),
+                              indexing="ij")
+        ot[(c * split_s + o * outer_s + i).reshape(-1)] = \
+            flat[((c + offset) * in_cat + o * in_outer + i).reshape(-1)]
+        outs.append(ot.reshape(out_shape))
+        offset += dim
+    return outs
+
+
+def slice_(data, starts, ends, axes=None, steps=None):
+    """cpu slice.ts:12-94 (Slice, opset >= 10), including its clamping rules:
+    start is clamped to [0, size-1] and stop to [-1, size] whatever the sign of the step."""
+    data = np.asarray(data, order="C")
+    if data.ndim > 6:
+        raise RefThrows("Slice: input dimension %d > 6 is not yet supported" % data.ndim)
+    starts = [int(v) for v in starts]
+    ends = [int(v) for v in ends]
+    if axes is not None:
+        axes = [int(a) + data.ndim if int(a) < 0 else int(a) for a in axes]
+    else:
+        axes = list(range(data.ndim))
+    steps = [int(v) for v in steps] if steps is not None else [1] * len(axes)
+    ranges = [[0, d, 1, d] for d in data.shape]
+    for i, a in enumerate(axes):
+        ranges[a] = [starts[i], ends[i], steps[i], data.shape[a]]
+    index = []
+    for start, stop, step, size in ranges:
+        if start < 0:
+            start += size
+        start = max(min(start, size - 1), 0)
+        if stop < 0:
+            stop += size
+        stop = max(min(stop, size), -1)
+        dst = max(int(np.ceil((stop - start) / step)), 0)
+        index.append(start + step * np.arange(dst))
+    out_shape = [len(ix) for ix in index]
+    if data.ndim == 0:
+        return data.copy()
+    return data[np.ix_(*index)].reshape(out_shape)
+
+
+def js_to_int32(values):
+    """ECMAScript ToInt32 of each element (what TypedArray.prototype.set does for Int32Array)."""
+    v = np.asarray(values, dtype=np.float64)
+    finite = np.isfinite(v)
+    t = np.trunc(np.where(finite, v, 0.0))
+    m = np.mod(t, 4294967296.0)
+    m = np.where(m >= 2147483648.0, m - 4294967296.0, m)
+    return m.astype(np.int64).astype(np.int32)
+
+
+def cast(X, to):
+    """cpu cast.ts:12-52: `to` is an ONNX TensorProto.DataType; FLOAT(1) -> float32,
+    UINT8(2) / INT32(6) / INT64(7) -> int32 (no clipping), anything else throws."""
+    X = np.asarray(X)
+    if to == 1:
+        return X.astype(np.float32)
+    if to in (2, 6, 7):
+        return js_to_int32(X) if X.dtype != np.int32 else X.copy()
+    raise RefThrows("Cast: converting to DataType %d is not yet supported" % to)

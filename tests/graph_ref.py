@@ -8,7 +8,9 @@ from oracle import ref
 def run_graph(model, feeds, keep=None):
     """model: webdnn_amd.modelgen.parse_model(...) result; feeds: {input name: array}.
     Returns {output name: array} (plus every tensor named in `keep`)."""
-    env = dict(model["initializers"])
+    # the runner clips INT64 tensors to int32 when it loads them (core/runnerImpl.ts:167-198)
+    to32 = lambda v: v.astype(np.int32) if isinstance(v, np.ndarray) and v.dtype == np.int64 else v
+    env = {k: to32(v) for k, v in model["initializers"].items()}
     env.update(feeds)
     for n in model["nodes"]:
         x = [env[i] for i in n["inputs"]]
@@ -45,6 +47,27 @@ def run_graph(model, feeds, keep=None):
         elif op == "ReduceMean":
             assert a.get("axes") in ([-1], [x[0].ndim - 1]) and a.get("keepdims", 1) == 1
             y = ref.reduce_mean_last(x[0])
+        elif op == "Squeeze":
+            y = ref.squeeze(x[0], x[1].reshape(-1) if len(x) > 1 else a.get("axes", []))
+        elif op == "Unsqueeze":
+            y = ref.unsqueeze(x[0], x[1].reshape(-1) if len(x) > 1 else a.get("axes", []))
+        elif op == "Concat":
+            y = ref.concat(x, a.get("axis", 0))
+        elif op == "Split":
+            parts = x[1].reshape(-1) if len(x) > 1 else a.get("split", [])
+            for name, part in zip(n["outputs"], ref.split(x[0], len(n["outputs"]), a.get("axis", 0), parts)):
+                env[name] = part
+            continue
+        elif op == "Slice":
+            y = ref.slice_(x[0], x[1], x[2], x[3] if len(x) > 3 else None, x[4] if len(x) > 4 else None)
+        elif op == "Cast":
+            y = ref.cast(x[0], a.get("to", 1))
+        elif op == "Constant":
+            y = to32(a["value"])
+        elif op == "Shape":
+            y = np.array(x[0].shape, np.int32)
+        elif op == "Gather":
+            y = ref.gather(x[0], x[1], a.get("axis", 0))
         else:
             raise NotImplementedError(op)
         env[n["outputs"][0]] = np.asarray(y)

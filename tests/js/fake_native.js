@@ -242,6 +242,29 @@ const native = {
     }
   },
 
+  cast(from, to, X, Y, length) {
+    count("cast");
+    need(X, length * 4, "wdh_cast: X"); need(Y, length * 4, "wdh_cast: Y");
+    const src = from === 0 ? f32(X) : i32(X), dst = to === 0 ? f32(Y) : i32(Y);
+    for (let i = 0; i < length; i++) dst[i] = src[i]; // typed-array stores convert like Cast
+  },
+
+  stridedCopy(X, xOffset, Y, yOffset, shape, xStrides, yStrides) {
+    count("stridedCopy");
+    const x = new Uint32Array(buf(X).buffer), y = new Uint32Array(buf(Y).buffer);
+    const total = shape.reduce((a, b) => a * b, 1), nd = shape.length, idx = new Array(nd).fill(0);
+    for (let n = 0; n < total; n++) {
+      let sx = xOffset, sy = yOffset;
+      for (let d = 0; d < nd; d++) { sx += idx[d] * xStrides[d]; sy += idx[d] * yStrides[d]; }
+      if (sx < 0 || sx >= x.length || sy < 0 || sy >= y.length) throw new Error("wdh_strided_copy failed (-2): view outside the buffer");
+      y[sy] = x[sx];
+      for (let d = nd - 1; d >= 0; d--) {
+        if (++idx[d] < shape[d]) break;
+        idx[d] = 0;
+      }
+    }
+  },
+
   // ---- test introspection ----
   __liveBuffers() {
     return buffers.size;

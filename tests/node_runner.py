@@ -41,6 +41,9 @@ def run_model(model_dir, inputs, backend, strict=True, fuse=True, oracle_cpu=Fal
     outputs, pos = [], 0
     for o in report["outputs"]:
         n = int(np.prod(o["dims"], dtype=np.int64)) if o["dims"] else 1
-        outputs.append(flat[pos:pos + n].reshape(o["dims"]))
+        part = flat[pos:pos + n]
+        if o.get("dataType") == "int32":
+            part = part.view(np.int32)
+        outputs.append(part.reshape(o["dims"]))
         pos += n
     return outputs, report

@@ -401,6 +401,137 @@ def test_flatten_reshape_alias_and_gather(ctx):
     assert_bit_exact(got, np.take(table, [2, 0, -2], axis=1), "gather axis 1")
 
 
+def test_squeeze_unsqueeze_alias(ctx):
+    x = nrm(2, 1, 3, 1)
+    t = ctx.move_tensor(x)
+    for axes in ([], [1], [-1, 1], [3]):
+        y = H.squeeze(ctx, t, axes)
+        assert y.handle == t.handle                               # zero-copy (cpu squeeze.ts:12-37)
+        assert_bit_exact(y.get_data(), ref.squeeze(x, axes), "squeeze %s" % axes)
+    with pytest.raises(H.OperatorError):
+        H.squeeze(ctx, t, [0])
+    for axes in ([0], [1, -1], [0, 5]):
+        y = H.unsqueeze(ctx, t, axes)
+        assert y.handle == t.handle
+        assert_bit_exact(y.get_data(), ref.unsqueeze(x, axes), "unsqueeze %s" % axes)
+
+
+@pytest.mark.parametrize("axis", [-4, -1, 0, 1, 2, 3])
+def test_concat(ctx, axis):
+    shape = [3, 5, 4, 6]
+    ax = axis % 4
+    parts = []
+    for n in (1, 7, 0, 2):
+        sh = list(shape)
+        sh[ax] = n
+        parts.append(nrm(*sh))
+    got = H.concat(ctx, [ctx.move_tensor(p) for p in parts], axis).get_data()
+    assert_bit_exact(got, ref.concat(parts, axis), "concat axis %d" % axis)
+
+
+def test_concat_model_shapes_ints_and_errors(ctx):
+    # DETR-style: positional halves [1,128,25,34] x2 on axis 1; shape pieces (int32) on axis 0
+    a, b = nrm(1, 128, 25, 34), nrm(1, 128, 25, 34)
+    assert_bit_exact(H.concat(ctx, [ctx.move_tensor(a), ctx.move_tensor(b)], 1).get_data(), ref.concat([a, b], 1))
+    big = [nrm(850, 8, 32) for _ in range(3)]
+    assert_bit_exact(H.concat(ctx, [ctx.move_tensor(t) for t in big], -1).get_data(), ref.concat(big, -1))
+    ints = [np.array([1, 2], np.int32), np.array([3], np.int32)]
+    got = H.concat(ctx, [ctx.move_tensor(t) for t in ints], 0).get_data()
+    assert_bit_exact(got, ref.concat(ints, 0))
+    with pytest.raises(H.OperatorError):
+        H.concat(ctx, [ctx.move_tensor(a)], 4)
+    with pytest.raises(H.OperatorError):
+        H.concat(ctx, [ctx.move_tensor(a), ctx.move_tensor(nrm(1, 128, 25, 33))], 1)
+
+
+@pytest.mark.parametrize("axis,n,parts", [(0, 2, ()), (1, 3, ()), (2, 5, ()), (-1, 1, ()), (1, 3, (1, 2, 3)),
+                                           (1, 4, ()), (2, 3, (0, 4, 1))])
+def test_split(ctx, axis, n, parts):
+    x = nrm(4, 6, 5)
+    got = H.split(ctx, ctx.move_tensor(x), n, axis, parts)
+    want = ref.split(x, n, axis, parts)
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        assert_bit_exact(g.get_data(), w, "split axis %d" % axis)
+
+
+def test_split_qkv_and_errors(ctx):
+    x = nrm(850, 768)                                             # packed q,k,v projections
+    got = H.split(ctx, ctx.move_tensor(x), 3, 1)
+    for g, w in zip(got, ref.split(x, 3, 1)):
+        assert_bit_exact(g.get_data(), w)
+    with pytest.raises(H.OperatorError):
+        H.split(ctx, ctx.move_tensor(x), 2, 2)
+    with pytest.raises(H.OperatorError):
+        H.split(ctx, ctx.move_tensor(x), 2, 1, (500, 500))
+
+
+@pytest.mark.parametrize("args", [
+    dict(starts=[1, 2], ends=[4, 6], axes=[0, 2]),
+    dict(starts=[0, 0, 0], ends=[5, 6, 7]),
+    dict(starts=[1], ends=[-1], axes=[-1], steps=[2]),
+    dict(starts=[-3], ends=[1000], axes=[1]),
+    dict(starts=[-1], ends=[-1000], axes=[2], steps=[-1]),
+    dict(starts=[5, 4], ends=[0, -100], axes=[1, 0], steps=[-2, -3]),
+    dict(starts=[3], ends=[2], axes=[0]),
+    dict(starts=[5], ends=[5], axes=[0]),                        # reference quirk: start clamps to size-1
+    dict(starts=[9], ends=[100], axes=[1]),
+])
+def test_slice(ctx, args):
+    x = nrm(5, 6, 7)
+    got = H.slice_(ctx, ctx.move_tensor(x), **args).get_data()
+    assert_bit_exact(got, ref.slice_(x, **args), "slice %s" % args)
+
+
+def test_slice_ranks_ints_and_errors(ctx):
+    x6 = nrm(2, 3, 2, 3, 2, 5)
+    args = dict(starts=[1, 0, 1], ends=[3, 2, 5], axes=[1, 3, 5], steps=[1, 1, 2])
+    assert_bit_exact(H.slice_(ctx, ctx.move_tensor(x6), **args).get_data(), ref.slice_(x6, **args))
+    v = np.arange(10, dtype=np.int32)
+    assert_bit_exact(H.slice_(ctx, ctx.move_tensor(v), [2], [9], [0], [3]).get_data(), ref.slice_(v, [2], [9], [0], [3]))
+    big = nrm(32, 256, 56, 56)                                     # crop of a feature map, 100 MB in
+    args = dict(starts=[4, 3], ends=[52, 53], axes=[2, 3])
+    assert_bit_exact(H.slice_(ctx, ctx.move_tensor(big), **args).get_data(), ref.slice_(big, **args))
+    with pytest.raises(H.OperatorError):
+        H.slice_(ctx, ctx.move_tensor(nrm(*([1] * 7))), [0], [1])
+    with pytest.raises(H.OperatorError):
+        H.slice_(ctx, ctx.move_tensor(v), [0], [1], [0], [0])
+
+
+def test_cast(ctx):
+    v = np.array([0.0, -0.0, 1.9, -1.9, 2147483648.0, -2147483648.0, 4294967296.0, 3e9, -3e9, 1e20,
+                  np.nan, np.inf, -np.inf, 123456.7], np.float32)
+    for to in (6, 7, 2):
+        assert_bit_exact(H.cast(ctx, ctx.move_tensor(v), to).get_data(), ref.cast(v, to), "f32 -> int32")
+    assert_bit_exact(H.cast(ctx, ctx.move_tensor(v), 1).get_data(), ref.cast(v, 1), "f32 -> f32")
+    i = np.array([3, -7, 2 ** 31 - 1, -2 ** 31, 16777217], np.int32)
+    assert_bit_exact(H.cast(ctx, ctx.move_tensor(i), 1).get_data(), ref.cast(i, 1), "int32 -> f32")
+    assert_bit_exact(H.cast(ctx, ctx.move_tensor(i), 7).get_data(), ref.cast(i, 7), "int32 -> int32")
+    big = uni(1000, 1001, lo=-5e9, hi=5e9)
+    assert_bit_exact(H.cast(ctx, ctx.move_tensor(big), 6).get_data(), ref.cast(big, 6), "f32 -> int32, 1M values")
+    with pytest.raises(H.OperatorError):
+        H.cast(ctx, ctx.move_tensor(v), 10)
+
+
+def test_strided_copy_rejects_views_outside_the_buffers(ctx):
+    t = ctx.move_tensor(nrm(4, 4))
+    y = ctx.empty_tensor([4, 4], "float32")
+    i32, i64 = ctypes.c_int32 * 2, ctypes.c_int64 * 2
+    ok = (t.handle, 0, y.handle, 0, 2, i32(4, 4), i64(4, 1), i64(4, 1))
+    capi.call("wdh_strided_copy", *ok)
+    for bad in [(t.handle, 1, y.handle, 0, 2, i32(4, 4), i64(4, 1), i64(4, 1)),      # X overruns
+                (t.handle, 0, y.handle, 0, 2, i32(4, 4), i64(4, 1), i64(5, 1)),      # Y overruns
+                (t.handle, 0, y.handle, 0, 2, i32(4, 4), i64(-4, 1), i64(4, 1)),     # X before its start
+                (t.handle, -1, y.handle, 0, 2, i32(4, 4), i64(4, 1), i64(4, 1)),
+                (t.handle, 0, y.handle, 0, 7, i32(4, 4), i64(4, 1), i64(4, 1))]:
+        with pytest.raises(capi.HipError) as err:
+            capi.call("wdh_strided_copy", *bad)
+        assert err.value.code == -2
+    # reversed rows through a negative X stride
+    capi.call("wdh_strided_copy", t.handle, 12, y.handle, 0, 2, i32(4, 4), i64(-4, 1), i64(4, 1))
+    assert_bit_exact(y.get_data(), t.get_data()[::-1].copy())
+
+
 # ------------------------------------------------------------------ runtime
 def test_buffers_offsets_large_copies_and_pool(ctx):
     n = 20 * 1024 * 1024 + 13                 # 80 MiB: several staging chunks each way

@@ -122,3 +122,19 @@ def test_detr_r50_config5(tmp_path):
     want = graph_ref.run_graph(model, {"input": X})
     assert np.abs(hip[0] - want["logits"]).max() <= 1e-3, np.abs(hip[0] - want["logits"]).max()
     assert np.abs(hip[1] - want["boxes"]).max() <= 1e-3
+
+
+@pytest.mark.parametrize("opset", [11, 13])
+def test_export_style_glue_graph(tmp_path, opset):
+    """Layout glue (Split / Concat / Slice / Cast / Squeeze / Unsqueeze / Gather) on the device and the
+    shape chain around Reshape; bit-exact, since nothing here does arithmetic except one Mul and Add."""
+    data, _ = modelgen.glue_model(opset)
+    X = np.random.default_rng(1).standard_normal((2, 6, 4, 5)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    model = modelgen.parse_model(data)
+    hip, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=True)
+    assert rep["stats"]["nodesByBackend"] == {"cpu": 2, "hip": len(model["nodes"]) - 2}, rep["stats"]
+    assert rep["stats"]["retriedOnCpu"] == []
+    want = graph_ref.run_graph(model, {"X": X})
+    assert_bit_exact(hip[0], want["Y"], "Y")
+    assert_bit_exact(hip[1], want["ints"], "ints")

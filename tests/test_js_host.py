@@ -161,3 +161,22 @@ def test_detr_style_graph_on_the_hip_host_path(tmp_path):
     plain, rep_p = node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fuse=False, fake_native=True)
     assert rep_p["nodes"] > rep["nodes"]
     assert_bit_exact(plain[0], outs[0], "fusion keeps the logits")
+
+
+@pytest.mark.parametrize("opset", [11, 13])
+def test_export_style_glue_graph(tmp_path, opset):
+    """Shape -> Gather -> Unsqueeze -> Concat -> Reshape on the metadata side and Split / Concat /
+    Slice / Cast / Squeeze / Unsqueeze on the data, with axes as attributes (opset 11) and as
+    inputs (opset 13).  Shape and Constant are the only nodes placed on the cpu, as in the
+    reference (operatorTable.ts:47-50; Constant exists for cpu only)."""
+    data, _ = modelgen.glue_model(opset)
+    X = np.random.default_rng(1).standard_normal((2, 6, 4, 5)).astype(np.float32)
+    model, hip, cpu, rep = both_paths(tmp_path, data, {"X": X})
+    assert rep["stats"]["nodesByBackend"] == {"cpu": 2, "hip": len(model["nodes"]) - 2}, rep["stats"]
+    assert rep["stats"]["retriedOnCpu"] == []
+    want = graph_ref.run_graph(model, {"X": X})
+    for got_hip, got_cpu, (name, _) in zip(hip, cpu, model["outputs"]):
+        assert_bit_exact(got_hip, got_cpu, name + ": hip host path vs cpu path")
+        assert_bit_exact(got_hip, want[name], name + ": vs the python oracle")
+    assert hip[1].dtype == np.int32
+    assert rep["liveBuffers"] == rep["initializerCopies"]

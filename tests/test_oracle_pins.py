@@ -384,3 +384,92 @@ def test_layout_ops():
     assert ref.gather(np.array([5, 6, 7], np.int32), np.array(2, np.int32)).tolist() == 7
     with pytest.raises(ref.RefThrows):
         ref.gather(np.zeros((2, 2), np.int32), np.array(0, np.int32))    # cpu gather.ts:23-27
+
+
+# ---- Squeeze / Unsqueeze / Concat / Split / Slice / Cast ----------------------------------
+# Pinned against numpy's own routines on cases where the reference's rules and numpy's
+# coincide, and against hand-derived answers where the reference deviates (Slice clamping,
+# ToInt32 wrap-around).
+
+def test_squeeze_unsqueeze():
+    x = np.arange(2 * 1 * 3 * 1, dtype=np.float32).reshape(2, 1, 3, 1)
+    assert ref.squeeze(x).shape == (2, 3)
+    assert ref.squeeze(x, [1]).shape == (2, 3, 1)
+    assert ref.squeeze(x, [-1, 1]).shape == (2, 3)
+    assert np.array_equal(ref.squeeze(x, [3]), np.squeeze(x, 3))
+    with pytest.raises(ref.RefThrows):
+        ref.squeeze(x, [0])
+    y = np.arange(6, dtype=np.float32).reshape(2, 3)
+    assert ref.unsqueeze(y, [0]).shape == (1, 2, 3)
+    assert ref.unsqueeze(y, [1, -1]).shape == (2, 1, 3, 1)
+    assert np.array_equal(ref.unsqueeze(y, [0, 3]), np.expand_dims(y, (0, 3)))
+    assert ref.unsqueeze(np.float32(3.0), [0]).shape == (1,)
+
+
+@pytest.mark.parametrize("axis", [-4, -1, 0, 1, 2, 3])
+def test_concat_is_numpy_concatenate(axis):
+    rng = np.random.default_rng(axis + 10)
+    shape = [2, 3, 4, 5]
+    parts = []
+    ax = axis % 4
+    for n in (1, 3, 2):
+        s = list(shape)
+        s[ax] = n
+        parts.append(rng.standard_normal(s).astype(np.float32))
+    assert_bit_exact(ref.concat(parts, axis), np.concatenate(parts, axis))
+    ints = [np.array([1, 2], np.int32), np.array([3], np.int32)]
+    assert_bit_exact(ref.concat(ints, 0), np.array([1, 2, 3], np.int32))
+    with pytest.raises(ref.RefThrows):
+        ref.concat(parts, 4)
+
+
+def test_split_is_numpy_split():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((4, 6, 5)).astype(np.float32)
+    for axis, n in [(0, 2), (1, 3), (2, 5), (-1, 1), (-2, 2)]:
+        for a, b in zip(ref.split(x, n, axis), np.split(x, n, axis)):
+            assert_bit_exact(a, np.ascontiguousarray(b))
+    a, b, c = ref.split(x, 3, 1, [1, 2, 3])
+    assert_bit_exact(a, np.ascontiguousarray(x[:, :1]))
+    assert_bit_exact(b, np.ascontiguousarray(x[:, 1:3]))
+    assert_bit_exact(c, np.ascontiguousarray(x[:, 3:]))
+    # an uneven axis without `split`: floor(len / n) each, the remainder is dropped (split.ts:26-30)
+    parts = ref.split(x, 4, 1)
+    assert [p.shape[1] for p in parts] == [1, 1, 1, 1]
+    assert_bit_exact(parts[3], x[:, 3:4])
+    with pytest.raises(ref.RefThrows):
+        ref.split(x, 2, 3)
+
+
+def test_slice_matches_numpy_where_rules_coincide_and_clamps_like_the_reference():
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((5, 6, 7)).astype(np.float32)
+    assert_bit_exact(ref.slice_(x, [1, 2], [4, 6], [0, 2]), x[1:4, :, 2:6])
+    assert_bit_exact(ref.slice_(x, [0, 0, 0], [5, 6, 7]), x)
+    assert_bit_exact(ref.slice_(x, [1], [-1], [-1], [2]), x[:, :, 1:-1:2])
+    assert_bit_exact(ref.slice_(x, [-3], [1000], [1]), x[:, -3:])
+    assert_bit_exact(ref.slice_(x, [-1], [-1000], [2], [-1]), x[:, :, ::-1])
+    assert_bit_exact(ref.slice_(x, [5], [0], [1], [-2]), x[:, 5:0:-2])
+    assert ref.slice_(x, [3], [2], [0]).shape == (0, 6, 7)
+    # the reference clamps start to size-1 even for a forward step: [5:5] on 5 elements
+    # yields the last one (numpy would return none)
+    assert_bit_exact(ref.slice_(x, [5], [5], [0]), x[4:5])
+    assert_bit_exact(ref.slice_(x, [9], [100], [1]), x[:, 5:6])
+    with pytest.raises(ref.RefThrows):
+        ref.slice_(np.zeros((1,) * 7, np.float32), [0], [1])
+
+
+def test_cast_and_toint32():
+    v = np.array([0.0, -0.0, 1.9, -1.9, 2147483647.0, 2147483648.0, -2147483648.0, 4294967296.0,
+                  4294967297.0, 3e9, -3e9, 1e20, np.nan, np.inf, -np.inf], np.float32)
+    want = np.array([0, 0, 1, -1, -2147483648, -2147483648, -2147483648, 0,
+                     0, -1294967296, 1294967296, 0, 0, 0, 0], np.int32)
+    # 2147483647 is not a float32: it rounds to 2^31; 4294967297 rounds to 2^32;
+    # 1e20f = 0x56bc76 * 2^44, a multiple of 2^32
+    assert_bit_exact(ref.cast(v, 6), want)
+    assert_bit_exact(ref.cast(v, 7), want)
+    assert_bit_exact(ref.cast(np.array([3, -7, 2 ** 31 - 1], np.int32), 1),
+                     np.array([3.0, -7.0, 2147483648.0], np.float32))
+    assert ref.cast(np.array([1.5], np.float32), 1).dtype == np.float32
+    with pytest.raises(ref.RefThrows):
+        ref.cast(v, 10)

@@ -50,6 +50,8 @@ SIGNATURES = {
     "wdh_global_avgpool": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
     "wdh_transpose": (_c.c_int, [c_buf, c_buf, _c.c_int, _i32p, _i64p]),
     "wdh_gather": (_c.c_int, [c_buf, c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64]),
+    "wdh_cast": (_c.c_int, [_c.c_int, _c.c_int, c_buf, c_buf, _c.c_size_t]),
+    "wdh_strided_copy": (_c.c_int, [c_buf, _c.c_int64, c_buf, _c.c_int64, _c.c_int, _i32p, _i64p, _i64p]),
 }
 
 

@@ -227,6 +227,21 @@ __global__ __launch_bounds__(256) void unary_i32(int op, const int *__restrict__
   }
 }
 
+// Cast between the two data types the runner has: storing a float into an
+// Int32Array applies ToInt32, storing an int into a Float32Array rounds to nearest.
+__global__ __launch_bounds__(256) void cast_f32_i32(const float *__restrict__ X,
+                                                    int *__restrict__ Y, long long total) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride)
+    Y[e] = js_to_int32((double)X[e]);
+}
+__global__ __launch_bounds__(256) void cast_i32_f32(const int *__restrict__ X,
+                                                    float *__restrict__ Y, long long total) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride)
+    Y[e] = (float)X[e];
+}
+
 template <int OP>
 int launch_unary(const float *X, float *Y, long long total) {
   bool vec = (((uintptr_t)X | (uintptr_t)Y) & 15) == 0;
@@ -341,4 +356,28 @@ extern "C" int wdh_unary(int op, int dtype, wdh_buf hX, wdh_buf hY, size_t lengt
     case WDH_UN_NEG: return launch_unary<WDH_UN_NEG>(X, Y, total);
     default: return launch_unary<WDH_UN_RECIPROCAL>(X, Y, total);
   }
+}
+
+extern "C" int wdh_cast(int from_dtype, int to_dtype, wdh_buf hX, wdh_buf hY, size_t length) {
+  WDH_REQUIRE_INIT();
+  if ((from_dtype != 0 && from_dtype != 1) || (to_dtype != 0 && to_dtype != 1))
+    return fail(WDH_EINVAL, "wdh_cast: dtype %d -> %d (0 = float32, 1 = int32)", from_dtype,
+                to_dtype);
+  if (length == 0) return WDH_OK;
+  void *px, *py;
+  if (!wdh::operand(hX, length * 4, "wdh_cast: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, length * 4, "wdh_cast: Y", &py)) return WDH_EINVAL;
+  const long long total = (long long)length;
+  if (from_dtype == to_dtype) {
+    WDH_HIP_CHECK(hipMemcpyAsync(py, px, length * 4, hipMemcpyDeviceToDevice, wdh::stream()));
+    return WDH_OK;
+  }
+  if (from_dtype == 0)
+    hipLaunchKernelGGL(cast_f32_i32, dim3(grid_for(total, 256)), dim3(256), 0, wdh::stream(),
+                       (const float *)px, (int *)py, total);
+  else
+    hipLaunchKernelGGL(cast_i32_f32, dim3(grid_for(total, 256)), dim3(256), 0, wdh::stream(),
+                       (const int *)px, (float *)py, total);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
 }

@@ -77,6 +77,38 @@ __global__ __launch_bounds__(256) void gather_copy_kernel(GatherCopyParams p) {
   }
 }
 
+// Strided copy (Slice, Concat, Split): both sides addressed through strides.
+struct StridedCopyParams {
+  const uint32_t *X;
+  uint32_t *Y;
+  long long total;
+  int ndim;
+  unsigned shape[MAXD];
+  long long sx[MAXD];
+  long long sy[MAXD];
+};
+
+// Thread per element, innermost axis fastest: coalesced wherever the innermost
+// stride is 1 (always on the dense side of a Slice/Concat/Split).
+__global__ __launch_bounds__(256) void strided_copy_kernel(StridedCopyParams p) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
+       i += stride) {
+    long long rem = i, ox = 0, oy = 0;
+#pragma unroll
+    for (int d = MAXD - 1; d >= 0; d--) {
+      if (d < p.ndim) {
+        const long long q = rem / p.shape[d];
+        const long long r = rem - q * p.shape[d];
+        ox += r * p.sx[d];
+        oy += r * p.sy[d];
+        rem = q;
+      }
+    }
+    p.Y[oy] = p.X[ox];
+  }
+}
+
 // Tiled: when the input-contiguous axis `a` is not the last output axis, a
 // workgroup moves a 64x64 tile spanned by (axis a, last axis) through LDS:
 // reads run along axis a (contiguous in X), writes along the last axis
@@ -271,6 +303,62 @@ extern "C" int wdh_gather(wdh_buf hD, wdh_buf hI, wdh_buf hY, int64_t outer,
                      wdh::stream(), (const uint32_t *)pd, (const int *)pi,
                      (uint32_t *)py, (long long)outer, axis_len, (long long)inner,
                      (long long)n_idx);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+extern "C" int wdh_strided_copy(wdh_buf hX, int64_t x_offset, wdh_buf hY, int64_t y_offset,
+                                int ndim, const int32_t *shape, const int64_t *x_strides,
+                                const int64_t *y_strides) {
+  WDH_REQUIRE_INIT();
+  if (ndim < 0 || ndim > MAXD)
+    return fail(WDH_EINVAL, "wdh_strided_copy: ndim %d outside 0..%d", ndim, MAXD);
+  if (ndim > 0 && (!shape || !x_strides || !y_strides))
+    return fail(WDH_EINVAL, "wdh_strided_copy: NULL shape or strides");
+  if (x_offset < 0 || y_offset < 0)
+    return fail(WDH_EINVAL, "wdh_strided_copy: negative offset");
+  // Negative strides are allowed on the X side (a Slice with a negative step);
+  // the lowest and highest element touched on each side are bounds-checked.
+  StridedCopyParams g = {};
+  long long total = 1, x_lo = x_offset, x_hi = x_offset, y_hi = y_offset;
+  int nd = 0;
+  for (int d = 0; d < ndim; d++) {
+    if (shape[d] < 0 || y_strides[d] < 0)
+      return fail(WDH_EINVAL, "wdh_strided_copy: negative extent or Y stride");
+    total *= shape[d];
+    if (shape[d] <= 1) continue;
+    const long long reach = (long long)(shape[d] - 1) * x_strides[d];
+    if (reach < 0) x_lo += reach; else x_hi += reach;
+    y_hi += (long long)(shape[d] - 1) * y_strides[d];
+    // merge with the previous axis when both sides step contiguously across it
+    if (nd > 0 && g.sx[nd - 1] == x_strides[d] * shape[d] &&
+        g.sy[nd - 1] == y_strides[d] * shape[d] &&
+        (unsigned long long)g.shape[nd - 1] * shape[d] <= 0xffffffffULL) {
+      g.shape[nd - 1] *= shape[d];
+      g.sx[nd - 1] = x_strides[d];
+      g.sy[nd - 1] = y_strides[d];
+    } else {
+      g.shape[nd] = shape[d];
+      g.sx[nd] = x_strides[d];
+      g.sy[nd] = y_strides[d];
+      nd++;
+    }
+  }
+  if (total == 0) return WDH_OK;
+  if (x_lo < 0) return fail(WDH_EINVAL, "wdh_strided_copy: X view starts before the buffer");
+  void *px, *py;
+  if (!wdh::operand(hX, (size_t)(x_hi + 1) * 4, "wdh_strided_copy: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)(y_hi + 1) * 4, "wdh_strided_copy: Y", &py)) return WDH_EINVAL;
+  g.X = (const uint32_t *)px + x_offset;
+  g.Y = (uint32_t *)py + y_offset;
+  g.total = total;
+  g.ndim = nd;
+  if (nd == 0 || (nd == 1 && g.sx[0] == 1 && g.sy[0] == 1)) {
+    WDH_HIP_CHECK(hipMemcpyAsync(g.Y, g.X, (size_t)total * 4, hipMemcpyDeviceToDevice,
+                                 wdh::stream()));
+    return WDH_OK;
+  }
+  hipLaunchKernelGGL(strided_copy_kernel, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }

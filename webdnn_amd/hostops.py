@@ -525,3 +525,161 @@ def gather(ctx, data, indices, axis=0):
     call("wdh_gather", data.handle, indices.handle, y.handle, outer, data.dims[axis], inner,
          indices.length)
     return y
+
+
+# ---- layout glue on the device --------------------------------------------------------
+
+def _dense_strides(dims):
+    out, acc = [], 1
+    for d in reversed(dims):
+        out.insert(0, acc)
+        acc *= d
+    return out
+
+
+def _strided_copy(x, x_offset, y, y_offset, shape, x_strides, y_strides):
+    nd = len(shape)
+    if nd > 6:
+        raise OperatorError("strided copy: rank %d is not supported" % nd)
+    call("wdh_strided_copy", x.handle, x_offset, y.handle, y_offset, nd,
+         (ctypes.c_int32 * max(nd, 1))(*shape), (ctypes.c_int64 * max(nd, 1))(*x_strides),
+         (ctypes.c_int64 * max(nd, 1))(*y_strides))
+
+
+def squeeze_shape(dims, axes):
+    """operators/base/squeeze.ts:8-22"""
+    if not axes:
+        return [s for s in dims if s != 1]
+    nn = [a if a >= 0 else a + len(dims) for a in axes]
+    return [s for i, s in enumerate(dims) if i not in nn]
+
+
+def squeeze(ctx, x, axes=()):
+    """Squeeze (both the attribute and the input-tensor form of `axes`): zero-copy alias,
+    as cpu squeeze.ts:12-37 shares the input buffer."""
+    shape = squeeze_shape(x.dims, [int(a) for a in axes])
+    if int(np.prod(shape, dtype=np.int64)) != x.length:
+        raise OperatorError("Squeeze: removed axis is not of extent 1")
+    return x.alias(shape)
+
+
+def unsqueeze_shape(dims, axes):
+    """operators/base/unsqueeze.ts:8-27"""
+    nd = len(dims) + len(axes)
+    nn = [a if a >= 0 else a + nd for a in axes]
+    shape, src = [], 0
+    for d in range(nd):
+        if d in nn:
+            shape.append(1)
+        else:
+            if src >= len(dims):
+                raise OperatorError("Unsqueeze: axes out of range")
+            shape.append(dims[src])
+            src += 1
+    if src != len(dims):
+        raise OperatorError("Unsqueeze: duplicate axes")
+    return shape
+
+
+def unsqueeze(ctx, x, axes):
+    return x.alias(unsqueeze_shape(x.dims, [int(a) for a in axes]))
+
+
+def concat(ctx, inputs, axis=0):
+    """cpu concat.ts:21-84: one strided copy per input into its band of the output."""
+    first = inputs[0]
+    ax = axis if axis >= 0 else first.ndim + axis
+    if ax < 0 or ax >= first.ndim:
+        raise OperatorError("Concat: axis %d out of range" % ax)
+    for t in inputs:
+        if t.ndim != first.ndim or any(t.dims[d] != first.dims[d] for d in range(first.ndim) if d != ax):
+            raise OperatorError("Concat: input shapes differ outside the axis")
+        if t.data_type != first.data_type:
+            raise OperatorError("Concat: input data types differ")
+    out_shape = list(first.dims)
+    out_shape[ax] = sum(t.dims[ax] for t in inputs)
+    y = ctx.empty_tensor(out_shape, first.data_type)
+    ys = _dense_strides(out_shape)
+    offset = 0
+    for t in inputs:
+        if t.length:
+            _strided_copy(t, 0, y, offset * ys[ax], t.dims, _dense_strides(t.dims), ys)
+        offset += t.dims[ax]
+    return y
+
+
+def split(ctx, x, n_outputs, axis=0, split=()):
+    """operators/base/split.ts:10-70 + cpu split.ts:12-45"""
+    ax = axis if axis >= 0 else axis + x.ndim
+    if ax < 0 or ax >= x.ndim:
+        raise OperatorError("Split: axis %d out of range" % ax)
+    parts = [int(s) for s in split] if len(split) else [x.dims[ax] // n_outputs] * n_outputs
+    if len(parts) < n_outputs or any(p < 0 for p in parts) or sum(parts[:n_outputs]) > x.dims[ax]:
+        raise OperatorError("Split: parts do not fit the axis")
+    xs = _dense_strides(x.dims)
+    outs, offset = [], 0
+    for n in range(n_outputs):
+        shape = list(x.dims)
+        shape[ax] = parts[n]
+        y = ctx.empty_tensor(shape, x.data_type)
+        if y.length:
+            _strided_copy(x, offset * xs[ax], y, 0, shape, xs, _dense_strides(shape))
+        outs.append(y)
+        offset += parts[n]
+    return outs
+
+
+def slice_ranges(dims, starts, ends, axes=None, steps=None):
+    """cpu slice.ts:19-58: per axis (start, step, extent of the result), with the reference's
+    clamping (start to [0, size-1], stop to [-1, size])."""
+    nd = len(dims)
+    if nd > 6:
+        raise OperatorError("Slice: input dimension %d > 6 is not yet supported" % nd)
+    if axes is not None:
+        axes = [int(a) + nd if int(a) < 0 else int(a) for a in axes]
+    else:
+        axes = list(range(nd))
+    steps = [int(s) for s in steps] if steps is not None else [1] * len(axes)
+    ranges = [[0, d, 1] for d in dims]
+    for i, a in enumerate(axes):
+        if not 0 <= a < nd:
+            raise OperatorError("Slice: axis out of range")
+        if steps[i] == 0:
+            raise OperatorError("Slice: step 0")
+        ranges[a] = [int(starts[i]), int(ends[i]), steps[i]]
+    out = []
+    for (start, stop, step), size in zip(ranges, dims):
+        if start < 0:
+            start += size
+        start = max(min(start, size - 1), 0)
+        if stop < 0:
+            stop += size
+        stop = max(min(stop, size), -1)
+        out.append((start, step, max(-((start - stop) // step), 0)))  # ceil((stop-start)/step)
+    return out
+
+
+def slice_(ctx, x, starts, ends, axes=None, steps=None):
+    """Slice (opset >= 10); starts/ends/axes/steps live on the CPU (lists here)."""
+    r = slice_ranges(x.dims, starts, ends, axes, steps)
+    shape = [n for (_, _, n) in r]
+    y = ctx.empty_tensor(shape, x.data_type)
+    if y.length:
+        xs = _dense_strides(x.dims)
+        _strided_copy(x, sum(st * s for (st, _, _), s in zip(r, xs)), y, 0, shape,
+                      [step * s for (_, step, _), s in zip(r, xs)], _dense_strides(shape))
+    return y
+
+
+_CAST_TO = {1: "float32", 2: "int32", 6: "int32", 7: "int32"}
+
+
+def cast(ctx, x, to):
+    """cpu cast.ts:12-52 (`to` is an ONNX TensorProto.DataType)."""
+    if to not in _CAST_TO:
+        raise OperatorError("Cast: converting to DataType %d is not yet supported" % to)
+    dt = _CAST_TO[to]
+    y = ctx.empty_tensor(x.dims, dt)
+    call("wdh_cast", 0 if x.data_type == "float32" else 1, 0 if dt == "float32" else 1,
+         x.handle, y.handle, x.length)
+    return y

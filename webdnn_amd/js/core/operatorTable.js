@@ -43,15 +43,21 @@ function instantiateOperator(opType, opset, backendOrder, currentTensorsBackends
       break;
   }
 
-  for (const backend of localBackendOrder) {
-    for (const entry of entries) {
-      if (entry.backend !== backend) continue;
-      if (entry.opsetMin > opset) continue;
-      if (entry.opsetMax != null && entry.opsetMax <= opset) continue;
-      return entry.factory();
+  const pick = (order) => {
+    for (const backend of order) {
+      for (const entry of entries) {
+        if (entry.backend !== backend) continue;
+        if (entry.opsetMin > opset) continue;
+        if (entry.opsetMax != null && entry.opsetMax <= opset) continue;
+        return entry.factory();
+      }
     }
-  }
-  return null;
+    return null;
+  };
+  // A layout operator whose data sits on a backend without an implementation of it (a
+  // model input reshaped before any device operator touched it: this package ships no cpu
+  // Reshape) is placed by the ordinary order instead; the runner then moves the tensor.
+  return pick(localBackendOrder) || (localBackendOrder !== backendOrder ? pick(backendOrder) : null);
 }
 
 module.exports = { registerOperators, instantiateOperator, clearOperators };

@@ -78,6 +78,8 @@ def attribute(name, value):
         return out + _len(4, value.encode("utf-8")) + _int(20, ATTR_STRING)
     if isinstance(value, (list, tuple)):
         return out + _packed_ints(8, value) + _int(20, ATTR_INTS)
+    if isinstance(value, np.ndarray):
+        return out + _len(5, tensor_proto("", value)) + _int(20, ATTR_TENSOR)
     raise TypeError("unsupported attribute %r" % (value,))
 
 
@@ -184,6 +186,8 @@ def parse_model(data):
                 value = _signed(v)
             elif f == 4:
                 value = bytes(v).decode()
+            elif f == 5:
+                value = parse_tensor(v)[1]
             elif f == 8:
                 value = (value or []) + _ints(w, v)
         return name, value
@@ -262,7 +266,9 @@ class GraphBuilder:
         return name
 
     def op(self, op_type, inputs, output, **attrs):
-        self.nodes.append(node(op_type, inputs, [output], "%s_%d" % (op_type, len(self.nodes)), **attrs))
+        """`output` is one tensor name, or a list of them for a multi-output operator (Split)."""
+        outputs = list(output) if isinstance(output, (list, tuple)) else [output]
+        self.nodes.append(node(op_type, inputs, outputs, "%s_%d" % (op_type, len(self.nodes)), **attrs))
         return output
 
     def finish(self, inputs, outputs, opset=13):
@@ -483,3 +489,48 @@ def detr_model(image=(800, 1088), d=256, heads=8, ffn=2048, enc_layers=6, dec_la
     data = g.finish([("input", [1, 3, image[0], image[1]])], [("logits", [queries, classes]), ("boxes", [queries, 4])],
                     opset=17)
     return data, g
+
+
+def glue_model(opset=11, seed=0):
+    """Shape arithmetic and layout glue as ONNX exporters emit around attention blocks:
+    Shape -> Gather -> Unsqueeze -> Concat -> Reshape on the metadata side, and
+    Split / Concat / Slice / Cast / Squeeze / Unsqueeze on the data.  `opset` below 13 puts
+    axes/split in attributes, 13 and above passes them as input tensors."""
+    g = GraphBuilder(seed)
+    as_input = opset >= 13
+    i64 = lambda *v: np.array(v, np.int64)
+
+    def unsqueeze(x, axes, out):
+        if as_input:
+            return g.op("Unsqueeze", [x, g.const(out + "_axes", i64(*axes))], out)
+        return g.op("Unsqueeze", [x], out, axes=list(axes))
+
+    def squeeze(x, axes, out):
+        if as_input:
+            return g.op("Squeeze", [x, g.const(out + "_axes", i64(*axes))], out)
+        return g.op("Squeeze", [x], out, axes=list(axes))
+
+    # metadata side: [batch, -1] computed from the input's shape
+    g.op("Shape", ["X"], "shape")
+    g.op("Gather", ["shape", g.const("zero", np.array(0, np.int64))], "batch", axis=0)
+    unsqueeze("batch", [0], "batch1")
+    g.op("Constant", [], "minus1", value=i64(-1))
+    g.op("Concat", ["batch1", "minus1"], "flat_shape", axis=0)
+    g.op("Reshape", ["X", "flat_shape"], "flat")                       # [2, 120]
+    # data side
+    if as_input:
+        g.op("Split", ["flat", g.const("parts", i64(40, 30, 50))], ["a", "b", "c"], axis=1)
+    else:
+        g.op("Split", ["flat"], ["a", "b", "c"], axis=1, split=[40, 30, 50])
+    g.op("Concat", ["c", "a", "b"], "cat", axis=-1)                    # [2, 120], bands rotated
+    g.op("Slice", ["cat", g.const("st", i64(1)), g.const("en", i64(-1)), g.const("ax", i64(1)),
+                   g.const("sp", i64(2))], "sl")                       # [2, 59]
+    g.op("Mul", ["sl", g.const("hundred", np.array(100.0, np.float32))], "scaled")
+    g.op("Cast", ["scaled"], "ints", to=INT32)
+    g.op("Cast", ["ints"], "floats", to=FLOAT)
+    unsqueeze("floats", [0, 3], "u")                                   # [1, 2, 59, 1]
+    squeeze("u", [3], "s")                                             # [1, 2, 59]
+    g.op("Slice", ["s", g.const("st2", i64(-1, 58)), g.const("en2", i64(-100, -100)),
+                   g.const("ax2", i64(1, 2)), g.const("sp2", i64(-1, -3))], "rev")   # [1, 2, 20]
+    g.op("Add", ["rev", g.const("bias", g.rng().standard_normal(20).astype(np.float32))], "Y")
+    return g.finish([("X", [2, 6, 4, 5])], [("Y", [1, 2, 20]), ("ints", [2, 59])], opset), g

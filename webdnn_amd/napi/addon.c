@@ -363,6 +363,27 @@ FN(js_gather) {
   return make_undefined(env);
 }
 
+FN(js_cast) {
+  ARGS("wdh_cast", 5);
+  I64(0, from); I64(1, to); I64(2, X); I64(3, Y); I64(4, length);
+  CHECK(wdh_cast((int)from, (int)to, X, Y, (size_t)length));
+  return make_undefined(env);
+}
+
+FN(js_strided_copy) { /* (X, xOffset, Y, yOffset, shape[], xStrides[], yStrides[]) */
+  ARGS("wdh_strided_copy", 7);
+  I64(0, X); I64(1, xoff); I64(2, Y); I64(3, yoff);
+  int64_t shape64[8], sx[8], sy[8];
+  int nd = 0, n2 = 0, n3 = 0;
+  if (!to_i64_list(env, argv[4], shape64, 8, &nd) || !to_i64_list(env, argv[5], sx, 8, &n2) ||
+      !to_i64_list(env, argv[6], sy, 8, &n3) || n2 != nd || n3 != nd)
+    return throw_arg(env, FNAME, "shape and strides must be integer arrays of equal length (<= 8)");
+  int32_t shape[8];
+  for (int i = 0; i < nd; i++) shape[i] = (int32_t)shape64[i];
+  CHECK(wdh_strided_copy(X, xoff, Y, yoff, nd, shape, sx, sy));
+  return make_undefined(env);
+}
+
 static napi_value init_module(napi_env env, napi_value exports) {
   static const struct {
     const char *name;
@@ -375,7 +396,8 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"gemm", js_gemm}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
       {"softmax", js_softmax}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
-      {"transpose", js_transpose}, {"gather", js_gather},
+      {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
+      {"stridedCopy", js_strided_copy},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {
     napi_value fn;
