@@ -138,3 +138,27 @@ def test_export_style_glue_graph(tmp_path, opset):
     want = graph_ref.run_graph(model, {"X": X})
     assert_bit_exact(hip[0], want["Y"], "Y")
     assert_bit_exact(hip[1], want["ints"], "ints")
+
+
+def test_optimized_model_directory(tmp_path):
+    """model-hip.onnx + WDN2 weight files (raw and 8-bit coded) through WebDNN.load({optimized: true})."""
+    from webdnn_amd import tensor_export
+    data, _ = modelgen.resnet50_model(batch=4, image=64, width=16, blocks=(1, 1, 1, 1), classes=10)
+    X = np.random.default_rng(2).standard_normal((4, 3, 64, 64)).astype(np.float32)
+    model, want, _ = run_both(tmp_path, data, {"input": X})
+    raw = tmp_path / "raw"
+    tensor_export.export_model_directory(str(raw), data, split_size=100000)
+    got, rep = node_runner.run_model(str(raw), [X], "hip", strict=True, extra=["--optimized"])
+    assert_bit_exact(got[0], want[0], "raw weight files")
+    assert list(rep["stats"]["nodesByBackend"]) == ["hip"]
+    # 8-bit coded weights: the same graph with the weights the reader reconstructs
+    coded = tmp_path / "coded"
+    _, paths = tensor_export.export_model_directory(str(coded), data, split_size=0, compression_algorithm=1)
+    got8, _ = node_runner.run_model(str(coded), [X], "hip", strict=True, extra=["--optimized"])
+    decoded = tensor_export.load_tensors(paths)
+    stripped, _ = modelgen.strip_initializers(data)
+    m = modelgen.parse_model(stripped)
+    m["initializers"] = decoded
+    ref8 = graph_ref.run_graph(m, {"input": X})
+    out_name = model["outputs"][0][0]
+    assert_close_max(got8[0], ref8[out_name], 1e-3, "8-bit coded weights")

@@ -2,7 +2,7 @@
 "use strict";
 // Runs an ONNX model directory through the descriptor runner from the command line.
 //
-//   node run_model.js --model DIR [--onnx model.onnx] [--backend hip|cpu]
+//   node run_model.js --model DIR [--onnx model.onnx | --optimized] [--backend hip|cpu]
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
@@ -23,7 +23,7 @@ const WebDNN = require("../index");
 const { registerOperators } = require("../core/operatorTable");
 
 function parseArgs(argv) {
-  const args = { backend: "hip", warmup: 0, runs: 1, onnx: "model.onnx" };
+  const args = { backend: "hip", warmup: 0, runs: 1, onnx: null };
   for (let i = 2; i < argv.length; i++) {
     const a = argv[i];
     const next = () => {
@@ -32,6 +32,7 @@ function parseArgs(argv) {
     };
     if (a === "--model") args.model = next();
     else if (a === "--onnx") args.onnx = next();
+    else if (a === "--optimized") args.optimized = true;
     else if (a === "--backend") args.backend = next();
     else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
     else if (a === "--output") args.output = next();
@@ -61,6 +62,7 @@ async function main() {
     backendOrder: args.backend === "cpu" ? ["cpu"] : ["hip", "cpu"],
     backendOptions: { hip: hipOption },
     onnxBaseName: args.onnx,
+    optimized: !!args.optimized,
   });
   if (args.backend === "hip" && runner.backendName !== "hip") {
     throw new Error("hip backend was requested but is not available");

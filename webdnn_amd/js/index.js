@@ -64,7 +64,10 @@ async function load(directory, options) {
     strict: !!hipOption.strict,
     fuse: hipOption.fuse,
   });
-  await runner.loadModel(directory, opts.onnxBaseName || "model.onnx");
+  // An optimized-model directory holds one graph per backend, named after it, and keeps the
+  // weights in WDN2 tensor files (separateBuild/coreOnly.ts:200-204).
+  const baseName = opts.onnxBaseName || (opts.optimized ? `model-${succeedBackend}.onnx` : "model.onnx");
+  await runner.loadModel(directory, baseName);
   return runner;
 }
 

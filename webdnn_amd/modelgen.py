@@ -534,3 +534,30 @@ def glue_model(opset=11, seed=0):
                    g.const("ax2", i64(1, 2)), g.const("sp2", i64(-1, -3))], "rev")   # [1, 2, 20]
     g.op("Add", ["rev", g.const("bias", g.rng().standard_normal(20).astype(np.float32))], "Y")
     return g.finish([("X", [2, 6, 4, 5])], [("Y", [1, 2, 20]), ("ints", [2, 59])], opset), g
+
+
+# ------------------------------------------------------------------ model surgery for optimized-model directories
+def _reencode(field, wire, v):
+    if wire == 0:
+        return _tag(field, 0) + _varint(v)
+    if wire == 2:
+        return _len(field, bytes(v))
+    return _tag(field, wire) + bytes(v)
+
+
+def strip_initializers(model_bytes):
+    """-> (the model without graph.initializer entries, {name: array} of what was removed)."""
+    tensors = parse_model(model_bytes)["initializers"]
+    out = b""
+    for f, w, v in _fields(memoryview(model_bytes)):
+        if f == 7 and w == 2:
+            graph = b"".join(_reencode(gf, gw, gv) for gf, gw, gv in _fields(v) if gf != 5)
+            out += _len(7, graph)
+        else:
+            out += _reencode(f, w, v)
+    return out, tensors
+
+
+def add_metadata(model_bytes, metadata):
+    """Appends ModelProto.metadata_props entries (key/value strings)."""
+    return bytes(model_bytes) + b"".join(_len(14, _str(1, k) + _str(2, v)) for k, v in metadata.items())
