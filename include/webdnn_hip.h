@@ -70,9 +70,9 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       wdh_gemm / wdh_conv2d (a tuning and test hook: every
  *                       tile shape computes the same result).
  *   "split_k"           -1 = choose per problem (default); n >= 1 = cut the
- *                       K loop of wdh_gemm / wdh_conv2d into n chunks whose
- *                       partial sums are added in chunk order by a second
- *                       kernel (1 = never split). */
+ *                       K loop of every tile of wdh_gemm / wdh_conv2d into n
+ *                       chunks whose partial sums are added in chunk order
+ *                       by a second kernel (1 = never split). */
 int wdh_set_option(const char *name, int value);
 
 /* ---- buffers --------------------------------------------------------- */

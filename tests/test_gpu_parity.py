@@ -615,7 +615,7 @@ def test_every_tile_shape_computes_the_same(ctx, tile):
 
 @pytest.mark.parametrize("split", [1, 2, 5, 64])
 def test_split_k_is_the_same_sum(ctx, split):
-    """Split-K cuts the K loop into chunks reduced by a second kernel in chunk order."""
+    """Split-K cuts the K loop into chunks whose sums a second kernel adds in chunk order."""
     A, B, C = uni(70, 333), uni(333, 90), uni(90)
     X, W, Bv, R = uni(2, 40, 7, 7, lo=0), he(24, 40, 3), nrm(24), nrm(2, 24, 7, 7)
     A3, B3 = nrm(3, 50, 200), nrm(3, 200, 30)
@@ -632,6 +632,20 @@ def test_split_k_is_the_same_sum(ctx, split):
     assert_close_max(c, want, GEMM_TOL, "conv split %d" % split)
     assert_close_max(m3, ref.matmul(A3, B3), GEMM_TOL, "batched matmul split %d" % split)
     assert cg.shape == (1, 6, 7, 7)
+
+
+def test_planned_splits_are_deterministic_and_match_forced_ones(ctx):
+    """Tail tiles beyond full rounds (ResNet stage 1/2 forms) and all-tile splits (stage 3/4 forms):
+    chunks are added in index order, so repeated runs agree bit for bit."""
+    cases = [(uni(8, 128, 28, 28, lo=0), he(128, 128, 3), nrm(128), [1, 1, 1, 1]),
+             (uni(32, 64, 56, 56, lo=0), he(64, 64, 3), nrm(64), [1, 1, 1, 1]),
+             (uni(4, 512, 7, 7, lo=0), he(512, 512, 3), nrm(512), [1, 1, 1, 1]),
+             (uni(8, 1024, 14, 14, lo=0), he(256, 1024, 1), nrm(256), [0, 0, 0, 0])]
+    for X, W, Bv, pads in cases:
+        outs = [hip_conv(ctx, X, W, Bv, pads=pads, epilogue="relu") for _ in range(3)]
+        for o in outs[1:]:
+            assert_bit_exact(o, outs[0], "conv %s" % (X.shape,))
+        assert_close_max(outs[0], ref.unary("Relu", ref.conv(X, W, Bv, pads=pads)), GEMM_TOL)
 
 
 def test_split_k_auto_on_deep_small_layers(ctx):

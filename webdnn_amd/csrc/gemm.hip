@@ -134,6 +134,7 @@ struct Params {
   // sums go to `partial` and are added up by splitk_reduce_kernel.
   int nz;
   int full_tiles;
+  int tail_tiles;
   int tail_split;   // 1: no tile is split
   int kchunk;       // a multiple of 16
   float *partial;   // [tail tile][chunk][BM][BN]
@@ -348,6 +349,41 @@ __device__ __forceinline__ void stash_im2col_fast(float *tile, int tid,
 
 constexpr int tile_floats(bool kc, int ext) { return kc ? ext * LDK : BK * (ext + MC_PAD); }
 
+// ---- adding up the chunks of a tail tile ---------------------------------------
+// Four consecutive columns (tile-local element e .. e+3) of tail tile j: the
+// chunks' partial sums are added in index order, then alpha, bias, residual
+// and Relu are applied as in the whole-tile epilogue.
+template <bool CONV>
+__device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int j, int bz,
+                                            int tm, int tn, int e) {
+  const int lr = e / bn, lc = e - lr * bn;
+  const int row = tm * bm + lr;
+  if (row >= p.m) return;
+  const float *part = p.partial + (long long)j * p.tail_split * (bm * bn) + e;
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int c = 0; c < p.tail_split; c++)
+    acc += *reinterpret_cast<const f32x4 *>(part + (long long)c * (bm * bn));
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int col = tn * bn + lc + i;
+    if (col >= p.n) break;
+    float y = p.alpha * acc[i];
+    long long off;
+    if (CONV) {
+      const int ohw = p.cv.oh * p.cv.ow;
+      const int img = col / ohw, q = col - img * ohw;
+      off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
+      if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
+    } else {
+      off = ((long long)bz * p.m + row) * p.n + col;
+      if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
+    }
+    if (p.R) y = y + p.R[off];
+    if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+    p.Y[off] = y;
+  }
+}
+
 // ---- the kernel -------------------------------------------------------------
 // Workgroups per CU the register budget must allow: the 64-accumulator tiles
 // are held to 128 registers so that four of them share a CU, the
@@ -384,9 +420,11 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   if (whole) {
     lin = xcd_contiguous(pid, p.full_tiles);
   } else {
-    const int c = pid - p.full_tiles;
-    lin = p.full_tiles + c / p.tail_split;
-    chunk = c % p.tail_split;
+    // chunk workgroups: an XCD takes a contiguous run of (chunk, tile) pairs with the
+    // tile varying fastest, so that tiles which share a slice of B meet in one L2
+    const int v = xcd_contiguous(pid - p.full_tiles, p.tail_tiles * p.tail_split);
+    chunk = v / p.tail_tiles;
+    lin = p.full_tiles + (v - chunk * p.tail_tiles);
   }
   const int tiles_per_z = p.tiles_m * p.tiles_n;
   const int bz = lin / tiles_per_z;  // batch entry (gemm) or group (conv)
@@ -634,7 +672,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
           const int lr = wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
           part[lr * BN + wcol + nt * 32 + li] = acc[mt][nt][r];
         }
-    return;
+    return;  // splitk_reduce_kernel adds the chunks up
   }
   // Bias and residual values of a 32x32 block are all requested before the
   // first is used, so the block pays one memory round trip, not thirty-two.
@@ -727,33 +765,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int bm, in
   const int bz = lin / tiles_per_z;
   int tm, tn;
   tile_coords(lin - bz * tiles_per_z, p.tiles_m, p.tiles_n, &tm, &tn);
-  const int e = ((int)blockIdx.y * 256 + (int)threadIdx.x) * 4;
-  const int lr = e / bn, lc = e - lr * bn;
-  const int row = tm * bm + lr;
-  if (row >= p.m) return;
-  const float *part = p.partial + (long long)j * p.tail_split * (bm * bn) + e;
-  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int c = 0; c < p.tail_split; c++)
-    acc += *reinterpret_cast<const f32x4 *>(part + (long long)c * (bm * bn));
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int col = tn * bn + lc + i;
-    if (col >= p.n) break;
-    float y = p.alpha * acc[i];
-    long long off;
-    if (CONV) {
-      const int ohw = p.cv.oh * p.cv.ow;
-      const int img = col / ohw, q = col - img * ohw;
-      off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
-      if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
-    } else {
-      off = ((long long)bz * p.m + row) * p.n + col;
-      if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
-    }
-    if (p.R) y = y + p.R[off];
-    if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
-    p.Y[off] = y;
-  }
+  reduce_quad<CONV>(p, bm, bn, j, bz, tm, tn, ((int)blockIdx.y * 256 + (int)threadIdx.x) * 4);
 }
 
 // ---- host-side dispatch -------------------------------------------------------
@@ -839,7 +851,7 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
     double t = work > solo * longest ? work : solo * longest;
     // reduce pass: a launch plus the partial sums written and read back (mostly
     // through the last-level cache, ~8 TB/s)
-    if (s > 1) t += 3.0 + 2.0 * tail * s * tile_bytes / 8.0e6;
+    if (s > 1) t += 6.0 + 2.0 * tail * s * tile_bytes / 8.0e6;
     return t;
   };
   const long long rem = tiles % cus;
@@ -876,6 +888,7 @@ int launch_tile(Params &p, int nz, bool vec) {
     return wdh::fail(WDH_EINVAL, "contraction: %lld workgroups exceed the grid limit", blocks);
   p.nz = nz;
   p.full_tiles = (int)w.full;
+  p.tail_tiles = (int)w.tail;
   p.tail_split = w.split;
   p.kchunk = w.kchunk;
   wdh_buf scratch = 0;
