@@ -176,13 +176,66 @@ def bench_kernels(steps, warmup, calibrate_copy=False):
     }
 
 
+def bench_bandwidth(steps, warmup):
+    """GB/s of the HBM-bound kernels at the shapes the configs use: algorithmic bytes (every input and
+    output element once) over the average launch time, against the 8 TB/s peak."""
+    from webdnn_amd import hostops as H
+
+    ctx = H.HipContext(0).initialize()
+    rng = np.random.default_rng(0)
+    f = lambda *shape: ctx.move_tensor(rng.standard_normal(shape).astype(np.float32))
+    out = {}
+
+    def run(name, workload, nbytes, fn):
+        ms = timed_steps(ctx, fn, steps, warmup)
+        gbs = nbytes / ms / 1e6
+        out[name] = {"workload": workload, "ms": round(ms, 4), "GB/s": round(gbs, 1),
+                     "frac_hbm_peak": round(gbs / 8000.0, 4)}
+
+    x = f(32, 256, 56, 56)
+    y = f(32, 256, 56, 56)
+    n = x.length * 4
+    run("add", "Add [32,256,56,56] + same shape (ResNet residual)", 3 * n, lambda: H.binary(ctx, "Add", x, y).dispose())
+    b = f(256, 1, 1)
+    run("add_bcast", "Add [32,256,56,56] + [256,1,1]", 2 * n, lambda: H.binary(ctx, "Add", x, b).dispose())
+    run("relu", "Relu [32,256,56,56]", 2 * n, lambda: H.unary(ctx, "Relu", x).dispose())
+    x.dispose(); y.dispose()
+    s = f(8, 850, 850)
+    run("softmax", "Softmax [8,850,850] (DETR encoder attention)", 2 * s.length * 4, lambda: H.softmax(ctx, s).dispose())
+    s.dispose()
+    ln, g, be = f(32 * 850, 256), f(256), f(256)
+    run("layernorm", "LayerNormalization [27200,256]", 2 * ln.length * 4,
+        lambda: H.layer_normalization(ctx, ln, g, be).dispose())
+    ln.dispose()
+    st = f(32, 64, 112, 112)
+    run("maxpool", "MaxPool 3x3 s2 p1 [32,64,112,112] (ResNet stem)", st.length * 4 + 32 * 64 * 56 * 56 * 4,
+        lambda: H.maxpool(ctx, st, kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2]).dispose())
+    st.dispose()
+    gp = f(32, 2048, 7, 7)
+    run("global_avgpool", "GlobalAveragePool [32,2048,7,7]", gp.length * 4 + 32 * 2048 * 4,
+        lambda: H.global_average_pool(ctx, gp).dispose())
+    gp.dispose()
+    t = f(32, 850, 8, 32)
+    run("transpose", "Transpose [32,850,8,32] perm (0,2,1,3) (attention heads)", 2 * t.length * 4,
+        lambda: H.transpose(ctx, t, [0, 2, 1, 3]).dispose())
+    run("transpose_last", "Transpose [32,850,8,32] perm (0,2,3,1) (K^T, through LDS tiles)", 2 * t.length * 4,
+        lambda: H.transpose(ctx, t, [0, 2, 3, 1]).dispose())
+    t.dispose()
+    c1, c2 = f(32, 128, 56, 56), f(32, 128, 56, 56)
+    run("concat", "Concat 2 x [32,128,56,56] on axis 1", 4 * c1.length * 4, lambda: H.concat(ctx, [c1, c2], 1).dispose())
+    run("slice", "Slice [32,128,56,56] -> [32,128,48,50]", 2 * 32 * 128 * 48 * 50 * 4,
+        lambda: H.slice_(ctx, c1, [4, 3], [52, 53], [2, 3]).dispose())
+    c1.dispose(); c2.dispose()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "kernels"], default="all",
+    ap.add_argument("--only", choices=["all", "kernels", "bandwidth"], default="all",
                     help="kernels: only the in-process Gemm 4096 / Conv C3 launches plus one device-to-device "
                          "copy of known size (the unit for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -190,6 +243,10 @@ def main():
         sys.exit("bench.py: this build runs on exactly one GPU (the path shards by batch with no "
                  "exchange; multi-GPU runs are not part of it). Use --gpus 1.")
 
+    if args.only == "bandwidth":
+        print(json.dumps({"bandwidth_kernels": bench_bandwidth(args.steps, args.warmup),
+                          "unit": "GB/s of algorithmic bytes", "peak": 8000.0}))
+        return
     if args.only == "kernels":
         print(json.dumps({"kernels": bench_kernels(args.steps, args.warmup, calibrate_copy=True)}))
         return

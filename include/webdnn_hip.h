@@ -105,6 +105,25 @@ int wdh_mem_stats(uint64_t *in_use, uint64_t *cached, uint64_t *peak);
  * backend/webgl/webglContextImpl.ts:541-568). */
 int wdh_trim(size_t keep_bytes);
 
+/* ---- captured runs --------------------------------------------------------
+ * The reference runs its node loop in JavaScript on every RunnerImpl.run
+ * (core/runnerImpl.ts:377-542); here the device work of one run can be recorded
+ * once into a HIP graph and replayed with a single launch.
+ * Between wdh_graph_begin and wdh_graph_end every operator entry point, wdh_copy,
+ * wdh_alloc and wdh_free records instead of executing; blocks allocated meanwhile
+ * become the graph's own memory (recycled among its tensors, lent to nobody else)
+ * until wdh_graph_destroy.  Calls that need the host to see device data or the
+ * stream to drain (wdh_write, wdh_read, wdh_sync, wdh_trim, events, the first
+ * wdh_conv2d of a geometry) fail with WDH_ESTATE and make wdh_graph_end fail:
+ * run the model once eagerly first.  Buffers that exist before the capture
+ * (weights, inputs) and handles still held after it (outputs) are what a replay
+ * reads and writes: refill the inputs with wdh_write, call wdh_graph_launch, read
+ * the outputs with wdh_read. */
+int wdh_graph_begin(void);
+int wdh_graph_end(int *graph_id);
+int wdh_graph_launch(int graph_id);
+int wdh_graph_destroy(int graph_id);
+
 /* ---- timing (measurePerformance, core/runnerImpl.ts:368-375,533-541) -- */
 
 #define WDH_MAX_EVENTS 4096

@@ -11,6 +11,7 @@ const buffers = new Map();
 let nextHandle = 1;
 let inUse = 0, peak = 0;
 const calls = {};
+const graphOwned = new Set(); // handles freed while capturing: their memory stays with the graph
 const options = {};
 
 function count(name) {
@@ -265,9 +266,11 @@ const native = {
     }
   },
 
+  // ---- captured runs: see the wrapper below ----
+
   // ---- test introspection ----
   __liveBuffers() {
-    return buffers.size;
+    return buffers.size - graphOwned.size;
   },
   __calls() {
     return Object.assign({}, calls);
@@ -275,6 +278,77 @@ const native = {
   __options() {
     return Object.assign({}, options);
   },
+};
+
+// ---- captured runs --------------------------------------------------------------------
+// Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
+// alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
+// calls that need device data on the host throw and spoil the capture.
+const RECORDED = ["copy", "gemm", "conv2d", "binary", "unary", "softmax", "layernorm", "reduceMean", "maxpool2d",
+  "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
+const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
+const graphs = new Map();
+let capture = null, nextGraph = 0;
+for (const name of RECORDED) {
+  const real = native[name];
+  native[name] = function (...args) {
+    if (!capture) return real.apply(native, args);
+    // arrays are copied: the caller may reuse them
+    capture.ops.push([real, args.map((a) => (Array.isArray(a) ? a.slice() : a))]);
+    return undefined;
+  };
+}
+for (const name of REFUSED) {
+  const real = native[name];
+  native[name] = function (...args) {
+    if (capture) {
+      capture.failed = true;
+      throw new Error(`wdh_${name} failed (-5): not possible while a graph is being captured`);
+    }
+    return real.apply(native, args);
+  };
+}
+const realFree = native.free;
+native.free = function (h) {
+  if (!capture) return realFree.call(native, h);
+  count("free");
+  buf(h, "wdh_free");
+  capture.freed.push(h);
+  graphOwned.add(h);
+  return undefined;
+};
+native.graphBegin = function () {
+  if (capture) throw new Error("wdh_graph_begin failed (-5): a capture is already open");
+  capture = { ops: [], freed: [], failed: false };
+};
+function dropGraphBuffers(g) {
+  for (const h of g.freed) {
+    graphOwned.delete(h);
+    realFree.call(native, h);
+  }
+}
+native.graphEnd = function () {
+  if (!capture) throw new Error("wdh_graph_end failed (-5): no capture is open");
+  const g = capture;
+  capture = null;
+  if (g.failed) {
+    dropGraphBuffers(g);
+    throw new Error("wdh_graph_end failed (-5): the capture was abandoned");
+  }
+  graphs.set(nextGraph, g);
+  return nextGraph++;
+};
+native.graphLaunch = function (id) {
+  count("graphLaunch");
+  const g = graphs.get(id);
+  if (!g) throw new Error(`wdh_graph_launch failed (-2): unknown graph ${id}`);
+  for (const [fn, args] of g.ops) fn.apply(native, args);
+};
+native.graphDestroy = function (id) {
+  const g = graphs.get(id);
+  if (!g) throw new Error(`wdh_graph_destroy failed (-2): unknown graph ${id}`);
+  graphs.delete(id);
+  dropGraphBuffers(g);
 };
 
 module.exports = native;

@@ -560,6 +560,90 @@ def test_buffers_offsets_large_copies_and_pool(ctx):
     z.dispose()
 
 
+def _small_net(ctx, x, w1, b1, w2, b2, wf, bf):
+    """conv+relu -> maxpool -> conv+residual+relu -> global pool -> flatten -> gemm; every tensor but the
+    result is disposed on the way, as the runner does."""
+    a = H.conv(ctx, x, w1, b1, pads=[1, 1, 1, 1], epilogue="relu")
+    p = H.maxpool(ctx, a, kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2])
+    a.dispose()
+    c = H.conv(ctx, p, w2, b2, pads=[1, 1, 1, 1], epilogue="relu", residual=p)
+    p.dispose()
+    g = H.global_average_pool(ctx, c)
+    c.dispose()
+    f = H.flatten(ctx, g)
+    g.dispose()
+    y = H.gemm(ctx, f, wf, bf, trans_b=1)
+    f.dispose()
+    return y
+
+
+def test_captured_graph_replays_like_eager_runs(ctx):
+    """One run recorded into a HIP graph, then replayed with new input contents; every replay is
+    compared with an eager run of the same input, with eager work, syncs and pool traffic in between."""
+    x_np = [uni(4, 16, 28, 28, lo=0) for _ in range(4)]
+    w1, b1 = ctx.move_tensor(he(32, 16, 3)), ctx.move_tensor(nrm(32))
+    w2, b2 = ctx.move_tensor(he(32, 32, 3)), ctx.move_tensor(nrm(32))
+    wf, bf = ctx.move_tensor(nrm(10, 32)), ctx.move_tensor(nrm(10))
+    x = ctx.move_tensor(x_np[0])
+    eager = []
+    for xn in x_np:                                   # also warms the pool and the conv tap tables
+        x.set_data(xn)
+        y = _small_net(ctx, x, w1, b1, w2, b2, wf, bf)
+        eager.append(y.get_data())
+        y.dispose()
+    before = ctx.mem_stats()
+    x.set_data(x_np[0])
+    ctx.graph_begin()
+    y = _small_net(ctx, x, w1, b1, w2, b2, wf, bf)    # recorded, not executed
+    gid = ctx.graph_end()
+    for i in (0, 1, 2, 3, 1):
+        x.set_data(x_np[i])
+        ctx.graph_launch(gid)
+        assert_bit_exact(y.get_data(), eager[i], "replay with input %d" % i)
+        # unrelated eager work between replays must neither disturb nor be disturbed
+        other = H.conv(ctx, x, w1, b1, pads=[1, 1, 1, 1])
+        junk = [ctx.move_tensor(nrm(64, 1024)) for _ in range(3)]
+        want_other = other.get_data()
+        ctx.graph_launch(gid)
+        assert_bit_exact(other.get_data(), want_other, "an eager tensor survives a replay")
+        assert_bit_exact(y.get_data(), eager[i], "second replay with input %d" % i)
+        other.dispose()
+        for j in junk:
+            j.dispose()
+    held = ctx.mem_stats()["in_use"]
+    ctx.graph_destroy(gid)
+    assert ctx.mem_stats()["in_use"] < held                        # the graph's blocks went back to the pool
+    assert_bit_exact(y.get_data(), eager[1], "the output handle outlives the graph")
+    y.dispose()
+    assert ctx.mem_stats()["in_use"] == before["in_use"]
+    with pytest.raises(capi.HipError):
+        ctx.graph_launch(gid)
+
+
+def test_capture_refuses_what_cannot_be_recorded(ctx):
+    x = ctx.move_tensor(uni(1, 4, 9, 9))
+    ctx.graph_begin()
+    with pytest.raises(capi.HipError) as err:
+        x.get_data()                                               # a read needs the stream drained
+    assert err.value.code == -5
+    with pytest.raises(capi.HipError) as err:
+        ctx.graph_end()
+    assert "abandoned" in str(err.value)
+    # a conv geometry never run before needs its tap table built, which cannot happen while capturing
+    w = ctx.move_tensor(he(5, 4, 3))
+    ctx.graph_begin()
+    with pytest.raises(capi.HipError) as err:
+        H.conv(ctx, x, w, None, pads=[2, 2, 2, 2], dilations=[2, 2])
+    assert "once before capturing" in str(err.value)
+    with pytest.raises(capi.HipError):
+        ctx.graph_end()
+    with pytest.raises(capi.HipError):
+        ctx.graph_end()                                            # no capture open any more
+    # the library is usable afterwards
+    y = H.conv(ctx, x, w, None, pads=[2, 2, 2, 2], dilations=[2, 2])
+    assert y.get_data().shape == (1, 5, 9, 9)
+
+
 def test_errors_are_reported_not_fatal(ctx):
     with pytest.raises(capi.HipError) as err:
         capi.call("wdh_free", 123456789)

@@ -162,3 +162,43 @@ def test_optimized_model_directory(tmp_path):
     ref8 = graph_ref.run_graph(m, {"input": X})
     out_name = model["outputs"][0][0]
     assert_close_max(got8[0], ref8[out_name], 1e-3, "8-bit coded weights")
+
+
+def _graph_runs(tmp_path, data, a, b, runs):
+    alt = []
+    for i, arr in enumerate(b):
+        p = tmp_path / ("alt_%d.bin" % i)
+        np.ascontiguousarray(arr).tofile(str(p))
+        alt.append(str(p))
+    return node_runner.run_model(str(tmp_path), a, "hip", strict=True, runs=runs,
+                                 extra=["--graph", "--alt-inputs", ",".join(alt)])
+
+
+def test_graph_replay_equals_eager_runs(tmp_path):
+    """runner.run(inputs, {graph: true}): eager warm-up, capture + launch, then replays with inputs that
+    change from run to run; every compared run must equal the eager run of the same input bit for bit
+    (same kernels, same order)."""
+    data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    ea, _ = node_runner.run_model(str(tmp_path), [Xa], "hip", strict=True)
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True)
+    for runs, want in ((2, eb), (3, ea), (6, eb), (7, ea)):
+        got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs)
+        assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
+        assert rep["stats"]["graphReplay"] is True
+        assert_bit_exact(got[0], want[0], "run %d of a graph-mode session" % runs)
+
+
+def test_graph_replay_detr_style(tmp_path):
+    data, g = modelgen.detr_model(image=(128, 160), d=64, heads=8, ffn=128, enc_layers=2, dec_layers=2, queries=20,
+                                  classes=11, width=16, blocks=(1, 1, 1, 1))
+    Xa = np.random.default_rng(9).standard_normal((1, 3, 128, 160)).astype(np.float32)
+    Xb = np.random.default_rng(10).standard_normal((1, 3, 128, 160)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True)
+    got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], 4)
+    assert rep["graph"]["captured"] is True
+    for g_, w in zip(got, eb):
+        assert_bit_exact(g_, w, "DETR-style graph, fourth run")

@@ -180,3 +180,47 @@ def test_export_style_glue_graph(tmp_path, opset):
         assert_bit_exact(got_hip, want[name], name + ": vs the python oracle")
     assert hip[1].dtype == np.int32
     assert rep["liveBuffers"] == rep["initializerCopies"]
+
+
+def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native):
+    """Runs 1..4 with {graph: true}: eager warm-up, capture + launch, replay, replay; even runs use
+    feeds_a, odd runs feeds_b.  Returns (outputs of run 3 (a), outputs of run 4 (b), eager a, eager b, report)."""
+    (tmp_path / "model.onnx").write_bytes(data)
+    model = modelgen.parse_model(data)
+    a = [feeds_a[n] for n, _ in model["inputs"]]
+    b = [feeds_b[n] for n, _ in model["inputs"]]
+    alt = []
+    for i, arr in enumerate(b):
+        p = tmp_path / ("alt_%d.bin" % i)
+        np.ascontiguousarray(arr).tofile(str(p))
+        alt.append(str(p))
+    kw = dict(strict=True, fake_native=fake_native)
+    eager_a, _ = node_runner.run_model(str(tmp_path), a, "hip", **kw)
+    eager_b, _ = node_runner.run_model(str(tmp_path), b, "hip", **kw)
+    g3, rep3 = node_runner.run_model(str(tmp_path), a, "hip", runs=3, extra=["--graph", "--alt-inputs", ",".join(alt)], **kw)
+    g4, rep4 = node_runner.run_model(str(tmp_path), a, "hip", runs=4, extra=["--graph", "--alt-inputs", ",".join(alt)], **kw)
+    return g3, g4, eager_a, eager_b, rep4
+
+
+def test_graph_replay_on_the_host_path(tmp_path):
+    data, _ = modelgen.resnet50_model(batch=2, image=32, width=8, blocks=(1, 1, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    g3, g4, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"input": Xa}, {"input": Xb}, True)
+    assert rep["graph"] == {"captured": True, "unsupported": None}
+    assert rep["stats"]["graphReplay"] is True and list(rep["stats"]["nodesByBackend"]) == ["hip"]
+    assert_bit_exact(g3[0], ea[0], "third run (replay, first input)")
+    assert_bit_exact(g4[0], eb[0], "fourth run (replay, second input)")
+    assert rep["nativeCalls"]["graphLaunch"] == 3
+    assert rep["liveBuffers"] == rep["initializerCopies"]          # the graph's buffers are gone after disposeGraph
+
+
+def test_graph_mode_falls_back_when_the_run_needs_device_data_on_the_host(tmp_path):
+    """The glue graph computes a Reshape shape on the device; reading it back cannot be recorded."""
+    data, _ = modelgen.glue_model(11)
+    X = np.random.default_rng(1).standard_normal((2, 6, 4, 5)).astype(np.float32)
+    g3, g4, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"X": X}, {"X": X * 2}, True)
+    assert rep["graph"]["captured"] is False and "captur" in rep["graph"]["unsupported"]
+    assert_bit_exact(g3[0], ea[0])
+    assert_bit_exact(g4[0], eb[0])
+    assert rep["liveBuffers"] == rep["initializerCopies"]

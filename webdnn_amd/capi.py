@@ -34,6 +34,10 @@ SIGNATURES = {
     "wdh_sync": (_c.c_int, []),
     "wdh_mem_stats": (_c.c_int, [_u64p, _u64p, _u64p]),
     "wdh_trim": (_c.c_int, [_c.c_size_t]),
+    "wdh_graph_begin": (_c.c_int, []),
+    "wdh_graph_end": (_c.c_int, [_c.POINTER(_c.c_int)]),
+    "wdh_graph_launch": (_c.c_int, [_c.c_int]),
+    "wdh_graph_destroy": (_c.c_int, [_c.c_int]),
     "wdh_event_record": (_c.c_int, [_c.c_int]),
     "wdh_event_elapsed_ms": (_c.c_int, [_c.c_int, _c.c_int, _c.POINTER(_c.c_float)]),
     "wdh_gemm": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int, _c.c_int, _c.c_int, _c.c_int,

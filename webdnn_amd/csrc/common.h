@@ -14,6 +14,8 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
 bool initialised();
+bool capturing();        // a graph capture is open on the stream
+void poison_capture();   // the open capture cannot be completed (wdh_graph_end will fail)
 hipStream_t stream();
 int compute_units();
 

@@ -1147,6 +1147,11 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   key.h = h; key.w = w; key.mode = mode;
   auto it = g_ktabs.find(key);
   if (it == g_ktabs.end()) {
+    if (wdh::capturing()) {
+      // building the table takes a synchronous copy
+      wdh::poison_capture();
+      return fail(WDH_ESTATE, "wdh_conv2d: first use of this geometry; run it once before capturing a graph");
+    }
     const int pad_tap = mode == B_IM2COL32 ? 31 : 63;
     std::vector<int2> tab((size_t)((kdim + BK - 1) / BK * BK),
                           mode == B_IM2COL_BIG ? int2{0, 0} : int2{0, pad_tap});

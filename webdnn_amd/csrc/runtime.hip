@@ -26,6 +26,18 @@ struct Slot {
   void *ptr = nullptr;   // nullptr => slot is free
   size_t bytes = 0;      // bytes the caller asked for
   size_t cap = 0;        // bytes of the underlying block
+  int arena = 0;         // > 0: the block belongs to the memory of captured graph arena-1
+};
+
+// A captured run (wdh_graph_begin .. wdh_graph_end).  The addresses of every
+// buffer the run touched are baked into the graph, so the blocks allocated
+// while capturing stay with the graph -- recycled among its own tensors, never
+// handed to anybody else -- until the graph is destroyed.
+struct GraphRec {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::multimap<size_t, void *> free_blocks;  // blocks of this graph not held by a handle
+  bool live = false;
 };
 
 struct Runtime {
@@ -47,6 +59,10 @@ struct Runtime {
   hipEvent_t events[WDH_MAX_EVENTS] = {};
   // one-element dummy so that zero-byte buffers have a valid address
   void *dummy = nullptr;
+  // captured graphs; `capturing` = index + 1 of the one being recorded, 0 = none
+  std::vector<GraphRec> graphs;
+  int capturing = 0;
+  bool capture_failed = false;
 };
 
 Runtime g;
@@ -69,6 +85,22 @@ void release_cache(size_t keep) {
   }
 }
 
+// Returns the blocks of graph `id` that no handle holds to the general pool and
+// hands the rest over to their handles.
+void dissolve_graph(int id) {
+  GraphRec &r = g.graphs[id];
+  if (r.exec) (void)hipGraphExecDestroy(r.exec);
+  if (r.graph) (void)hipGraphDestroy(r.graph);
+  for (auto &kv : r.free_blocks) {
+    g.cache.emplace(kv.first, kv.second);
+    g.cached += kv.first;
+    g.in_use -= kv.first;
+  }
+  for (auto &s : g.slots)
+    if (s.ptr && s.arena == id + 1) s.arena = 0;
+  r = GraphRec();
+}
+
 }  // namespace
 
 namespace wdh {
@@ -83,6 +115,8 @@ int fail(int code, const char *fmt, ...) {
 
 void clear_error() { g_error[0] = '\0'; }
 bool initialised() { return g.ready; }
+bool capturing() { return g.capturing != 0; }
+void poison_capture() { g.capture_failed = true; }
 hipStream_t stream() { return g.stream; }
 int compute_units() { return g.prop.multiProcessorCount; }
 
@@ -162,7 +196,16 @@ int wdh_init(int device) {
 
 void wdh_shutdown(void) {
   if (!g.ready) return;
+  if (g.capturing) {
+    hipGraph_t dropped = nullptr;
+    (void)hipStreamEndCapture(g.stream, &dropped);
+    if (dropped) (void)hipGraphDestroy(dropped);
+    g.capturing = 0;
+  }
   (void)hipStreamSynchronize(g.stream);
+  for (size_t i = 0; i < g.graphs.size(); i++)
+    if (g.graphs[i].live) dissolve_graph((int)i);
+  g.graphs.clear();
   wdh::release_conv_tables();
   for (auto &s : g.slots)
     if (s.ptr && s.ptr != g.dummy) (void)hipFree(s.ptr);
@@ -210,34 +253,50 @@ wdh_buf wdh_alloc(size_t bytes) {
     s.ptr = g.dummy;
     s.cap = 0;
   } else {
-    size_t cap = round_up(bytes);
-    auto it = g.cache.lower_bound(cap);
-    if (it != g.cache.end() && it->first <= cap + cap / 4) {
-      s.ptr = it->second;
-      s.cap = it->first;
-      g.cached -= s.cap;
-      g.cache.erase(it);
-    } else {
-      void *p = nullptr;
-      hipError_t e = hipMalloc(&p, cap);
-      if (e != hipSuccess) {
-        // give cached blocks back to the driver and retry once
-        (void)hipGetLastError();
-        release_cache(0);
-        e = hipMalloc(&p, cap);
+    const size_t cap = round_up(bytes);
+    const auto fits = [cap](size_t have) { return have <= cap + cap / 4; };
+    s.arena = g.capturing;
+    if (g.capturing) {
+      // first choice: a block this graph already owns and no tensor holds any
+      // more (such blocks stay counted as in use until the graph is destroyed)
+      auto &mine = g.graphs[g.capturing - 1].free_blocks;
+      auto mt = mine.lower_bound(cap);
+      if (mt != mine.end() && fits(mt->first)) {
+        s.ptr = mt->second;
+        s.cap = mt->first;
+        mine.erase(mt);
       }
-      if (e != hipSuccess) {
-        (void)hipGetLastError();
-        fail(WDH_ENOMEM, "wdh_alloc: hipMalloc(%zu) failed: %s", cap,
-             hipGetErrorString(e));
-        return 0;
-      }
-      s.ptr = p;
-      s.cap = cap;
-      g.reserved += cap;
-      if (g.reserved > g.peak) g.peak = g.reserved;
     }
-    g.in_use += s.cap;
+    if (!s.ptr) {
+      auto it = g.cache.lower_bound(cap);
+      if (it != g.cache.end() && fits(it->first)) {
+        s.ptr = it->second;
+        s.cap = it->first;
+        g.cached -= s.cap;
+        g.cache.erase(it);
+      } else {
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, cap);
+        if (e != hipSuccess && !g.capturing) {
+          // give cached blocks back to the driver and retry once (this drains
+          // the stream, which a capture would not survive)
+          (void)hipGetLastError();
+          release_cache(0);
+          e = hipMalloc(&p, cap);
+        }
+        if (e != hipSuccess) {
+          (void)hipGetLastError();
+          fail(WDH_ENOMEM, "wdh_alloc: hipMalloc(%zu) failed: %s", cap,
+               hipGetErrorString(e));
+          return 0;
+        }
+        s.ptr = p;
+        s.cap = cap;
+        g.reserved += cap;
+        if (g.reserved > g.peak) g.peak = g.reserved;
+      }
+      g.in_use += s.cap;
+    }
   }
   int64_t idx;
   if (!g.free_slots.empty()) {
@@ -258,17 +317,98 @@ int wdh_free(wdh_buf h) {
                 (long long)h);
   Slot &s = g.slots[h - 1];
   if (s.cap) {
-    g.cache.emplace(s.cap, s.ptr);
-    g.cached += s.cap;
-    g.in_use -= s.cap;
+    if (s.arena && g.graphs[s.arena - 1].live) {
+      // memory of a captured graph: stays with it
+      g.graphs[s.arena - 1].free_blocks.emplace(s.cap, s.ptr);
+    } else {
+      g.cache.emplace(s.cap, s.ptr);
+      g.cached += s.cap;
+      g.in_use -= s.cap;
+    }
   }
   s = Slot();
   g.free_slots.push_back(h - 1);
   return WDH_OK;
 }
 
+// ---- captured runs ----------------------------------------------------------
+#define WDH_NOT_WHILE_CAPTURING(what)                                             \
+  do {                                                                            \
+    if (g.capturing) {                                                            \
+      g.capture_failed = true;                                                    \
+      return fail(WDH_ESTATE, what ": not possible while a graph is being captured"); \
+    }                                                                             \
+  } while (0)
+
+int wdh_graph_begin(void) {
+  WDH_REQUIRE_INIT();
+  if (g.capturing) return fail(WDH_ESTATE, "wdh_graph_begin: a capture is already open");
+  for (int i = 0; i < 2; i++)
+    if (g.stage_busy[i]) {
+      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[i]));
+      g.stage_busy[i] = false;
+    }
+  int id = -1;
+  for (size_t i = 0; i < g.graphs.size(); i++)
+    if (!g.graphs[i].live) id = (int)i;
+  if (id < 0) {
+    id = (int)g.graphs.size();
+    g.graphs.emplace_back();
+  }
+  // relaxed: hipMalloc stays legal while capturing (a pool miss)
+  WDH_HIP_CHECK(hipStreamBeginCapture(g.stream, hipStreamCaptureModeRelaxed));
+  g.graphs[id] = GraphRec();
+  g.graphs[id].live = true;
+  g.capturing = id + 1;
+  g.capture_failed = false;
+  return WDH_OK;
+}
+
+int wdh_graph_end(int *graph_id) {
+  WDH_REQUIRE_INIT();
+  if (!g.capturing) return fail(WDH_ESTATE, "wdh_graph_end: no capture is open");
+  const int id = g.capturing - 1;
+  g.capturing = 0;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(g.stream, &graph);
+  g.graphs[id].graph = graph;
+  if (e == hipSuccess && graph && !g.capture_failed)
+    e = hipGraphInstantiate(&g.graphs[id].exec, graph, nullptr, nullptr, 0);
+  if (e != hipSuccess || !graph || g.capture_failed || !graph_id) {
+    const bool poisoned = g.capture_failed;
+    (void)hipGetLastError();
+    dissolve_graph(id);
+    if (!graph_id) return fail(WDH_EINVAL, "wdh_graph_end: graph_id is NULL");
+    if (poisoned)
+      return fail(WDH_ESTATE, "wdh_graph_end: the capture was abandoned: a call made while capturing cannot be recorded");
+    return fail(WDH_EHIP, "wdh_graph_end: %s", e == hipSuccess ? "empty capture" : hipGetErrorString(e));
+  }
+  *graph_id = id;
+  return WDH_OK;
+}
+
+int wdh_graph_launch(int graph_id) {
+  WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_graph_launch");
+  if (graph_id < 0 || (size_t)graph_id >= g.graphs.size() || !g.graphs[graph_id].live ||
+      !g.graphs[graph_id].exec)
+    return fail(WDH_EINVAL, "wdh_graph_launch: unknown graph %d", graph_id);
+  WDH_HIP_CHECK(hipGraphLaunch(g.graphs[graph_id].exec, g.stream));
+  return WDH_OK;
+}
+
+int wdh_graph_destroy(int graph_id) {
+  WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_graph_destroy");
+  if (graph_id < 0 || (size_t)graph_id >= g.graphs.size() || !g.graphs[graph_id].live)
+    return fail(WDH_EINVAL, "wdh_graph_destroy: unknown graph %d", graph_id);
+  dissolve_graph(graph_id);
+  return WDH_OK;
+}
+
 int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_write");
   size_t have = 0;
   char *dst = (char *)wdh::resolve(h, &have);
   if (!dst) return WDH_EINVAL;
@@ -298,6 +438,7 @@ int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
 
 int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_read");
   size_t have = 0;
   const char *src = (const char *)wdh::resolve(h, &have);
   if (!src) return WDH_EINVAL;
@@ -363,6 +504,7 @@ int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
 
 int wdh_sync(void) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_sync");
   WDH_HIP_CHECK(hipStreamSynchronize(g.stream));
   return WDH_OK;
 }
@@ -377,12 +519,14 @@ int wdh_mem_stats(uint64_t *in_use, uint64_t *cached, uint64_t *peak) {
 
 int wdh_trim(size_t keep_bytes) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_trim");
   release_cache(keep_bytes);
   return WDH_OK;
 }
 
 int wdh_event_record(int id) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_event_record");
   if (id < 0 || id >= WDH_MAX_EVENTS)
     return fail(WDH_EINVAL, "wdh_event_record: id %d out of range", id);
   if (!g.events[id]) WDH_HIP_CHECK(hipEventCreate(&g.events[id]));
@@ -392,6 +536,7 @@ int wdh_event_record(int id) {
 
 int wdh_event_elapsed_ms(int start_id, int stop_id, float *ms) {
   WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_event_elapsed_ms");
   if (start_id < 0 || start_id >= WDH_MAX_EVENTS || stop_id < 0 ||
       stop_id >= WDH_MAX_EVENTS || !g.events[start_id] || !g.events[stop_id])
     return fail(WDH_EINVAL, "wdh_event_elapsed_ms: event not recorded");

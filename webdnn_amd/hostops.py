@@ -176,6 +176,21 @@ class HipContext:
         call("wdh_mem_stats", ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
         return {"in_use": a.value, "cached": b.value, "peak": c.value}
 
+    # captured runs (wdh_graph_*): record the device work between begin and end once, replay it
+    def graph_begin(self):
+        call("wdh_graph_begin")
+
+    def graph_end(self):
+        gid = ctypes.c_int(-1)
+        call("wdh_graph_end", ctypes.byref(gid))
+        return gid.value
+
+    def graph_launch(self, graph_id):
+        call("wdh_graph_launch", graph_id)
+
+    def graph_destroy(self, graph_id):
+        call("wdh_graph_destroy", graph_id)
+
     def event_record(self, idx):
         call("wdh_event_record", idx)
 

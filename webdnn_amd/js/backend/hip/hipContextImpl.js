@@ -51,7 +51,12 @@ class WebDNNHipContextImpl {
   // eslint-disable-next-line no-unused-vars
   async moveTensor(tensor, option) {
     const dst = new HipTensorImpl(this, tensor.dims, tensor.dataType);
-    await dst.setData(await tensor.getData());
+    try {
+      await dst.setData(await tensor.getData());
+    } catch (error) {
+      dst.dispose(); // e.g. an upload attempted while a graph is being captured
+      throw error;
+    }
     return dst;
   }
 

@@ -6,6 +6,7 @@
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
+//        [--graph] [--alt-inputs a2.bin[,b2.bin...]]
 //
 // Inputs are raw little-endian files (float32, or int32 where the graph input says
 // so) in the order of the graph's non-initializer inputs; outputs are written the same
@@ -14,6 +15,10 @@
 // times.  --cpu-entries registers extra cpu OperatorEntry objects exported by a module
 // (getOpEntries()); parity tests and the CPU baseline pass the CPU restatement of the
 // reference operators that way, the product itself ships hot-path operators for hip only.
+//
+// --graph passes {graph: true} to runner.run: the second call records the run into a HIP graph,
+// later calls replay it.  --alt-inputs names a second set of input files used by every other
+// run (odd run numbers), so that replays see changing data.
 //
 // Methodology follows the reference's harness (example/benchmark/runner/bench.js:130-167):
 // warm-up runs, then timed runner.run() calls.
@@ -33,6 +38,8 @@ function parseArgs(argv) {
     if (a === "--model") args.model = next();
     else if (a === "--onnx") args.onnx = next();
     else if (a === "--optimized") args.optimized = true;
+    else if (a === "--graph") args.graph = true;
+    else if (a === "--alt-inputs") args.altInputs = next().split(",");
     else if (a === "--backend") args.backend = next();
     else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
     else if (a === "--output") args.output = next();
@@ -72,19 +79,21 @@ async function main() {
   if (files.length !== graphInputs.length) {
     throw new Error(`model has ${graphInputs.length} inputs, ${files.length} files given`);
   }
-  const inputs = graphInputs.map((gi, idx) => {
+  const readInputs = (paths) => graphInputs.map((gi, idx) => {
     const tt = gi.type.tensorType;
     const dims = tt.shape.dim.map((d) => d.dimValue);
     const dataType = tt.elemType === 1 ? "float32" : "int32";
-    const buf = fs.readFileSync(files[idx]);
+    const buf = fs.readFileSync(paths[idx]);
     const Ctor = dataType === "float32" ? Float32Array : Int32Array;
     const copy = new Uint8Array(buf.byteLength);
     copy.set(buf);
     const data = new Ctor(copy.buffer, 0, copy.byteLength / 4);
     const expect = dims.reduce((a, b) => a * b, 1);
-    if (data.length !== expect) throw new Error(`${files[idx]}: ${data.length} elements, graph input needs ${expect}`);
+    if (data.length !== expect) throw new Error(`${paths[idx]}: ${data.length} elements, graph input needs ${expect}`);
     return new WebDNN.CPUTensor(dims, dataType, data);
   });
+  const inputs = readInputs(files);
+  const altInputs = args.altInputs ? readInputs(args.altInputs) : null;
 
   // --resident-inputs: upload the inputs once; the timed runs then start with their data in HBM
   let runInputs = inputs;
@@ -93,12 +102,13 @@ async function main() {
     for (const t of inputs) runInputs.push(await runner.backendContexts.hip.moveTensor(t, {}));
     runner.backendContexts.hip.sync();
   }
-  for (let i = 0; i < args.warmup; i++) await runner.run(runInputs);
+  for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, { graph: !!args.graph });
   const times = [];
   let outputs = null;
   for (let i = 0; i < args.runs; i++) {
     const t0 = process.hrtime.bigint();
-    outputs = await runner.run(runInputs, { measurePerformance: !!args.measure && i === args.runs - 1 });
+    outputs = await runner.run(altInputs && i % 2 === 1 ? altInputs : runInputs,
+      { measurePerformance: !!args.measure && i === args.runs - 1, graph: !!args.graph });
     times.push(Number(process.hrtime.bigint() - t0) / 1e6);
   }
   if (args.output) {
@@ -116,7 +126,9 @@ async function main() {
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
     node: process.version,
+    graph: args.graph ? { captured: !!runner.graphState, unsupported: runner.graphUnsupported } : undefined,
   };
+  runner.disposeGraph();
   if (args.measure && runner.lastPerformance) {
     report.performance = runner.lastPerformance.map((p) => ({
       name: p.name, opType: p.opType, backend: p.backend, outputDims: p.outputDims,

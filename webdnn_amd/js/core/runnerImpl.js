@@ -11,7 +11,10 @@
 //     silently pass on the fallback;
 //   * lastRunStats: how many nodes ran on which backend, and which were retried;
 //   * measurePerformance uses HIP events on the library's stream for hip nodes
-//     (Date.now() only sees enqueue time there).
+//     (Date.now() only sees enqueue time there);
+//   * run(inputs, {graph: true}) records the device work of one run into a HIP graph
+//     and replays it on later calls with inputs of the same shapes: the node loop
+//     below (runnerImpl.ts:377-542 in the reference) then runs once, not per call.
 const fs = require("fs");
 const path = require("path");
 const { backends, backendsWithoutCPU } = require("../interface/constants");
@@ -37,9 +40,16 @@ class RunnerImpl {
     this.forceOperatorBackendOrder = {};
     this.lastRunStats = null;
     this.lastPerformance = null;
+    // captured run: {id, inputs, ownedInputs, outputs, signature, stats}; see runWithGraph
+    this.graphState = null;
+    this.graphWarm = false;
+    this.graphUnsupported = null; // reason, once a capture has failed for this model
   }
 
   async loadModel(directory, onnxBasename) {
+    this.disposeGraph();
+    this.graphWarm = false;
+    this.graphUnsupported = null;
     const bytes = fs.readFileSync(path.join(directory, onnxBasename));
     this.loadModelFromBytes(bytes, directory);
   }
@@ -119,6 +129,108 @@ class RunnerImpl {
     const opts = options || {};
     if (!this.model || !this.loaded) throw new Error("not initialized");
     if (!inputs) throw new Error("inputs are required");
+    const hipContext = this.backendContexts.hip;
+    if (opts.graph && hipContext && hipContext.initialized && hipContext.native.graphBegin && !this.graphUnsupported) {
+      return this.runWithGraph(inputs, opts);
+    }
+    return this.runEager(inputs, opts);
+  }
+
+  // Frees the captured run, if any (its output and input buffers included).
+  disposeGraph() {
+    const state = this.graphState;
+    if (!state) return;
+    this.graphState = null;
+    const hip = this.backendContexts.hip;
+    for (const t of state.outputs) if (t.backend === "hip") t.dispose();
+    for (const t of state.ownedInputs) t.dispose();
+    hip.native.graphDestroy(state.id);
+  }
+
+  // First call: an ordinary run (it uploads the weights, fills the buffer pool and builds
+  // the conv tap tables, none of which can happen while capturing).  Second call: the node
+  // loop runs once more with the stream in capture mode -- operators record their kernels
+  // instead of executing them -- and the resulting graph is launched.  Later calls with
+  // inputs of the same shapes and types refill the captured input buffers, launch the graph
+  // and read the captured output buffers.  A model whose run needs the host to look at
+  // device data (a shape computed on the device, a node that fails over to the cpu) cannot
+  // be captured: the capture is dropped, the reason kept in graphUnsupported, and this and
+  // all later calls run eagerly.
+  async runWithGraph(inputs, opts) {
+    const hip = this.backendContexts.hip,
+      cpu = this.backendContexts.cpu;
+    if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
+    const signature = inputs.map((t) => `${t.dataType}[${t.dims.join(",")}]`).join(";");
+    if (this.graphState && this.graphState.signature !== signature) this.disposeGraph();
+    if (!this.graphState) {
+      if (!this.graphWarm) {
+        this.graphWarm = true;
+        return this.runEager(inputs, opts);
+      }
+      const graphInputs = [],
+        ownedInputs = [];
+      for (const t of inputs) {
+        if (t.backend === "hip") {
+          graphInputs.push(t);
+        } else {
+          const moved = await hip.moveTensor(t, {});
+          graphInputs.push(moved);
+          ownedInputs.push(moved);
+        }
+      }
+      let outputs = null,
+        failure = null;
+      hip.native.graphBegin();
+      try {
+        outputs = await this.runEager(graphInputs, { capture: true });
+      } catch (error) {
+        failure = error;
+      }
+      let id = -1;
+      try {
+        id = hip.native.graphEnd();
+      } catch (error) {
+        failure = failure || error;
+      }
+      if (failure) {
+        if (id >= 0) hip.native.graphDestroy(id);
+        for (const t of outputs || []) if (t.backend === "hip") t.dispose();
+        for (const t of ownedInputs) t.dispose();
+        this.graphUnsupported = failure.message;
+        logger.warn(`run could not be captured into a graph (${failure.message}); running eagerly`);
+        return this.runEager(inputs, opts);
+      }
+      this.graphState = { id, inputs: graphInputs, ownedInputs, outputs, signature, stats: this.lastRunStats };
+    } else {
+      const state = this.graphState;
+      for (let i = 0; i < inputs.length; i++) {
+        const src = inputs[i],
+          dst = state.inputs[i];
+        if (src === dst) continue;
+        if (src.backend === "hip") hip.native.copy(dst.handle, 0, src.handle, 0, dst.length * 4);
+        else await dst.setData(await src.getData());
+      }
+    }
+    const state = this.graphState;
+    if (opts.measurePerformance) hip.native.eventRecord(0);
+    hip.native.graphLaunch(state.id);
+    if (opts.measurePerformance) hip.native.eventRecord(1);
+    const results = [];
+    for (const t of state.outputs) {
+      // device -> host, the run's only synchronisation; a cpu output (a constant) is copied
+      results.push(await cpu.moveTensor(t, {}));
+    }
+    if (opts.measurePerformance) {
+      this.lastPerformance = [{ opType: "(captured graph)", name: "graph", backend: "hip", deviceElapsed: hip.native.eventElapsedMs(0, 1) }];
+    }
+    this.lastRunStats = Object.assign({}, state.stats, { graphReplay: true });
+    return results;
+  }
+
+  // opts.capture (internal): the stream is recording; keep the outputs where they are and
+  // never retry on the cpu.
+  async runEager(inputs, options) {
+    const opts = options || {};
     const graph = this.model.graph;
     const tensorsForBackends = {};
     for (const backend of backends) tensorsForBackends[backend] = new Map();
@@ -143,9 +255,9 @@ class RunnerImpl {
     const tensorReleaseTiming = findTensorReleaseTiming(this.model, new Set(this.initializerTensors.keys()));
     const nodePerformances = [];
     const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length };
-    const strict = !!this.options.strict;
+    const strict = !!this.options.strict || !!opts.capture;
     const hip = this.backendContexts.hip;
-    const useEvents = !!opts.measurePerformance && hip && hip.initialized && graph.node.length * 2 <= 4096;
+    const useEvents = !opts.capture && !!opts.measurePerformance && hip && hip.initialized && graph.node.length * 2 <= 4096;
 
     try {
       for (let i = 0; i < graph.node.length; i++) {
@@ -261,6 +373,17 @@ class RunnerImpl {
       const outputs = [];
       for (const outputInfo of graph.output) {
         let outputTensor = tensorsForBackends.cpu.get(outputInfo.name);
+        if (!outputTensor && opts.capture) {
+          // recorded, not computed yet: the tensor stays on the device for the replays
+          for (const otherBackend of this.backendOrder) {
+            const otherT = tensorsForBackends[otherBackend].get(outputInfo.name);
+            if (otherT) {
+              outputTensor = otherT;
+              callerOwned.add(otherT);
+              break;
+            }
+          }
+        }
         if (!outputTensor) {
           for (const otherBackend of this.backendOrder) {
             const otherT = tensorsForBackends[otherBackend].get(outputInfo.name);

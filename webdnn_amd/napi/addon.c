@@ -384,6 +384,35 @@ FN(js_strided_copy) { /* (X, xOffset, Y, yOffset, shape[], xStrides[], yStrides[
   return make_undefined(env);
 }
 
+FN(js_graph_begin) {
+  ARGS("wdh_graph_begin", 0);
+  CHECK(wdh_graph_begin());
+  return make_undefined(env);
+}
+
+FN(js_graph_end) { /* -> graph id */
+  ARGS("wdh_graph_end", 0);
+  int id = -1;
+  CHECK(wdh_graph_end(&id));
+  napi_value out;
+  if (napi_create_int32(env, id, &out) != napi_ok) return NULL;
+  return out;
+}
+
+FN(js_graph_launch) {
+  ARGS("wdh_graph_launch", 1);
+  I64(0, id);
+  CHECK(wdh_graph_launch((int)id));
+  return make_undefined(env);
+}
+
+FN(js_graph_destroy) {
+  ARGS("wdh_graph_destroy", 1);
+  I64(0, id);
+  CHECK(wdh_graph_destroy((int)id));
+  return make_undefined(env);
+}
+
 static napi_value init_module(napi_env env, napi_value exports) {
   static const struct {
     const char *name;
@@ -397,7 +426,8 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"softmax", js_softmax}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
-      {"stridedCopy", js_strided_copy},
+      {"stridedCopy", js_strided_copy}, {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end},
+      {"graphLaunch", js_graph_launch}, {"graphDestroy", js_graph_destroy},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {
     napi_value fn;
