@@ -8,7 +8,10 @@ Workload of `value` (BASELINE config 4): ResNet-50 v1, batch 32, fp32, random-in
 (seeded), BatchNorm folded, run through the Node.js descriptor runner on the `hip` backend
 (WebDNN.load + runner.run) in strict mode — no CPU fallback.  A step is one runner.run() over one
 batch whose input tensor is already resident in HBM; the step ends when the logits are back on the
-host (the run's only synchronisation).  `value` = 32 * steps / total time.
+host (the run's only synchronisation).  Steps call runner.run(x, {graph: true}): the first warm-up
+run is eager, the second records the run's kernels into a HIP graph, every timed step launches that
+graph (same kernels, same order, one launch) and reads the logits; `extra.resnet50_ms_per_step_eager`
+is the same step through the node-by-node loop.  `value` = 32 * steps / total time.
 
 `roofline` is for the dominant kernel of that workload, the implicit-GEMM contraction kernel: its
 algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over its device time,
@@ -60,9 +63,12 @@ def bench_resnet(steps, warmup, workdir):
     x = np.random.default_rng(6).standard_normal((batch, 3, 224, 224)).astype(np.float32)
     inp = os.path.join(workdir, "input.bin")
     x.tofile(inp)
-    timed = node_run(workdir, inp, "hip", steps, warmup, ["--strict", "--resident-inputs"])
+    # graph mode: warm-up run 1 is eager, run 2 records the HIP graph, every timed step replays it
+    timed = node_run(workdir, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--graph"])
     assert timed["backend"] == "hip" and list(timed["stats"]["nodesByBackend"]) == ["hip"], timed["stats"]
+    assert timed["graph"]["captured"], timed["graph"]
     total_ms = sum(timed["msPerRun"])
+    eager = node_run(workdir, inp, "hip", max(3, steps // 2), max(warmup, 2), ["--strict", "--resident-inputs"])
     # one more run with per-node HIP events for the kernel-level figure
     prof = node_run(workdir, inp, "hip", 1, 2, ["--strict", "--resident-inputs", "--measure"])
     contraction_ms = sum(p["deviceElapsed"] for p in prof["performance"]
@@ -76,6 +82,7 @@ def bench_resnet(steps, warmup, workdir):
         "images_per_s": batch * steps / total_ms * 1e3, "contraction_ms": contraction_ms,
         "contraction_launches": launches, "device_ms": all_ms,
         "images_per_s_host_input": batch / (sum(host_in["msPerRun"]) / len(host_in["msPerRun"])) * 1e3,
+        "ms_per_step_eager": sum(eager["msPerRun"]) / len(eager["msPerRun"]),
         "device": timed.get("device"), "node_version": timed["node"],
     }
 
@@ -97,10 +104,13 @@ def bench_report_only(workdir, steps, warmup):
             f.write(data)
         inp = os.path.join(d, "input.bin")
         np.random.default_rng(11).standard_normal(shape).astype(np.float32).tofile(inp)
-        rep = node_run(d, inp, "hip", steps, warmup, ["--strict", "--resident-inputs"])
+        rep = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--graph"])
         assert list(rep["stats"]["nodesByBackend"]) == ["hip"], rep["stats"]
         ms = sum(rep["msPerRun"]) / len(rep["msPerRun"])
+        eager = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs"])
         out[key] = {"workload": label, "nodes": rep["nodes"], "ms_per_run": round(ms, 4),
+                    "graph_replay": bool(rep["graph"]["captured"]),
+                    "ms_per_run_eager": round(sum(eager["msPerRun"]) / len(eager["msPerRun"]), 4),
                     "gflops": round(g.flops / ms / 1e6, 1),
                     "frac_mfma_peak": round(g.flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
     return out
@@ -272,7 +282,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "ResNet-50 v1 batch 32 [32,3,224,224] fp32, random init (seeded), BN folded, "
-                               "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict "
+                               "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict, "
+                               "runner.run(x, {graph: true}) replaying the step's captured HIP graph "
                                "(BASELINE config 4)" % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
@@ -293,6 +304,7 @@ def main():
             "ffn_c2": report_only["ffn_c2"],
             "detr_r50_b1": report_only["detr_r50_b1"],
             "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
+            "resnet50_ms_per_step_eager": round(resnet["ms_per_step_eager"], 4),
             "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),
             "device": resnet["device"],
         },
