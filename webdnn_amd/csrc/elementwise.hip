@@ -82,7 +82,9 @@ __global__ __launch_bounds__(256) void binary_dense_f32(const float *__restrict_
 // Broadcast path with a vectorisable innermost axis: each thread produces 4
 // consecutive outputs of the innermost axis; an operand whose innermost stride
 // is 1 is read with one 16-byte load, one whose stride is 0 with one scalar load.
-template <int OP>
+// IDX is the type the output index is decomposed in: unsigned when the tensor
+// has fewer than 2^32 elements (32-bit divisions), long long otherwise.
+template <int OP, typename IDX>
 __global__ __launch_bounds__(256) void binary_bcast_vec_f32(BinaryParams p) {
   const long long nvec = p.total >> 2;
   const long long stride = (long long)gridDim.x * blockDim.x;
@@ -90,12 +92,13 @@ __global__ __launch_bounds__(256) void binary_bcast_vec_f32(BinaryParams p) {
   float *Y = (float *)p.Y;
   for (long long v = (long long)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
        v += stride) {
-    long long rem = v << 2, ol = 0, orr = 0;
+    IDX rem = (IDX)(v << 2);
+    long long ol = 0, orr = 0;
 #pragma unroll
     for (int d = MAXD - 1; d >= 0; d--) {
       if (d < p.ndim) {
-        long long q = rem / p.shape[d];
-        long long c = rem - q * p.shape[d];
+        const IDX q = rem / (IDX)p.shape[d];
+        const long long c = (long long)(rem - q * (IDX)p.shape[d]);
         rem = q;
         ol += c * p.sl[d];
         orr += c * p.sr[d];
@@ -115,19 +118,20 @@ __global__ __launch_bounds__(256) void binary_bcast_vec_f32(BinaryParams p) {
 }
 
 // General path: one output element per thread per step, any strides.
-template <int OP, typename T>
+template <int OP, typename T, typename IDX>
 __global__ __launch_bounds__(256) void binary_general(BinaryParams p) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   const T *L = (const T *)p.L, *R = (const T *)p.R;
   T *Y = (T *)p.Y;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
        i < p.total; i += stride) {
-    long long rem = i, ol = 0, orr = 0;
+    IDX rem = (IDX)i;
+    long long ol = 0, orr = 0;
 #pragma unroll
     for (int d = MAXD - 1; d >= 0; d--) {
       if (d < p.ndim) {
-        long long q = rem / p.shape[d];
-        long long c = rem - q * p.shape[d];
+        const IDX q = rem / (IDX)p.shape[d];
+        const long long c = (long long)(rem - q * (IDX)p.shape[d]);
         rem = q;
         ol += c * p.sl[d];
         orr += c * p.sr[d];
@@ -151,19 +155,29 @@ unsigned grid_for(long long work_items, int per_block) {
 template <int OP>
 int launch_binary(const BinaryParams &p, int dtype, bool dense, bool vec) {
   hipStream_t st = wdh::stream();
+  const bool small = p.total <= 0xffffffffLL;
   if (dtype == 0 && dense) {
     hipLaunchKernelGGL(binary_dense_f32<OP>, dim3(grid_for((p.total + 3) / 4, 256)),
                        dim3(256), 0, st, (const float *)p.L, (const float *)p.R,
                        (float *)p.Y, p.total);
   } else if (dtype == 0 && vec) {
-    hipLaunchKernelGGL(binary_bcast_vec_f32<OP>, dim3(grid_for(p.total / 4, 256)),
-                       dim3(256), 0, st, p);
+    const dim3 grid(grid_for(p.total / 4, 256));
+    if (small)
+      hipLaunchKernelGGL((binary_bcast_vec_f32<OP, unsigned>), grid, dim3(256), 0, st, p);
+    else
+      hipLaunchKernelGGL((binary_bcast_vec_f32<OP, long long>), grid, dim3(256), 0, st, p);
   } else if (dtype == 0) {
-    hipLaunchKernelGGL((binary_general<OP, float>), dim3(grid_for(p.total, 256)),
-                       dim3(256), 0, st, p);
+    const dim3 grid(grid_for(p.total, 256));
+    if (small)
+      hipLaunchKernelGGL((binary_general<OP, float, unsigned>), grid, dim3(256), 0, st, p);
+    else
+      hipLaunchKernelGGL((binary_general<OP, float, long long>), grid, dim3(256), 0, st, p);
   } else {
-    hipLaunchKernelGGL((binary_general<OP, int>), dim3(grid_for(p.total, 256)),
-                       dim3(256), 0, st, p);
+    const dim3 grid(grid_for(p.total, 256));
+    if (small)
+      hipLaunchKernelGGL((binary_general<OP, int, unsigned>), grid, dim3(256), 0, st, p);
+    else
+      hipLaunchKernelGGL((binary_general<OP, int, long long>), grid, dim3(256), 0, st, p);
   }
   WDH_LAUNCH_CHECK();
   return WDH_OK;

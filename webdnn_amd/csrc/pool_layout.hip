@@ -24,15 +24,17 @@ struct PoolParams {
   int h, w, oh, ow, kh, kw, pt, pl, sh, sw, dh, dw;
 };
 
+// IDX: the type the output index is decomposed in (unsigned below 2^32 cells).
+template <typename IDX>
 __global__ __launch_bounds__(256) void maxpool2d_kernel(PoolParams p) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
        i += stride) {
-    const int ox = (int)(i % p.ow);
-    const long long t = i / p.ow;
-    const int oy = (int)(t % p.oh);
-    const long long plane = t / p.oh;  // n*c + c
-    const float *x = p.X + plane * p.h * p.w;
+    const IDX t = (IDX)i / (IDX)p.ow;
+    const int ox = (int)((IDX)i - t * (IDX)p.ow);
+    const IDX plane = t / (IDX)p.oh;  // n*c + c
+    const int oy = (int)(t - plane * (IDX)p.oh);
+    const float *x = p.X + (long long)plane * p.h * p.w;
     float mv = -INFINITY;
     for (int ky = 0; ky < p.kh; ky++) {
       const int iy = oy * p.sh - p.pt + ky * p.dh;
@@ -60,16 +62,19 @@ struct GatherCopyParams {
 
 // Generic: thread per output element.  Coalesced on the output side always,
 // on the input side when the last output axis has input stride 1.
+// IDX: the type the output index is decomposed in (unsigned below 2^32 elements).
+template <typename IDX>
 __global__ __launch_bounds__(256) void gather_copy_kernel(GatherCopyParams p) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
        i += stride) {
-    long long rem = i, off = 0;
+    IDX rem = (IDX)i;
+    long long off = 0;
 #pragma unroll
     for (int d = MAXD - 1; d >= 0; d--) {
       if (d < p.ndim) {
-        long long q = rem / p.shape[d];
-        off += (rem - q * p.shape[d]) * p.sin[d];
+        const IDX q = rem / (IDX)p.shape[d];
+        off += (long long)(rem - q * (IDX)p.shape[d]) * p.sin[d];
         rem = q;
       }
     }
@@ -90,16 +95,18 @@ struct StridedCopyParams {
 
 // Thread per element, innermost axis fastest: coalesced wherever the innermost
 // stride is 1 (always on the dense side of a Slice/Concat/Split).
+template <typename IDX>
 __global__ __launch_bounds__(256) void strided_copy_kernel(StridedCopyParams p) {
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
        i += stride) {
-    long long rem = i, ox = 0, oy = 0;
+    IDX rem = (IDX)i;
+    long long ox = 0, oy = 0;
 #pragma unroll
     for (int d = MAXD - 1; d >= 0; d--) {
       if (d < p.ndim) {
-        const long long q = rem / p.shape[d];
-        const long long r = rem - q * p.shape[d];
+        const IDX q = rem / (IDX)p.shape[d];
+        const long long r = (long long)(rem - q * (IDX)p.shape[d]);
         ox += r * p.sx[d];
         oy += r * p.sy[d];
         rem = q;
@@ -204,8 +211,12 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
   p.X = (const float *)px; p.Y = (float *)py;
   p.h = h; p.w = w; p.oh = oh; p.ow = ow; p.kh = kh; p.kw = kw;
   p.pt = pt; p.pl = pl; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
-  hipLaunchKernelGGL(maxpool2d_kernel, dim3(grid_for(p.total)), dim3(256), 0,
-                     wdh::stream(), p);
+  if (p.total <= 0xffffffffLL)
+    hipLaunchKernelGGL(maxpool2d_kernel<unsigned>, dim3(grid_for(p.total)), dim3(256), 0,
+                       wdh::stream(), p);
+  else
+    hipLaunchKernelGGL(maxpool2d_kernel<long long>, dim3(grid_for(p.total)), dim3(256), 0,
+                       wdh::stream(), p);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }
@@ -282,7 +293,10 @@ extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
   g.X = (const uint32_t *)px; g.Y = (uint32_t *)py;
   g.total = total; g.ndim = nd;
   for (int d = 0; d < nd; d++) { g.shape[d] = shape[d]; g.sin[d] = sin[d]; }
-  hipLaunchKernelGGL(gather_copy_kernel, dim3(grid_for(total)), dim3(256), 0, st, g);
+  if (total <= 0xffffffffLL)
+    hipLaunchKernelGGL(gather_copy_kernel<unsigned>, dim3(grid_for(total)), dim3(256), 0, st, g);
+  else
+    hipLaunchKernelGGL(gather_copy_kernel<long long>, dim3(grid_for(total)), dim3(256), 0, st, g);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }
@@ -358,7 +372,10 @@ extern "C" int wdh_strided_copy(wdh_buf hX, int64_t x_offset, wdh_buf hY, int64_
                                  wdh::stream()));
     return WDH_OK;
   }
-  hipLaunchKernelGGL(strided_copy_kernel, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
+  if (total <= 0xffffffffLL)
+    hipLaunchKernelGGL(strided_copy_kernel<unsigned>, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
+  else
+    hipLaunchKernelGGL(strided_copy_kernel<long long>, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }
