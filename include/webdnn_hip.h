@@ -66,7 +66,7 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
 /* Backend options (the counterpart of InitOption.backendOptions,
  * src/descriptor_runner/index.ts:26-30).  Known names:
  *   "contraction_tile"  -1 = choose per problem (default); 0 = 128x128,
- *                       1 = 64x256, 2 = 64x128, 3 = 64x64 workgroup tiles for
+ *                       1 = 64x256, 2 = 64x128, 3 = 64x64, 4 = 128x64 workgroup tiles for
  *                       wdh_gemm / wdh_conv2d (a tuning and test hook: every
  *                       tile shape computes the same result).
  *   "split_k"           -1 = choose per problem (default); n >= 1 = cut the

@@ -675,7 +675,7 @@ def test_errors_are_reported_not_fatal(ctx):
 
 
 # ------------------------------------------------------------------ tile shapes
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 def test_every_tile_shape_computes_the_same(ctx, tile):
     """wdh_gemm / wdh_conv2d pick a workgroup tile per problem; every shape must agree."""
     A, B, C = uni(150, 70), uni(70, 300), uni(300)

@@ -769,9 +769,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int bm, in
 }
 
 // ---- host-side dispatch -------------------------------------------------------
-enum TileId { T128x128 = 0, T64x256 = 1, T64x128 = 2, T64x64 = 3 };
-const int kTileM[] = {128, 64, 64, 64};
-const int kTileN[] = {128, 256, 128, 64};
+enum TileId { T128x128 = 0, T64x256 = 1, T64x128 = 2, T64x64 = 3, T128x64 = 4 };
+const int kTileM[] = {128, 64, 64, 64, 128};
+const int kTileN[] = {128, 256, 128, 64, 64};
 
 // Tile choice by a small cost model: every CU works through ceil(tiles/CUs)
 // tiles, each costing its full area (rows or columns beyond the result are
@@ -925,16 +925,19 @@ int launch_tile(Params &p, int nz, bool vec) {
 
 template <bool A_KC, int BMODE>
 int launch(Params &p, int nz, bool vec) {
-  // Convs measured best on 64x64 tiles at every ResNet-50 layer shape (more
-  // wavefronts in flight to cover the gather's latency); Gemm/MatMul use the
-  // cost model.
+  // Convs measured best on 64x64 tiles at nearly every ResNet-50 layer shape;
+  // Gemm/MatMul use the cost model.
   const bool conv = BMODE >= B_IM2COL32;
+  // deep convs with many output channels (ResNet stage 3/4 3x3) gain ~5 % from two
+  // accumulator tiles per wavefront
+  const TileId conv_tile = (p.m >= 256 && p.k >= 2048) ? T128x64 : T64x64;
   TileId t = g_forced_tile >= 0 ? (TileId)g_forced_tile
-                                : (conv ? T64x64 : pick_tile(p.m, p.n, nz));
+                                : (conv ? conv_tile : pick_tile(p.m, p.n, nz));
   switch (t) {
     case T128x128: return launch_tile<128, 128, 2, 2, A_KC, BMODE>(p, nz, vec);
     case T64x256: return launch_tile<64, 256, 1, 4, A_KC, BMODE>(p, nz, vec);
     case T64x128: return launch_tile<64, 128, 1, 4, A_KC, BMODE>(p, nz, vec);
+    case T128x64: return launch_tile<128, 64, 2, 2, A_KC, BMODE>(p, nz, vec);
     default: return launch_tile<64, 64, 2, 2, A_KC, BMODE>(p, nz, vec);
   }
 }
@@ -954,9 +957,9 @@ using wdh::fail;
 extern "C" int wdh_set_option(const char *name, int value) {
   if (!name) return fail(WDH_EINVAL, "wdh_set_option: name is NULL");
   if (strcmp(name, "contraction_tile") == 0) {
-    if (value < -1 || value > T64x64)
+    if (value < -1 || value > T128x64)
       return fail(WDH_EINVAL, "wdh_set_option: contraction_tile %d outside -1..%d", value,
-                  (int)T64x64);
+                  (int)T128x64);
     g_forced_tile = value;
     return WDH_OK;
   }
