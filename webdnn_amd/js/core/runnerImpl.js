@@ -257,7 +257,7 @@ class RunnerImpl {
     const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length };
     const strict = !!this.options.strict || !!opts.capture;
     const hip = this.backendContexts.hip;
-    const useEvents = !opts.capture && !!opts.measurePerformance && hip && hip.initialized && graph.node.length * 2 <= 4096;
+    const useEvents = !opts.capture && !!opts.measurePerformance && hip && hip.initialized && graph.node.length + 1 <= 4096;
 
     try {
       for (let i = 0; i < graph.node.length; i++) {
@@ -328,9 +328,10 @@ class RunnerImpl {
 
             const context = this.contextFor(operator.backend);
             logger.debug(`Running ${node.name}(${opType}) on ${operator.backend}`);
-            if (useEvents) hip.native.eventRecord(2 * i);
+            // one event per node boundary: node i's device time runs from event i to event i+1
+            // (every event costs the stream a small bubble, so as few as possible)
+            if (useEvents) hip.native.eventRecord(i);
             const operatorOutputs = await operator.run(context, operatorInputs, node.output.length);
-            if (useEvents) hip.native.eventRecord(2 * i + 1);
             actualInputDims = operatorInputs.map((t) => t.dims);
             actualOutputDims = operatorOutputs.map((t) => t.dims);
             for (let j = 0; j < node.output.length; j++) {
@@ -401,9 +402,10 @@ class RunnerImpl {
 
       if (opts.measurePerformance) {
         if (useEvents) {
+          hip.native.eventRecord(nodePerformances.length);
           for (let i = 0; i < nodePerformances.length; i++) {
             if (nodePerformances[i].backend === "hip") {
-              nodePerformances[i].deviceElapsed = hip.native.eventElapsedMs(2 * i, 2 * i + 1);
+              nodePerformances[i].deviceElapsed = hip.native.eventElapsedMs(i, i + 1);
             }
           }
         }
