@@ -252,6 +252,7 @@ class RunnerImpl {
       callerOwned.add(inputs[i]);
     }
 
+    const runStart = process.hrtime.bigint();
     const tensorReleaseTiming = findTensorReleaseTiming(this.model, new Set(this.initializerTensors.keys()));
     const nodePerformances = [];
     const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length };
@@ -371,6 +372,8 @@ class RunnerImpl {
         });
       }
 
+      // host time of the node loop: everything is enqueued, nothing has been waited for yet
+      stats.enqueueMs = Number(process.hrtime.bigint() - runStart) / 1e6;
       const outputs = [];
       for (const outputInfo of graph.output) {
         let outputTensor = tensorsForBackends.cpu.get(outputInfo.name);
