@@ -227,7 +227,9 @@ def test_conv_1x1_equals_gemm(ctx):
 @pytest.mark.parametrize("sl,sr", [((2, 3, 10, 12), ()), ((2, 3, 10, 12), (1, 3, 1, 12)), ((), ()),
                                    ((2, 3, 10, 12), (2, 3, 10, 12)), ((4, 1), (3,)), ((8, 512, 3072), (3072,)),
                                    ((2, 1, 3, 1, 2, 1), (1, 2, 1, 2, 1, 3)), ((5, 7), (5, 1)), ((1, 3, 1, 12), (2, 3, 10, 12)),
-                                   ((3, 1031), (3, 1031)), ((2, 64, 7, 7), (1, 64, 1, 1)), ((850, 1, 256), (850, 1, 1))])
+                                   ((3, 1031), (3, 1031)), ((2, 64, 7, 7), (1, 64, 1, 1)), ((850, 1, 256), (850, 1, 1)),
+                                   ((3, 5000), (3, 1)), ((2, 5, 4101), (5, 1)), ((4, 16, 28, 28), (16, 1, 1)),
+                                   ((16, 1, 1), (4, 16, 28, 28)), ((7, 300), (300,)), ((4100,), (1,))])
 def test_binary_bit_exact(ctx, op, sl, sr):
     L, R = uni(*sl, lo=-3, hi=3), uni(*sr, lo=-3, hi=3)
     got = H.binary(ctx, op, ctx.move_tensor(L), ctx.move_tensor(R))
@@ -276,7 +278,7 @@ def test_unary(ctx):
 
 # ------------------------------------------------------------------ row reductions
 @pytest.mark.parametrize("shape", [(8, 850, 850), (8, 100, 850), (8, 100, 100), (3, 4, 5, 6), (7, 1), (5, 64), (3, 129),
-                                   (4, 1025), (2, 2049), (3, 5000), (1, 1)])
+                                   (4, 1025), (2, 2049), (3, 5000), (1, 1), (5, 256), (3, 1024), (2, 2048), (4, 852), (9, 132)])
 def test_softmax(ctx, shape):
     x = nrm(*shape, std=3.0)
     got = H.softmax(ctx, ctx.move_tensor(x)).get_data()
@@ -291,7 +293,8 @@ def test_softmax_edges(ctx):
         H.softmax(ctx, ctx.move_tensor(nrm(2, 3, 4)), axis=1)
 
 
-@pytest.mark.parametrize("shape", [(850, 1, 256), (100, 1, 256), (6, 2048), (3, 5000), (4, 7), (2, 3, 1)])
+@pytest.mark.parametrize("shape", [(850, 1, 256), (100, 1, 256), (6, 2048), (3, 5000), (4, 7), (2, 3, 1), (9, 1000),
+                                   (5, 250), (7, 1024), (3, 132)])
 def test_layernorm(ctx, shape):
     x, g, b = nrm(*shape, std=2.0), nrm(shape[-1]), nrm(shape[-1])
     got = H.layer_normalization(ctx, ctx.move_tensor(x), ctx.move_tensor(g), ctx.move_tensor(b)).get_data()
@@ -300,7 +303,8 @@ def test_layernorm(ctx, shape):
     assert_close_max(plain, ref.layernorm_decomposed(x, None, None, 1e-5), 1e-5, "layernorm no affine")
 
 
-@pytest.mark.parametrize("shape", [(32, 2048, 7, 7), (4, 16, 56, 56), (1, 3, 1, 1), (2, 5, 3, 300)])
+@pytest.mark.parametrize("shape", [(32, 2048, 7, 7), (4, 16, 56, 56), (1, 3, 1, 1), (2, 5, 3, 300), (3, 1400, 5, 5),
+                                   (70, 64, 8, 8), (5, 1000, 1, 2)])
 def test_global_average_pool_and_reduce_mean(ctx, shape):
     x = nrm(*shape)
     got = H.global_average_pool(ctx, ctx.move_tensor(x))
@@ -330,6 +334,9 @@ def test_maxpool_resnet_stem_full(ctx):
     dict(kernel_shape=[2, 2], strides=[2, 2], dilations=[2, 2], pads=[1, 1, 1, 1]),
     dict(kernel_shape=[2, 2], strides=[3, 3], pads=[1, 1, 1, 1], ceil_mode=1),
     dict(kernel_shape=[1, 1]),
+    dict(kernel_shape=[5, 5], strides=[2, 2], pads=[2, 2, 2, 2]),
+    dict(kernel_shape=[3, 2], strides=[1, 2], pads=[1, 0, 1, 1]),
+    dict(kernel_shape=[3, 3], strides=[4, 4], pads=[1, 1, 1, 1]),
 ])
 def test_maxpool_attributes(ctx, attrs):
     x = nrm(2, 3, 10, 13)
@@ -367,7 +374,8 @@ def test_transpose_all_permutations(ctx, ndim):
 @pytest.mark.parametrize("shape,perm", [((1, 256, 850), (2, 0, 1)), ((850, 8, 32), (1, 0, 2)), ((8, 850, 32), (0, 2, 1)),
                                          ((8, 850, 32), (1, 0, 2)), ((2, 3, 2, 2, 3), (4, 0, 3, 1, 2)),
                                          ((2, 3, 2, 2, 3, 2), (5, 3, 0, 4, 1, 2)), ((64, 64, 3, 3), (2, 3, 1, 0)),
-                                         ((1000, 2048), (1, 0)), ((3, 1, 5), (2, 1, 0))])
+                                         ((1000, 2048), (1, 0)), ((3, 1, 5), (2, 1, 0)), ((4, 300, 16), (0, 2, 1)),
+                                         ((2, 40, 3000), (1, 0, 2)), ((5, 6, 7, 4100), (2, 0, 1, 3))])
 def test_transpose_model_shapes(ctx, shape, perm):
     x = nrm(*shape)
     got = H.transpose(ctx, ctx.move_tensor(x), list(perm)).get_data()
@@ -492,6 +500,12 @@ def test_slice_ranks_ints_and_errors(ctx):
     big = nrm(32, 256, 56, 56)                                     # crop of a feature map, 100 MB in
     args = dict(starts=[4, 3], ends=[52, 53], axes=[2, 3])
     assert_bit_exact(H.slice_(ctx, ctx.move_tensor(big), **args).get_data(), ref.slice_(big, **args))
+    wide = nrm(6, 8, 4400)                                         # long rows: 16-byte pieces where alignment allows
+    tw = ctx.move_tensor(wide)
+    for args in (dict(starts=[7], ends=[-100], axes=[1], steps=[-1]), dict(starts=[4], ends=[4300], axes=[2]),
+                 dict(starts=[1], ends=[4399], axes=[2]), dict(starts=[5, 8], ends=[0, 4104], axes=[0, 2], steps=[-2, 1]),
+                 dict(starts=[4399], ends=[-5000], axes=[2], steps=[-1])):
+        assert_bit_exact(H.slice_(ctx, tw, **args).get_data(), ref.slice_(wide, **args), "slice %s" % args)
     with pytest.raises(H.OperatorError):
         H.slice_(ctx, ctx.move_tensor(nrm(*([1] * 7))), [0], [1])
     with pytest.raises(H.OperatorError):

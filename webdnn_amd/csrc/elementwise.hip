@@ -9,6 +9,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "plane_walk.h"
 
 namespace {
 
@@ -79,41 +80,78 @@ __global__ __launch_bounds__(256) void binary_dense_f32(const float *__restrict_
   if (i < (total & 3)) Y[tail] = apply_f<OP>(L[tail], R[tail]);
 }
 
-// Broadcast path with a vectorisable innermost axis: each thread produces 4
-// consecutive outputs of the innermost axis; an operand whose innermost stride
-// is 1 is read with one 16-byte load, one whose stride is 0 with one scalar load.
-// IDX is the type the output index is decomposed in: unsigned when the tensor
-// has fewer than 2^32 elements (32-bit divisions), long long otherwise.
-template <int OP, typename IDX>
-__global__ __launch_bounds__(256) void binary_bcast_vec_f32(BinaryParams p) {
-  const long long nvec = p.total >> 2;
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  const float *L = (const float *)p.L, *R = (const float *)p.R;
-  float *Y = (float *)p.Y;
-  for (long long v = (long long)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
-       v += stride) {
-    IDX rem = (IDX)(v << 2);
-    long long ol = 0, orr = 0;
+// Broadcast path: the workgroup-tiled walk of plane_walk.h.  UNIT = 4 when the
+// innermost axis can be moved in 16-byte pieces: an operand whose innermost
+// stride is 1 is read with one 16-byte load, one whose stride is 0 with one
+// scalar load.  A thread issues the loads of its four items before it uses any.
+template <int OP, typename T, int UNIT>
+__global__ __launch_bounds__(256) void binary_plane(BinaryParams p, wdh::PlaneWalk w) {
+  const wdh::PlanePos q = wdh::plane_position(w);
+  long long bl = 0, br = 0;
 #pragma unroll
-    for (int d = MAXD - 1; d >= 0; d--) {
-      if (d < p.ndim) {
-        const IDX q = rem / (IDX)p.shape[d];
-        const long long c = (long long)(rem - q * (IDX)p.shape[d]);
-        rem = q;
-        ol += c * p.sl[d];
-        orr += c * p.sr[d];
+  for (int d = 0; d < MAXD - 2; d++) {
+    if (d < w.nd - 2) {
+      bl += (long long)q.oc[d] * p.sl[d];
+      br += (long long)q.oc[d] * p.sr[d];
+    }
+  }
+  const unsigned inner = w.shape[w.nd - 1], second = w.shape[w.nd - 2];
+  const long long sl2 = p.sl[w.nd - 2], sr2 = p.sr[w.nd - 2];
+  const long long sl1 = p.sl[w.nd - 1], sr1 = p.sr[w.nd - 1];
+  const T *L = (const T *)p.L, *R = (const T *)p.R;
+  T *Y = (T *)p.Y;
+  const long long row0 = (long long)q.outer_linear * second;
+  if (UNIT == 4) {
+    f32x4 a[4], b[4];
+    bool ok[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+      ok[k] = x < inner && y < second;
+      if (ok[k]) {
+        const float *l = (const float *)L + bl + (long long)y * sl2 + (long long)x * 4 * sl1;
+        const float *r = (const float *)R + br + (long long)y * sr2 + (long long)x * 4 * sr1;
+        if (sl1) a[k] = *reinterpret_cast<const f32x4 *>(l);
+        else { const float s = *l; a[k] = f32x4{s, s, s, s}; }
+        if (sr1) b[k] = *reinterpret_cast<const f32x4 *>(r);
+        else { const float s = *r; b[k] = f32x4{s, s, s, s}; }
       }
     }
-    f32x4 a, b, y;
-    if (p.sl[p.ndim - 1]) a = *reinterpret_cast<const f32x4 *>(L + ol);
-    else { float s = L[ol]; a = f32x4{s, s, s, s}; }
-    if (p.sr[p.ndim - 1]) b = *reinterpret_cast<const f32x4 *>(R + orr);
-    else { float s = R[orr]; b = f32x4{s, s, s, s}; }
-    y.x = apply_f<OP>(a.x, b.x);
-    y.y = apply_f<OP>(a.y, b.y);
-    y.z = apply_f<OP>(a.z, b.z);
-    y.w = apply_f<OP>(a.w, b.w);
-    *reinterpret_cast<f32x4 *>(Y + (v << 2)) = y;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      if (ok[k]) {
+        const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+        f32x4 v;
+        v.x = apply_f<OP>(a[k].x, b[k].x);
+        v.y = apply_f<OP>(a[k].y, b[k].y);
+        v.z = apply_f<OP>(a[k].z, b[k].z);
+        v.w = apply_f<OP>(a[k].w, b[k].w);
+        *reinterpret_cast<f32x4 *>((float *)Y + ((row0 + y) * inner + x) * 4) = v;
+      }
+    }
+  } else {
+    T a[4], b[4];
+    bool ok[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+      ok[k] = x < inner && y < second;
+      if (ok[k]) {
+        a[k] = L[bl + (long long)y * sl2 + (long long)x * sl1];
+        b[k] = R[br + (long long)y * sr2 + (long long)x * sr1];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      if (ok[k]) {
+        const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+        const long long o = (row0 + y) * inner + x;
+        if (__is_same(T, float))
+          ((float *)Y)[o] = apply_f<OP>((float)a[k], (float)b[k]);
+        else
+          ((int *)Y)[o] = apply_i<OP>((int)a[k], (int)b[k]);
+      }
+    }
   }
 }
 
@@ -152,20 +190,35 @@ unsigned grid_for(long long work_items, int per_block) {
   return (unsigned)blocks;
 }
 
+// Shifts the strides of a rank-1 view by the leading axis the walk adds.
+BinaryParams for_walk(const BinaryParams &p, const wdh::PlaneWalk &w) {
+  if (w.nd == p.ndim) return p;
+  BinaryParams s = p;
+  for (int d = p.ndim; d > 0; d--) { s.sl[d] = p.sl[d - 1]; s.sr[d] = p.sr[d - 1]; }
+  s.sl[0] = s.sr[0] = 0;
+  return s;
+}
+
 template <int OP>
 int launch_binary(const BinaryParams &p, int dtype, bool dense, bool vec) {
   hipStream_t st = wdh::stream();
   const bool small = p.total <= 0xffffffffLL;
+  wdh::PlaneWalk w;
   if (dtype == 0 && dense) {
     hipLaunchKernelGGL(binary_dense_f32<OP>, dim3(grid_for((p.total + 3) / 4, 256)),
                        dim3(256), 0, st, (const float *)p.L, (const float *)p.R,
                        (float *)p.Y, p.total);
-  } else if (dtype == 0 && vec) {
-    const dim3 grid(grid_for(p.total / 4, 256));
-    if (small)
-      hipLaunchKernelGGL((binary_bcast_vec_f32<OP, unsigned>), grid, dim3(256), 0, st, p);
+  } else if (dtype == 0 && vec &&
+             wdh::plan_plane_walk(&w, p.ndim, p.shape, p.shape[p.ndim - 1] / 4)) {
+    hipLaunchKernelGGL((binary_plane<OP, float, 4>), dim3(w.blocks), dim3(256), 0, st,
+                       for_walk(p, w), w);
+  } else if (wdh::plan_plane_walk(&w, p.ndim, p.shape, p.shape[p.ndim - 1])) {
+    if (dtype == 0)
+      hipLaunchKernelGGL((binary_plane<OP, float, 1>), dim3(w.blocks), dim3(256), 0, st,
+                         for_walk(p, w), w);
     else
-      hipLaunchKernelGGL((binary_bcast_vec_f32<OP, long long>), grid, dim3(256), 0, st, p);
+      hipLaunchKernelGGL((binary_plane<OP, int, 1>), dim3(w.blocks), dim3(256), 0, st,
+                         for_walk(p, w), w);
   } else if (dtype == 0) {
     const dim3 grid(grid_for(p.total, 256));
     if (small)
@@ -326,10 +379,18 @@ extern "C" int wdh_binary(int op, int dtype, wdh_buf hL, wdh_buf hR, wdh_buf hY,
   const bool aligned =
       (((uintptr_t)p.L | (uintptr_t)p.R | (uintptr_t)p.Y) & 15) == 0;
   const bool dense = aligned && nd == 1 && p.sl[0] == 1 && p.sr[0] == 1;
-  bool vec = aligned && p.shape[nd - 1] % 4 == 0 && p.sl[nd - 1] <= 1 &&
-             p.sr[nd - 1] <= 1;
-  for (int d = 0; d + 1 < nd && vec; d++)
-    vec = p.sl[d] % 4 == 0 && p.sr[d] % 4 == 0;
+  // 16-byte accesses: the output always; an operand that steps by 1 along the
+  // innermost axis needs an aligned base and outer strides that are multiples
+  // of 4; one that does not step there (stride 0) is read with scalar loads
+  auto vec_ok = [&](const void *base, const long long *st) {
+    if (st[nd - 1] == 0) return true;
+    if (st[nd - 1] != 1 || ((uintptr_t)base & 15)) return false;
+    for (int d = 0; d + 1 < nd; d++)
+      if (st[d] % 4) return false;
+    return true;
+  };
+  const bool vec = ((uintptr_t)p.Y & 15) == 0 && p.shape[nd - 1] % 4 == 0 &&
+                   vec_ok(p.L, p.sl) && vec_ok(p.R, p.sr);
   switch (op) {
     case WDH_BIN_ADD: return launch_binary<WDH_BIN_ADD>(p, dtype, dense, vec);
     case WDH_BIN_SUB: return launch_binary<WDH_BIN_SUB>(p, dtype, dense, vec);

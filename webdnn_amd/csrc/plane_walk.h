@@ -1,0 +1,105 @@
+// Index walk shared by the strided elementwise and copy kernels.
+//
+// A strided tensor view of rank <= 6 (axes already merged on the host) is cut
+// into workgroup tiles over its last two axes; the coordinates on all outer
+// axes come from the workgroup index alone, so they are decomposed once per
+// workgroup (wavefront-uniform arithmetic) and a thread needs no division.
+// Threads run along the innermost axis first: TX = 2^tx_log2 of them, the
+// remaining 256 / TX along the second axis.  Each thread owns four items:
+//   wide   (long innermost axis) : x0 + k*TX on one row,
+//   narrow (short innermost axis): one x on rows y0 + k*TY.
+// The innermost extent is counted in units of UNIT elements (4 for 16-byte
+// accesses, 1 otherwise).
+#pragma once
+#include <stdint.h>
+
+namespace wdh {
+
+constexpr int WALK_MAXD = 6;
+
+struct PlaneWalk {
+  int nd;                     // rank after merging, >= 2 (a leading 1 is added to rank 1)
+  unsigned shape[WALK_MAXD];  // extents, outermost first; shape[nd-1] in units
+  unsigned tx_log2;
+  unsigned xchunks, ychunks;  // workgroups along the innermost / the second axis
+  bool wide;
+  unsigned blocks;            // xchunks * ychunks * product of the outer extents
+};
+
+// Fills `w` for a view of `nd` merged axes whose innermost extent is
+// `inner_units` units.  Returns false when the walk would waste more than half
+// of its threads or needs more workgroups than a grid holds; the caller then
+// uses its per-element kernel.
+inline bool plan_plane_walk(PlaneWalk *w, int nd, const unsigned *shape, unsigned inner_units) {
+  if (nd < 1 || nd > WALK_MAXD || inner_units == 0) return false;
+  unsigned s[WALK_MAXD];
+  int n = 0;
+  if (nd == 1) s[n++] = 1;
+  for (int d = 0; d < nd; d++) s[n++] = shape[d];
+  if (n > WALK_MAXD) return false;
+  s[n - 1] = inner_units;
+  w->nd = n;
+  for (int d = 0; d < n; d++) w->shape[d] = s[d];
+  unsigned lg = 0;
+  while (lg < 8 && (1u << lg) < inner_units) lg++;
+  w->tx_log2 = lg;
+  const unsigned tx = 1u << lg, ty = 256u >> lg;
+  w->wide = inner_units >= 4 * tx;
+  const unsigned long long per_x = w->wide ? 4ull * tx : tx, per_y = w->wide ? ty : 4ull * ty;
+  const unsigned long long xc = (inner_units + per_x - 1) / per_x;
+  const unsigned long long yc = (s[n - 2] + per_y - 1) / per_y;
+  unsigned long long blocks = xc * yc;
+  for (int d = 0; d + 2 < n; d++) {
+    blocks *= s[d];
+    if (blocks > 0x7fffffffULL) return false;
+  }
+  if (blocks > 0x7fffffffULL) return false;
+  const double covered = (double)xc * per_x * (double)yc * per_y;
+  if ((double)inner_units * s[n - 2] < 0.5 * covered) return false;
+  w->xchunks = (unsigned)xc;
+  w->ychunks = (unsigned)yc;
+  w->blocks = (unsigned)blocks;
+  return true;
+}
+
+#ifdef __HIPCC__
+// Position of the calling thread: coordinates on the outer axes (oc[0..nd-3]),
+// the linear index over those axes, the first item (x0, y0) and the step
+// between a thread's four items (dx along the innermost axis, dy along the second).
+struct PlanePos {
+  unsigned oc[WALK_MAXD];
+  unsigned outer_linear;
+  unsigned x0, y0, dx, dy;
+};
+
+__device__ __forceinline__ PlanePos plane_position(const PlaneWalk &w) {
+  PlanePos q;
+  unsigned b = blockIdx.x;
+  const unsigned cx = b % w.xchunks;
+  b /= w.xchunks;
+  const unsigned cy = b % w.ychunks;
+  b /= w.ychunks;
+  q.outer_linear = b;
+#pragma unroll
+  for (int d = WALK_MAXD - 3; d >= 0; d--) {
+    q.oc[d] = 0;
+    if (d < w.nd - 2) {
+      const unsigned t = b / w.shape[d];
+      q.oc[d] = b - t * w.shape[d];
+      b = t;
+    }
+  }
+  const unsigned tx_n = 1u << w.tx_log2, ty_n = 256u >> w.tx_log2;
+  const unsigned tx = threadIdx.x & (tx_n - 1), ty = threadIdx.x >> w.tx_log2;
+  if (w.wide) {
+    q.x0 = cx * tx_n * 4 + tx; q.dx = tx_n;
+    q.y0 = cy * ty_n + ty;     q.dy = 0;
+  } else {
+    q.x0 = cx * tx_n + tx;     q.dx = 0;
+    q.y0 = cy * ty_n * 4 + ty; q.dy = ty_n;
+  }
+  return q;
+}
+#endif
+
+}  // namespace wdh

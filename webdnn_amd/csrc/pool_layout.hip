@@ -8,6 +8,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "plane_walk.h"
 
 namespace {
 
@@ -16,72 +17,60 @@ constexpr int MAXD = 6;
 // ---- max pooling -------------------------------------------------------------
 // One thread per output cell, consecutive threads along ow, so stores are
 // coalesced and the overlapping input windows of neighbouring threads are
-// served by the vector L1.
+// served by the vector L1.  blockIdx.x is the (n, c) plane, blockIdx.y a run of
+// blockDim.x cells of it: one division per thread.  For windows of up to 3x3 (KH, KW
+// > 0) the taps are unrolled and read without branches, so all of a thread's
+// loads are in flight together; taps that fall in the padding read a clamped
+// address and are replaced by -inf, which the strict comparison never selects.
 struct PoolParams {
   const float *X;
   float *Y;
-  long long total;  // n*c*oh*ow
   int h, w, oh, ow, kh, kw, pt, pl, sh, sw, dh, dw;
 };
 
-// IDX: the type the output index is decomposed in (unsigned below 2^32 cells).
-template <typename IDX>
+template <int KH, int KW>
 __global__ __launch_bounds__(256) void maxpool2d_kernel(PoolParams p) {
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
-       i += stride) {
-    const IDX t = (IDX)i / (IDX)p.ow;
-    const int ox = (int)((IDX)i - t * (IDX)p.ow);
-    const IDX plane = t / (IDX)p.oh;  // n*c + c
-    const int oy = (int)(t - plane * (IDX)p.oh);
-    const float *x = p.X + (long long)plane * p.h * p.w;
-    float mv = -INFINITY;
+  const unsigned cell = blockIdx.y * blockDim.x + threadIdx.x;
+  if (cell >= (unsigned)(p.oh * p.ow)) return;
+  const int oy = (int)(cell / (unsigned)p.ow);
+  const int ox = (int)(cell - (unsigned)oy * (unsigned)p.ow);
+  const float *x = p.X + (long long)blockIdx.x * p.h * p.w;
+  float *y = p.Y + (long long)blockIdx.x * p.oh * p.ow;
+  float mv = -INFINITY;
+  if constexpr (KH > 0) {
+    float v[KH * KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ky++) {
+      const int iy = oy * p.sh - p.pt + ky * p.dh;
+      const bool rok = (unsigned)iy < (unsigned)p.h;
+      const int cy = rok ? iy : 0;
+#pragma unroll
+      for (int kx = 0; kx < KW; kx++) {
+        const int ix = ox * p.sw - p.pl + kx * p.dw;
+        const bool ok = rok && (unsigned)ix < (unsigned)p.w;
+        const float t = x[cy * p.w + (ok ? ix : 0)];
+        v[ky * KW + kx] = ok ? t : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < KH * KW; i++)
+      if (v[i] > mv) mv = v[i];  // strict, NaN never selected: maxpool.ts:98-101
+  } else {
     for (int ky = 0; ky < p.kh; ky++) {
       const int iy = oy * p.sh - p.pt + ky * p.dh;
       if ((unsigned)iy >= (unsigned)p.h) continue;
       for (int kx = 0; kx < p.kw; kx++) {
         const int ix = ox * p.sw - p.pl + kx * p.dw;
         if ((unsigned)ix >= (unsigned)p.w) continue;
-        const float v = x[iy * p.w + ix];
-        if (v > mv) mv = v;  // strict, NaN never selected: maxpool.ts:98-101
+        const float t = x[iy * p.w + ix];
+        if (t > mv) mv = t;
       }
     }
-    p.Y[i] = mv;
   }
+  y[cell] = mv;
 }
 
 // ---- transpose -----------------------------------------------------------------
-struct GatherCopyParams {
-  const uint32_t *X;
-  uint32_t *Y;
-  long long total;
-  int ndim;
-  unsigned shape[MAXD];   // output shape
-  long long sin[MAXD];    // input stride of each output axis
-};
-
-// Generic: thread per output element.  Coalesced on the output side always,
-// on the input side when the last output axis has input stride 1.
-// IDX: the type the output index is decomposed in (unsigned below 2^32 elements).
-template <typename IDX>
-__global__ __launch_bounds__(256) void gather_copy_kernel(GatherCopyParams p) {
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < p.total;
-       i += stride) {
-    IDX rem = (IDX)i;
-    long long off = 0;
-#pragma unroll
-    for (int d = MAXD - 1; d >= 0; d--) {
-      if (d < p.ndim) {
-        const IDX q = rem / (IDX)p.shape[d];
-        off += (long long)(rem - q * (IDX)p.shape[d]) * p.sin[d];
-        rem = q;
-      }
-    }
-    p.Y[i] = p.X[off];
-  }
-}
-
 // Strided copy (Slice, Concat, Split): both sides addressed through strides.
 struct StridedCopyParams {
   const uint32_t *X;
@@ -116,10 +105,53 @@ __global__ __launch_bounds__(256) void strided_copy_kernel(StridedCopyParams p) 
   }
 }
 
+// Strided copy through the workgroup-tiled walk of plane_walk.h: no division
+// per thread, and 16 bytes per access (UNIT = 4) when both sides step by 1
+// along the innermost axis and every other stride and both bases are
+// multiples of 4 elements.  A thread issues its four loads before its stores.
+template <int UNIT>
+__global__ __launch_bounds__(256) void copy_plane(StridedCopyParams p, wdh::PlaneWalk w) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const wdh::PlanePos q = wdh::plane_position(w);
+  long long bx = 0, by = 0;
+#pragma unroll
+  for (int d = 0; d < MAXD - 2; d++) {
+    if (d < w.nd - 2) {
+      bx += (long long)q.oc[d] * p.sx[d];
+      by += (long long)q.oc[d] * p.sy[d];
+    }
+  }
+  const unsigned inner = w.shape[w.nd - 1], second = w.shape[w.nd - 2];
+  const long long sx2 = p.sx[w.nd - 2], sy2 = p.sy[w.nd - 2];
+  const long long sx1 = p.sx[w.nd - 1] * UNIT, sy1 = p.sy[w.nd - 1] * UNIT;
+  u32x4 v4[4];
+  uint32_t v1[4];
+  bool ok[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+    ok[k] = x < inner && y < second;
+    if (ok[k]) {
+      const uint32_t *src = p.X + bx + (long long)y * sx2 + (long long)x * sx1;
+      if (UNIT == 4) v4[k] = *reinterpret_cast<const u32x4 *>(src);
+      else v1[k] = *src;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    if (ok[k]) {
+      const unsigned x = q.x0 + k * q.dx, y = q.y0 + k * q.dy;
+      uint32_t *dst = p.Y + by + (long long)y * sy2 + (long long)x * sy1;
+      if (UNIT == 4) *reinterpret_cast<u32x4 *>(dst) = v4[k];
+      else *dst = v1[k];
+    }
+  }
+}
+
 // Tiled: when the input-contiguous axis `a` is not the last output axis, a
-// workgroup moves a 64x64 tile spanned by (axis a, last axis) through LDS:
+// workgroup moves a 4096-element tile spanned by (axis a, last axis) through LDS:
 // reads run along axis a (contiguous in X), writes along the last axis
-// (contiguous in Y).  The 65-float row pitch keeps both phases free of bank
+// (contiguous in Y).  The odd row pitch keeps both phases free of bank
 // conflicts.  All remaining axes are folded into blockIdx.z.
 struct TileParams {
   const uint32_t *X;
@@ -133,8 +165,12 @@ struct TileParams {
   long long l_in;         // input stride of the last axis (its output stride is 1)
 };
 
+// TA x TL tile (TA along axis a, TL = 4096 / TA along the last axis): the
+// narrower TA shapes keep all threads busy when axis a is short.
+template <int TA>
 __global__ __launch_bounds__(256) void transpose_tiled_kernel(TileParams p) {
-  __shared__ uint32_t tile[64][65];
+  constexpr int TL = 4096 / TA;
+  __shared__ uint32_t tile[TL][TA + 1];
   long long rem = blockIdx.z, in_off = 0, out_off = 0;
 #pragma unroll
   for (int d = MAXD - 1; d >= 0; d--) {
@@ -146,18 +182,24 @@ __global__ __launch_bounds__(256) void transpose_tiled_kernel(TileParams p) {
       out_off += c * p.osout[d];
     }
   }
-  const unsigned a0 = blockIdx.x * 64, l0 = blockIdx.y * 64;
-  const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
-  // read: tx runs along axis a
-  for (unsigned r = ty; r < 64; r += 4) {
-    unsigned a = a0 + tx, l = l0 + r;
-    if (a < p.na && l < p.nl) tile[r][tx] = p.X[in_off + (long long)l * p.l_in + a];
+  const unsigned a0 = blockIdx.x * TA, l0 = blockIdx.y * TL;
+  {  // read: consecutive threads run along axis a
+    const unsigned ta = threadIdx.x % TA, a = a0 + ta;
+    for (unsigned r = threadIdx.x / TA; r < TL; r += 256 / TA) {
+      const unsigned l = l0 + r;
+      if (a < p.na && l < p.nl) tile[r][ta] = p.X[in_off + (long long)l * p.l_in + a];
+    }
   }
   __syncthreads();
-  // write: tx runs along the last axis
-  for (unsigned r = ty; r < 64; r += 4) {
-    unsigned a = a0 + r, l = l0 + tx;
-    if (a < p.na && l < p.nl) p.Y[out_off + (long long)a * p.a_out + l] = tile[tx][r];
+  {  // write: consecutive threads run along the last axis
+    const unsigned tl = threadIdx.x & 63;
+    for (unsigned r = threadIdx.x >> 6; r < TA; r += 4) {
+      const unsigned a = a0 + r;
+      for (unsigned c = tl; c < TL; c += 64) {
+        const unsigned l = l0 + c;
+        if (a < p.na && l < p.nl) p.Y[out_off + (long long)a * p.a_out + l] = tile[c][r];
+      }
+    }
   }
 }
 
@@ -189,6 +231,31 @@ unsigned grid_for(long long items) {
   return (unsigned)blocks;
 }
 
+// Launches the copy described by `g` (axes merged, total > 0).
+int launch_strided_copy(const StridedCopyParams &g) {
+  hipStream_t st = wdh::stream();
+  const int nd = g.ndim;
+  bool vec = g.shape[nd - 1] % 4 == 0 && g.sx[nd - 1] == 1 && g.sy[nd - 1] == 1 &&
+             (((uintptr_t)g.X | (uintptr_t)g.Y) & 15) == 0;
+  for (int d = 0; d + 1 < nd && vec; d++) vec = g.sx[d] % 4 == 0 && g.sy[d] % 4 == 0;
+  wdh::PlaneWalk w;
+  if (wdh::plan_plane_walk(&w, nd, g.shape, vec ? g.shape[nd - 1] / 4 : g.shape[nd - 1])) {
+    StridedCopyParams s = g;
+    if (w.nd != nd) {  // rank 1: the walk adds a leading axis of extent 1
+      for (int d = nd; d > 0; d--) { s.sx[d] = g.sx[d - 1]; s.sy[d] = g.sy[d - 1]; }
+      s.sx[0] = s.sy[0] = 0;
+    }
+    if (vec) hipLaunchKernelGGL(copy_plane<4>, dim3(w.blocks), dim3(256), 0, st, s, w);
+    else hipLaunchKernelGGL(copy_plane<1>, dim3(w.blocks), dim3(256), 0, st, s, w);
+  } else if (g.total <= 0xffffffffLL) {
+    hipLaunchKernelGGL(strided_copy_kernel<unsigned>, dim3(grid_for(g.total)), dim3(256), 0, st, g);
+  } else {
+    hipLaunchKernelGGL(strided_copy_kernel<long long>, dim3(grid_for(g.total)), dim3(256), 0, st, g);
+  }
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
 }  // namespace
 
 using wdh::fail;
@@ -202,21 +269,24 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
     return fail(WDH_EINVAL, "wdh_maxpool2d: bad geometry");
   // every input read is bounds-checked in the kernel, so an (oh, ow) larger than
   // the geometry implies only yields windows that lie in the padding (-inf)
+  const long long planes = (long long)n * c, cells = (long long)oh * ow;
+  if (planes == 0 || cells == 0) return WDH_OK;
+  if (planes > 0x7fffffffLL || cells > 65535LL * 256 || (long long)h * w > 0x7fffffffLL)
+    return fail(WDH_EINVAL, "wdh_maxpool2d: %lld planes of %lld cells exceed the launch grid",
+                planes, cells);
   PoolParams p;
-  p.total = (long long)n * c * oh * ow;
-  if (p.total == 0) return WDH_OK;
   void *px, *py;
-  if (!wdh::operand(hX, (size_t)n * c * h * w * 4, "wdh_maxpool2d: X", &px)) return WDH_EINVAL;
-  if (!wdh::operand(hY, (size_t)p.total * 4, "wdh_maxpool2d: Y", &py)) return WDH_EINVAL;
+  if (!wdh::operand(hX, (size_t)planes * h * w * 4, "wdh_maxpool2d: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)planes * cells * 4, "wdh_maxpool2d: Y", &py)) return WDH_EINVAL;
   p.X = (const float *)px; p.Y = (float *)py;
   p.h = h; p.w = w; p.oh = oh; p.ow = ow; p.kh = kh; p.kw = kw;
   p.pt = pt; p.pl = pl; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
-  if (p.total <= 0xffffffffLL)
-    hipLaunchKernelGGL(maxpool2d_kernel<unsigned>, dim3(grid_for(p.total)), dim3(256), 0,
-                       wdh::stream(), p);
-  else
-    hipLaunchKernelGGL(maxpool2d_kernel<long long>, dim3(grid_for(p.total)), dim3(256), 0,
-                       wdh::stream(), p);
+  const unsigned threads = cells <= 64 ? 64 : cells <= 128 ? 128 : 256;
+  const dim3 grid((unsigned)planes, (unsigned)((cells + threads - 1) / threads)), block(threads);
+  hipStream_t st = wdh::stream();
+  if (kh == 3 && kw == 3) hipLaunchKernelGGL((maxpool2d_kernel<3, 3>), grid, block, 0, st, p);
+  else if (kh == 2 && kw == 2) hipLaunchKernelGGL((maxpool2d_kernel<2, 2>), grid, block, 0, st, p);
+  else hipLaunchKernelGGL((maxpool2d_kernel<0, 0>), grid, block, 0, st, p);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }
@@ -281,24 +351,24 @@ extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
     }
     t.na = shape[a]; t.nl = shape[nd - 1];
     t.a_out = sout[a]; t.l_in = sin[nd - 1];
-    unsigned gx = (t.na + 63) / 64, gy = (t.nl + 63) / 64;
+    const unsigned ta = (t.na <= 16 && t.nl >= 256) ? 16 : (t.na <= 32 && t.nl >= 128) ? 32 : 64;
+    const unsigned tl = 4096 / ta;
+    const unsigned gx = (t.na + ta - 1) / ta, gy = (t.nl + tl - 1) / tl;
     if (nouter <= 65535 && gy <= 65535) {
-      hipLaunchKernelGGL(transpose_tiled_kernel, dim3(gx, gy, (unsigned)nouter),
-                         dim3(256), 0, st, t);
+      const dim3 grid(gx, gy, (unsigned)nouter);
+      if (ta == 16) hipLaunchKernelGGL(transpose_tiled_kernel<16>, grid, dim3(256), 0, st, t);
+      else if (ta == 32) hipLaunchKernelGGL(transpose_tiled_kernel<32>, grid, dim3(256), 0, st, t);
+      else hipLaunchKernelGGL(transpose_tiled_kernel<64>, grid, dim3(256), 0, st, t);
       WDH_LAUNCH_CHECK();
       return WDH_OK;
     }
   }
-  GatherCopyParams g = {};
+  // no tile to exchange: a strided read into the dense output
+  StridedCopyParams g = {};
   g.X = (const uint32_t *)px; g.Y = (uint32_t *)py;
   g.total = total; g.ndim = nd;
-  for (int d = 0; d < nd; d++) { g.shape[d] = shape[d]; g.sin[d] = sin[d]; }
-  if (total <= 0xffffffffLL)
-    hipLaunchKernelGGL(gather_copy_kernel<unsigned>, dim3(grid_for(total)), dim3(256), 0, st, g);
-  else
-    hipLaunchKernelGGL(gather_copy_kernel<long long>, dim3(grid_for(total)), dim3(256), 0, st, g);
-  WDH_LAUNCH_CHECK();
-  return WDH_OK;
+  for (int d = 0; d < nd; d++) { g.shape[d] = shape[d]; g.sx[d] = sin[d]; g.sy[d] = sout[d]; }
+  return launch_strided_copy(g);
 }
 
 extern "C" int wdh_gather(wdh_buf hD, wdh_buf hI, wdh_buf hY, int64_t outer,
@@ -372,10 +442,5 @@ extern "C" int wdh_strided_copy(wdh_buf hX, int64_t x_offset, wdh_buf hY, int64_
                                  wdh::stream()));
     return WDH_OK;
   }
-  if (total <= 0xffffffffLL)
-    hipLaunchKernelGGL(strided_copy_kernel<unsigned>, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
-  else
-    hipLaunchKernelGGL(strided_copy_kernel<long long>, dim3(grid_for(total)), dim3(256), 0, wdh::stream(), g);
-  WDH_LAUNCH_CHECK();
-  return WDH_OK;
+  return launch_strided_copy(g);
 }

@@ -38,38 +38,77 @@ __device__ __forceinline__ double wave_sum_d(double v) {
   return v;
 }
 
+// Register-resident rows.  VEC: rows are 16-byte aligned and a multiple of 4
+// long, and lane l holds elements 4l..4l+3 of every 256-element segment (one
+// 16-byte access each); otherwise lane l holds elements l, l+64, ...
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <bool VEC>
+__device__ __forceinline__ int elem_index(int lane, int i) {
+  return VEC ? lane * 4 + 256 * (i >> 2) + (i & 3) : lane + 64 * i;
+}
+
+template <int NV, bool VEC>
+__device__ __forceinline__ void load_row(const float *x, int len, int lane, float fill,
+                                         float (&v)[NV]) {
+  if constexpr (VEC) {
+#pragma unroll
+    for (int i = 0; i < NV; i += 4) {
+      const int idx = lane * 4 + 64 * i;
+      f32x4 t = {fill, fill, fill, fill};
+      if (idx < len) t = *reinterpret_cast<const f32x4 *>(x + idx);
+      v[i] = t.x; v[i + 1] = t.y; v[i + 2] = t.z; v[i + 3] = t.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int idx = lane + 64 * i;
+      v[i] = idx < len ? x[idx] : fill;
+    }
+  }
+}
+
+template <int NV, bool VEC>
+__device__ __forceinline__ void store_row(float *y, int len, int lane, const float (&v)[NV]) {
+  if constexpr (VEC) {
+#pragma unroll
+    for (int i = 0; i < NV; i += 4) {
+      const int idx = lane * 4 + 64 * i;
+      if (idx < len) *reinterpret_cast<f32x4 *>(y + idx) = f32x4{v[i], v[i + 1], v[i + 2], v[i + 3]};
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int idx = lane + 64 * i;
+      if (idx < len) y[idx] = v[i];
+    }
+  }
+}
+
 // ---- softmax ---------------------------------------------------------------
-template <int NV>
+template <int NV, bool VEC>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_reg(
     const float *__restrict__ X, float *__restrict__ Y, long long outer, int len) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
-  const float *x = X + row * len;
-  float *y = Y + row * len;
   float v[NV];
+  load_row<NV, VEC>(X + row * len, len, lane, -INFINITY, v);
   float mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    v[i] = idx < len ? x[idx] : -INFINITY;
-    mx = fmaxf(mx, v[i]);  // fmaxf skips NaN, like `if (v > max)`
-  }
+  for (int i = 0; i < NV; i++) mx = fmaxf(mx, v[i]);  // fmaxf skips NaN, like `if (v > max)`
   mx = wave_max(mx);
   float sum = 0.0f;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    float e = idx < len ? expf(v[i] - mx) : 0.0f;
+    const float e = elem_index<VEC>(lane, i) < len ? expf(v[i] - mx) : 0.0f;
     v[i] = e;
     sum += e;
   }
   sum = wave_sum(sum);
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    if (idx < len) y[idx] = v[i] / sum;
-  }
+  for (int i = 0; i < NV; i++) v[i] = v[i] / sum;
+  store_row<NV, VEC>(Y + row * len, len, lane, v);
 }
 
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_stream(
@@ -93,7 +132,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_stream(
 }
 
 // ---- layer normalisation -----------------------------------------------------
-template <int NV>
+template <int NV, bool VEC>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
     const float *__restrict__ X, const float *__restrict__ G,
     const float *__restrict__ Bt, float *__restrict__ Y, long long outer, int len,
@@ -101,38 +140,32 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
-  const float *x = X + row * len;
-  float *y = Y + row * len;
-  float v[NV];
+  float v[NV], g[NV], bt[NV];
+  load_row<NV, VEC>(X + row * len, len, lane, 0.0f, v);
+  if (G) load_row<NV, VEC>(G, len, lane, 0.0f, g);
+  if (Bt) load_row<NV, VEC>(Bt, len, lane, 0.0f, bt);
   double s = 0.0;
 #pragma unroll
-  for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    v[i] = idx < len ? x[idx] : 0.0f;
-    s += (double)v[i];
-  }
+  for (int i = 0; i < NV; i++) s += (double)v[i];
   const float mean = (float)(wave_sum_d(s) / (double)len);
   double q = 0.0;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    float d = v[i] - mean;
+    const float d = v[i] - mean;
     v[i] = d;
-    float sq = d * d;
-    q += idx < len ? (double)sq : 0.0;
+    const float sq = d * d;
+    q += elem_index<VEC>(lane, i) < len ? (double)sq : 0.0;
   }
   const float var = (float)(wave_sum_d(q) / (double)len);
   const float denom = (float)sqrt((double)(var + eps));
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    int idx = lane + 64 * i;
-    if (idx < len) {
-      float t = v[i] / denom;
-      if (G) t = t * G[idx];
-      if (Bt) t = t + Bt[idx];
-      y[idx] = t;
-    }
+    float t = v[i] / denom;
+    if (G) t = t * g[i];
+    if (Bt) t = t + bt[i];
+    v[i] = t;
   }
+  store_row<NV, VEC>(Y + row * len, len, lane, v);
 }
 
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_stream(
@@ -164,18 +197,35 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_stream(
 
 // ---- mean over trailing elements ------------------------------------------------
 // Short rows (len <= 64, e.g. the 7x7 = 49 cells of ResNet's final pooling):
-// one thread per row, summing in the reference's order.  Neighbouring threads
-// own neighbouring rows, so a wavefront's loads together cover one contiguous
-// span of 64*len floats that stays in the vector L1 between iterations.
-__global__ __launch_bounds__(256) void mean_rows_small(const float *__restrict__ X,
-                                                       float *__restrict__ Y,
-                                                       long long outer, int len) {
-  const long long row = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (row >= outer) return;
-  const float *x = X + row * len;
-  double s = 0.0;
-  for (int i = 0; i < len; i++) s += (double)x[i];
-  Y[row] = (float)(s / (double)len);
+// a wavefront owns 64 consecutive rows, which are one contiguous span of
+// 64*len floats.  It copies them row by row into LDS (each load instruction
+// reads one row: contiguous, coalesced), then every lane sums its own row from
+// LDS in the reference's order.  The odd row pitch keeps the lanes' LDS reads
+// on distinct banks.
+constexpr int SMALL_ROW_WAVES = 2;
+__global__ __launch_bounds__(64 * SMALL_ROW_WAVES) void mean_rows_small(
+    const float *__restrict__ X, float *__restrict__ Y, long long outer, int len) {
+  __shared__ float stage[SMALL_ROW_WAVES][64 * 65];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long long row0 = ((long long)blockIdx.x * SMALL_ROW_WAVES + wave) * 64;
+  if (row0 >= outer) return;
+  const int rows = outer - row0 < 64 ? (int)(outer - row0) : 64;
+  const int pitch = len | 1;
+  float *mine = stage[wave];
+  const float *x = X + row0 * len;
+  if (lane < len) {
+#pragma unroll 8
+    for (int r = 0; r < rows; r++) mine[r * pitch + lane] = x[(long long)r * len + lane];
+  }
+  // the wavefront reads back only what it wrote itself
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane < rows) {
+    double s = 0.0;
+    for (int i = 0; i < len; i++) s += (double)mine[lane * pitch + i];
+    Y[row0 + lane] = (float)(s / (double)len);
+  }
 }
 
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void mean_rows_wave(
@@ -217,14 +267,21 @@ extern "C" int wdh_softmax(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   float *Y = (float *)py;
   dim3 grid(row_blocks(outer)), block(64 * WAVES_PER_BLOCK);
   hipStream_t st = wdh::stream();
+  const bool vec = len % 4 == 0 && (((uintptr_t)px | (uintptr_t)py) & 15) == 0;
   if (len <= 64 * 2)
-    hipLaunchKernelGGL(softmax_rows_reg<2>, grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<2, false>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 8 && vec)
+    hipLaunchKernelGGL((softmax_rows_reg<8, true>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 8)
-    hipLaunchKernelGGL(softmax_rows_reg<8>, grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<8, false>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 16 && vec)
+    hipLaunchKernelGGL((softmax_rows_reg<16, true>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 16)
-    hipLaunchKernelGGL(softmax_rows_reg<16>, grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<16, false>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 32 && vec)
+    hipLaunchKernelGGL((softmax_rows_reg<32, true>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 32)
-    hipLaunchKernelGGL(softmax_rows_reg<32>, grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<32, false>), grid, block, 0, st, X, Y, outer, len);
   else
     hipLaunchKernelGGL(softmax_rows_stream, grid, block, 0, st, X, Y, outer, len);
   WDH_LAUNCH_CHECK();
@@ -246,10 +303,16 @@ extern "C" int wdh_layernorm(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY,
   float *Y = (float *)py;
   dim3 grid(row_blocks(outer)), block(64 * WAVES_PER_BLOCK);
   hipStream_t st = wdh::stream();
-  if (len <= 64 * 4)
-    hipLaunchKernelGGL(layernorm_rows_reg<4>, grid, block, 0, st, X, G, B, Y, outer, len, eps);
+  const bool vec = len % 4 == 0 &&
+                   (((uintptr_t)px | (uintptr_t)py | (uintptr_t)pg | (uintptr_t)pb) & 15) == 0;
+  if (len <= 64 * 4 && vec)
+    hipLaunchKernelGGL((layernorm_rows_reg<4, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+  else if (len <= 64 * 4)
+    hipLaunchKernelGGL((layernorm_rows_reg<4, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+  else if (len <= 64 * 16 && vec)
+    hipLaunchKernelGGL((layernorm_rows_reg<16, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
   else if (len <= 64 * 16)
-    hipLaunchKernelGGL(layernorm_rows_reg<16>, grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL((layernorm_rows_reg<16, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
   else
     hipLaunchKernelGGL(layernorm_rows_stream, grid, block, 0, st, X, G, B, Y, outer, len, eps);
   WDH_LAUNCH_CHECK();
@@ -266,8 +329,10 @@ extern "C" int wdh_reduce_mean(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   if (!wdh::operand(hY, (size_t)outer * 4, "wdh_reduce_mean: Y", &py)) return WDH_EINVAL;
   hipStream_t st = wdh::stream();
   if (len <= 64 && outer >= 4096)
-    hipLaunchKernelGGL(mean_rows_small, dim3((unsigned)((outer + 255) / 256)), dim3(256),
-                       0, st, (const float *)px, (float *)py, (long long)outer, len);
+    hipLaunchKernelGGL(mean_rows_small,
+                       dim3((unsigned)((outer + 64 * SMALL_ROW_WAVES - 1) / (64 * SMALL_ROW_WAVES))),
+                       dim3(64 * SMALL_ROW_WAVES), 0, st, (const float *)px, (float *)py,
+                       (long long)outer, len);
   else
     hipLaunchKernelGGL(mean_rows_wave, dim3(row_blocks(outer)),
                        dim3(64 * WAVES_PER_BLOCK), 0, st, (const float *)px,
