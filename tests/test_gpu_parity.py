@@ -339,12 +339,17 @@ def test_maxpool_resnet_stem_full(ctx):
     dict(kernel_shape=[3, 3], strides=[4, 4], pads=[1, 1, 1, 1]),
 ])
 def test_maxpool_attributes(ctx, attrs):
-    x = nrm(2, 3, 10, 13)
-    x[0, 0, 0, 0] = np.nan
-    got = H.maxpool(ctx, ctx.move_tensor(x), **attrs)
-    want = ref.maxpool(x, **attrs)
-    assert tuple(got.dims) == want.shape
-    assert_bit_exact(got.get_data(), want, "maxpool %s" % (attrs,))
+    # small planes take the thread-per-cell kernel, the larger ones the LDS band kernel
+    # (with and without 16-byte loads)
+    for shape in ((2, 3, 10, 13), (2, 3, 40, 46), (1, 2, 36, 48), (1, 1, 70, 130)):
+        x = nrm(*shape)
+        x[0, 0, 0, 0] = np.nan
+        x[0, 0, 5, 7] = np.nan
+        x[0, 0, -1, -1] = -np.inf
+        got = H.maxpool(ctx, ctx.move_tensor(x), **attrs)
+        want = ref.maxpool(x, **attrs)
+        assert tuple(got.dims) == want.shape
+        assert_bit_exact(got.get_data(), want, "maxpool %s on %s" % (attrs, shape))
 
 
 def test_maxpool_errors(ctx):

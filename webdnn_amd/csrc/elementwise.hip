@@ -210,14 +210,14 @@ int launch_binary(const BinaryParams &p, int dtype, bool dense, bool vec) {
                        (float *)p.Y, p.total);
   } else if (dtype == 0 && vec &&
              wdh::plan_plane_walk(&w, p.ndim, p.shape, p.shape[p.ndim - 1] / 4)) {
-    hipLaunchKernelGGL((binary_plane<OP, float, 4>), dim3(w.blocks), dim3(256), 0, st,
+    hipLaunchKernelGGL((binary_plane<OP, float, 4>), wdh::plane_grid(w), dim3(256), 0, st,
                        for_walk(p, w), w);
   } else if (wdh::plan_plane_walk(&w, p.ndim, p.shape, p.shape[p.ndim - 1])) {
     if (dtype == 0)
-      hipLaunchKernelGGL((binary_plane<OP, float, 1>), dim3(w.blocks), dim3(256), 0, st,
+      hipLaunchKernelGGL((binary_plane<OP, float, 1>), wdh::plane_grid(w), dim3(256), 0, st,
                          for_walk(p, w), w);
     else
-      hipLaunchKernelGGL((binary_plane<OP, int, 1>), dim3(w.blocks), dim3(256), 0, st,
+      hipLaunchKernelGGL((binary_plane<OP, int, 1>), wdh::plane_grid(w), dim3(256), 0, st,
                          for_walk(p, w), w);
   } else if (dtype == 0) {
     const dim3 grid(grid_for(p.total, 256));

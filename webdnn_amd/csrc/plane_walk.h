@@ -23,7 +23,9 @@ struct PlaneWalk {
   unsigned tx_log2;
   unsigned xchunks, ychunks;  // workgroups along the innermost / the second axis
   bool wide;
+  bool grid3d;                // launch grid (xchunks, ychunks, outer) instead of one folded axis
   unsigned blocks;            // xchunks * ychunks * product of the outer extents
+  unsigned outer;             // product of the outer extents
 };
 
 // Fills `w` for a view of `nd` merged axes whose innermost extent is
@@ -31,38 +33,60 @@ struct PlaneWalk {
 // of its threads or needs more workgroups than a grid holds; the caller then
 // uses its per-element kernel.
 inline bool plan_plane_walk(PlaneWalk *w, int nd, const unsigned *shape, unsigned inner_units) {
-  if (nd < 1 || nd > WALK_MAXD || inner_units == 0) return false;
+  if (nd < 1 || nd > WALK_MAXD || inner_units == 0 || inner_units > 0x7fffffffu) return false;
   unsigned s[WALK_MAXD];
   int n = 0;
   if (nd == 1) s[n++] = 1;
   for (int d = 0; d < nd; d++) s[n++] = shape[d];
   if (n > WALK_MAXD) return false;
   s[n - 1] = inner_units;
+  if (s[n - 2] > 0x7fffffffu) return false;
   w->nd = n;
   for (int d = 0; d < n; d++) w->shape[d] = s[d];
-  unsigned lg = 0;
-  while (lg < 8 && (1u << lg) < inner_units) lg++;
-  w->tx_log2 = lg;
-  const unsigned tx = 1u << lg, ty = 256u >> lg;
-  w->wide = inner_units >= 4 * tx;
-  const unsigned long long per_x = w->wide ? 4ull * tx : tx, per_y = w->wide ? ty : 4ull * ty;
-  const unsigned long long xc = (inner_units + per_x - 1) / per_x;
-  const unsigned long long yc = (s[n - 2] + per_y - 1) / per_y;
-  unsigned long long blocks = xc * yc;
-  for (int d = 0; d + 2 < n; d++) {
-    blocks *= s[d];
-    if (blocks > 0x7fffffffULL) return false;
+  // TX: the power of two that covers a short innermost axis; for longer ones
+  // whichever of 64 / 128 / 256 leaves the fewest threads without an item
+  unsigned lg_lo = 0;
+  while (lg_lo < 8 && (1u << lg_lo) < inner_units) lg_lo++;
+  if (lg_lo > 6) lg_lo = 6;
+  const unsigned lg_hi = inner_units > 64 ? 8 : lg_lo;
+  double best = -1.0;
+  unsigned long long xc = 0, yc = 0;
+  for (unsigned lg = lg_hi; lg >= lg_lo; lg--) {
+    const unsigned tx = 1u << lg, ty = 256u >> lg;
+    const bool wide = inner_units >= 4 * tx;
+    const unsigned long long px = wide ? 4ull * tx : tx, py = wide ? ty : 4ull * ty;
+    const unsigned long long cx = (inner_units + px - 1) / px, cy = (s[n - 2] + py - 1) / py;
+    const double eff = (double)inner_units * s[n - 2] / ((double)cx * px * (double)cy * py);
+    if (eff > best + 1e-9) {
+      best = eff; w->tx_log2 = lg; w->wide = wide;
+      xc = cx; yc = cy;
+    }
+    if (lg == 0) break;
   }
+  unsigned long long outer = 1;
+  for (int d = 0; d + 2 < n; d++) {
+    outer *= s[d];
+    if (outer > 0x7fffffffULL) return false;
+  }
+  const unsigned long long blocks = xc * yc * outer;
   if (blocks > 0x7fffffffULL) return false;
-  const double covered = (double)xc * per_x * (double)yc * per_y;
-  if ((double)inner_units * s[n - 2] < 0.5 * covered) return false;
+  if (best < 0.5) return false;
   w->xchunks = (unsigned)xc;
   w->ychunks = (unsigned)yc;
   w->blocks = (unsigned)blocks;
+  w->outer = (unsigned)outer;
+  w->grid3d = yc <= 65535 && outer <= 65535;
   return true;
 }
 
 #ifdef __HIPCC__
+// The launch grid of a planned walk.  The three-axis form hands the kernel its
+// tile and outer index without any division; extents beyond a grid axis's
+// limit fall back to one folded axis.
+inline dim3 plane_grid(const PlaneWalk &w) {
+  return w.grid3d ? dim3(w.xchunks, w.ychunks, w.outer) : dim3(w.blocks);
+}
+
 // Position of the calling thread: coordinates on the outer axes (oc[0..nd-3]),
 // the linear index over those axes, the first item (x0, y0) and the step
 // between a thread's four items (dx along the innermost axis, dy along the second).
@@ -74,14 +98,19 @@ struct PlanePos {
 
 __device__ __forceinline__ PlanePos plane_position(const PlaneWalk &w) {
   PlanePos q;
-  unsigned b = blockIdx.x;
-  const unsigned cx = b % w.xchunks;
-  b /= w.xchunks;
-  const unsigned cy = b % w.ychunks;
-  b /= w.ychunks;
+  unsigned b, cx, cy;
+  if (w.grid3d) {
+    cx = blockIdx.x; cy = blockIdx.y; b = blockIdx.z;
+  } else {
+    b = blockIdx.x;
+    cx = b % w.xchunks;
+    b /= w.xchunks;
+    cy = b % w.ychunks;
+    b /= w.ychunks;
+  }
   q.outer_linear = b;
 #pragma unroll
-  for (int d = WALK_MAXD - 3; d >= 0; d--) {
+  for (int d = WALK_MAXD - 3; d >= 1; d--) {
     q.oc[d] = 0;
     if (d < w.nd - 2) {
       const unsigned t = b / w.shape[d];
@@ -89,6 +118,7 @@ __device__ __forceinline__ PlanePos plane_position(const PlaneWalk &w) {
       b = t;
     }
   }
+  q.oc[0] = w.nd > 2 ? b : 0;  // the outermost coordinate is what remains
   const unsigned tx_n = 1u << w.tx_log2, ty_n = 256u >> w.tx_log2;
   const unsigned tx = threadIdx.x & (tx_n - 1), ty = threadIdx.x >> w.tx_log2;
   if (w.wide) {

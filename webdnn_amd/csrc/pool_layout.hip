@@ -70,6 +70,64 @@ __global__ __launch_bounds__(256) void maxpool2d_kernel(PoolParams p) {
   y[cell] = mv;
 }
 
+// Band variant: a workgroup owns `rows` output rows of one plane.  The input
+// rows they touch are whole rows, hence one contiguous span; it is copied to
+// LDS with coalesced (16-byte where VEC) loads, and the window taps are read
+// from there.  Global memory then sees every input element about once per
+// band instead of once per tap.
+struct PoolBand {
+  int rows;     // output rows per workgroup
+  int in_rows;  // input rows one band can touch: (rows-1)*sh + (kh-1)*dh + 1
+  int tx_log2;  // threads along ow = 2^tx_log2 (at most one wavefront)
+};
+
+template <int KH, int KW, bool VEC>
+__global__ __launch_bounds__(256) void maxpool2d_band_kernel(PoolParams p, PoolBand b) {
+  extern __shared__ float band[];
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const int oy0 = blockIdx.y * b.rows;
+  const int iy0 = oy0 * p.sh - p.pt;                // may lie in the top padding
+  const int lo = iy0 < 0 ? 0 : iy0;
+  const int hi = iy0 + b.in_rows < p.h ? iy0 + b.in_rows : p.h;
+  const float *x = p.X + (long long)blockIdx.x * p.h * p.w + (long long)lo * p.w;
+  const int count = (hi - lo) * p.w;                // floats of rows lo..hi-1
+  if (VEC) {
+    for (int i = threadIdx.x * 4; i < count; i += 1024)
+      *reinterpret_cast<f32x4 *>(band + i) = *reinterpret_cast<const f32x4 *>(x + i);
+  } else {
+    for (int i = threadIdx.x; i < count; i += 256) band[i] = x[i];
+  }
+  __syncthreads();
+  const int nrows = p.oh - oy0 < b.rows ? p.oh - oy0 : b.rows;
+  float *y = p.Y + ((long long)blockIdx.x * p.oh + oy0) * p.ow;
+  // threads: 2^tx_log2 along ow, the rest along the band's rows
+  const int tx_n = 1 << b.tx_log2;
+  for (int r = threadIdx.x >> b.tx_log2; r < nrows; r += 256 >> b.tx_log2) {
+    const int iyb = (oy0 + r) * p.sh - p.pt;
+    for (int ox = threadIdx.x & (tx_n - 1); ox < p.ow; ox += tx_n) {
+      const int ixb = ox * p.sw - p.pl;
+      float mv = -INFINITY;
+      auto tap = [&](int ky, int kx) {
+        const int iy = iyb + ky * p.dh, ix = ixb + kx * p.dw;
+        // rows outside [lo, hi) and columns outside [0, w) are padding
+        const bool ok = iy >= lo && iy < hi && (unsigned)ix < (unsigned)p.w;
+        const float t = band[ok ? (iy - lo) * p.w + ix : 0];
+        if (ok && t > mv) mv = t;                   // strict, NaN never selected: maxpool.ts:98-101
+      };
+      if constexpr (KH > 0) {
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+          for (int kx = 0; kx < KW; kx++) tap(ky, kx);
+      } else {
+        for (int ky = 0; ky < p.kh; ky++)
+          for (int kx = 0; kx < p.kw; kx++) tap(ky, kx);
+      }
+      y[r * p.ow + ox] = mv;
+    }
+  }
+}
+
 // ---- transpose -----------------------------------------------------------------
 // Strided copy (Slice, Concat, Split): both sides addressed through strides.
 struct StridedCopyParams {
@@ -245,8 +303,8 @@ int launch_strided_copy(const StridedCopyParams &g) {
       for (int d = nd; d > 0; d--) { s.sx[d] = g.sx[d - 1]; s.sy[d] = g.sy[d - 1]; }
       s.sx[0] = s.sy[0] = 0;
     }
-    if (vec) hipLaunchKernelGGL(copy_plane<4>, dim3(w.blocks), dim3(256), 0, st, s, w);
-    else hipLaunchKernelGGL(copy_plane<1>, dim3(w.blocks), dim3(256), 0, st, s, w);
+    if (vec) hipLaunchKernelGGL(copy_plane<4>, wdh::plane_grid(w), dim3(256), 0, st, s, w);
+    else hipLaunchKernelGGL(copy_plane<1>, wdh::plane_grid(w), dim3(256), 0, st, s, w);
   } else if (g.total <= 0xffffffffLL) {
     hipLaunchKernelGGL(strided_copy_kernel<unsigned>, dim3(grid_for(g.total)), dim3(256), 0, st, g);
   } else {
@@ -281,9 +339,37 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
   p.X = (const float *)px; p.Y = (float *)py;
   p.h = h; p.w = w; p.oh = oh; p.ow = ow; p.kh = kh; p.kw = kw;
   p.pt = pt; p.pl = pl; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
+  hipStream_t st = wdh::stream();
+  // band variant: enough rows for two cells per thread, the span within 32 KB of LDS
+  {
+    PoolBand b;
+    b.tx_log2 = 0;
+    while (b.tx_log2 < 6 && (1 << b.tx_log2) < ow) b.tx_log2++;
+    const int rows_per_pass = 256 >> b.tx_log2;
+    b.rows = ((512 + ow - 1) / ow + rows_per_pass - 1) / rows_per_pass * rows_per_pass;
+    if (b.rows > oh) b.rows = oh;
+    const long long in_rows = (long long)(b.rows - 1) * sh + (long long)(kh - 1) * dh + 1;
+    const long long bands = (oh + b.rows - 1) / b.rows;
+    if (cells >= 256 && in_rows * w <= 8192 && bands <= 65535) {
+      b.in_rows = (int)in_rows;
+      const bool vec = w % 4 == 0 && ((long long)h * w) % 4 == 0 && ((uintptr_t)px & 15) == 0;
+      const dim3 grid((unsigned)planes, (unsigned)bands);
+      const size_t lds = (size_t)in_rows * w * 4;
+#define WDH_POOL_BAND(KH, KW)                                                                     \
+  do {                                                                                            \
+    if (vec) hipLaunchKernelGGL((maxpool2d_band_kernel<KH, KW, true>), grid, dim3(256), lds, st, p, b); \
+    else hipLaunchKernelGGL((maxpool2d_band_kernel<KH, KW, false>), grid, dim3(256), lds, st, p, b);    \
+  } while (0)
+      if (kh == 3 && kw == 3) WDH_POOL_BAND(3, 3);
+      else if (kh == 2 && kw == 2) WDH_POOL_BAND(2, 2);
+      else WDH_POOL_BAND(0, 0);
+#undef WDH_POOL_BAND
+      WDH_LAUNCH_CHECK();
+      return WDH_OK;
+    }
+  }
   const unsigned threads = cells <= 64 ? 64 : cells <= 128 ? 128 : 256;
   const dim3 grid((unsigned)planes, (unsigned)((cells + threads - 1) / threads)), block(threads);
-  hipStream_t st = wdh::stream();
   if (kh == 3 && kw == 3) hipLaunchKernelGGL((maxpool2d_kernel<3, 3>), grid, block, 0, st, p);
   else if (kh == 2 && kw == 2) hipLaunchKernelGGL((maxpool2d_kernel<2, 2>), grid, block, 0, st, p);
   else hipLaunchKernelGGL((maxpool2d_kernel<0, 0>), grid, block, 0, st, p);
