@@ -49,6 +49,24 @@ def test_every_config_graph_on_the_hip_host_path(tmp_path):
             assert rep["liveBuffers"] == rep["initializerCopies"], rep
 
 
+def test_operator_instances_are_reused_across_runs(tmp_path):
+    """The first run creates one instance per node; the second may create some again (weights that were
+    on the cpu now have device copies, so the inputs' placement differs); from the third on, none."""
+    data, _ = modelgen.resnet50_model(batch=1, image=32, classes=7, width=4, blocks=(1, 1, 1, 1))
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(0).standard_normal((1, 3, 32, 32)).astype(np.float32)
+    created = []
+    outs = []
+    for runs in (1, 2, 3, 4):
+        out, rep = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=runs)
+        created.append(rep["stats"]["operatorsCreated"])
+        outs.append(out[0])
+        nodes = rep["stats"]["nodes"]
+    assert created[0] == nodes and created[1] <= nodes and created[2] == 0 and created[3] == 0
+    for o in outs[1:]:
+        assert_bit_exact(o, outs[0], "same result whichever run is reported")
+
+
 def test_fusion_rewrites_the_expected_chains(tmp_path):
     data, _ = modelgen.resnet50_model(batch=1, image=32, classes=7, width=4, blocks=(2, 1, 1, 1))
     feeds = {"input": np.random.default_rng(1).standard_normal((1, 3, 32, 32)).astype(np.float32)}

@@ -44,6 +44,10 @@ class RunnerImpl {
     this.graphState = null;
     this.graphWarm = false;
     this.graphUnsupported = null; // reason, once a capture has failed for this model
+    // Operator instances by node and by where its inputs live.  The reference builds
+    // and initializes a new instance per node per run (runnerImpl.ts:441-452);
+    // instances here keep no state beyond their attributes, so later runs reuse them.
+    this.operatorCache = new Map();
   }
 
   async loadModel(directory, onnxBasename) {
@@ -57,6 +61,7 @@ class RunnerImpl {
   // `bytes`: the serialized ModelProto; `directory`: where external weight files live
   loadModelFromBytes(bytes, directory) {
     this.model = decodeModel(new Uint8Array(bytes.buffer, bytes.byteOffset, bytes.byteLength));
+    this.operatorCache.clear();
     modelTransform(this.model, this.backendOrder, { fuse: this.options.fuse });
     if (this.model.opsetImport.length !== 1) {
       logger.warn("Specifying multiple opset_import is not supported. Using first one.");
@@ -255,7 +260,7 @@ class RunnerImpl {
     const runStart = process.hrtime.bigint();
     const tensorReleaseTiming = findTensorReleaseTiming(this.model, new Set(this.initializerTensors.keys()));
     const nodePerformances = [];
-    const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length };
+    const stats = { nodesByBackend: {}, retriedOnCpu: [], nodes: graph.node.length, operatorsCreated: 0 };
     const strict = !!this.options.strict || !!opts.capture;
     const hip = this.backendContexts.hip;
     const useEvents = !opts.capture && !!opts.measurePerformance && hip && hip.initialized && graph.node.length + 1 <= 4096;
@@ -287,11 +292,17 @@ class RunnerImpl {
               }
               currentTensorsBackends.push(bs);
             }
-            const operator = instantiateOperator(opType, this.opset, backendOrderForNode, currentTensorsBackends);
+            const cacheKey = `${i}:${backendOrderForNode.join()}:${currentTensorsBackends.map((b) => b.join("+")).join("|")}`;
+            let operator = this.operatorCache.get(cacheKey);
             if (!operator) {
-              throw new Error(`Operator implementation for ${opType}, opset=${this.opset} does not exist.`);
+              operator = instantiateOperator(opType, this.opset, backendOrderForNode, currentTensorsBackends);
+              if (!operator) {
+                throw new Error(`Operator implementation for ${opType}, opset=${this.opset} does not exist.`);
+              }
+              operator.initialize(nonnull(node.attribute));
+              this.operatorCache.set(cacheKey, operator);
+              stats.operatorsCreated++;
             }
-            operator.initialize(nonnull(node.attribute));
             const requirement = operator.getTensorBackendRequirement(node.input.length, node.output.length);
             const operatorInputs = [];
             for (let j = 0; j < node.input.length; j++) {
