@@ -190,6 +190,12 @@ CONV_SHAPES = [
     (2, 16, 9, 9, 16, 3, [1, 1, 1, 1], [1, 1], [1, 1], 16),       # depthwise
     (1, 5, 6, 7, 3, 2, [0, 0, 0, 0], [1, 1], [1, 1], 1),          # even kernel, no pad
     (1, 2048, 25, 34, 256, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),   # DETR input projection
+    # 1x1 stride 1 with whole tiles: X is read in place as the B matrix
+    (16, 32, 14, 14, 80, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),     # 64-pixel tiles straddle images (196 each)
+    (4, 64, 8, 8, 48, 1, [0, 0, 0, 0], [1, 1], [1, 1], 2),        # groups
+    (16, 1024, 14, 14, 256, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),  # deep K: tiles cut along K, reduce pass
+    (2, 256, 56, 56, 64, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),
+    (2, 48, 12, 12, 24, 1, [0, 0, 0, 0], [1, 1], [1, 1], 1),      # 288 pixels: not whole tiles, gathers instead
 ]
 
 
@@ -220,6 +226,14 @@ def test_conv_1x1_equals_gemm(ctx):
     for b in range(2):
         g = hip_gemm(ctx, W.reshape(24, 40), X[b].reshape(40, 30))
         assert_close_max(got[b].reshape(24, 30), g, 1e-6, "1x1 == gemm")
+    # whole tiles (256 pixels, 32 channels): the in-place path, with residual and Relu fused
+    X, W, R = uni(4, 32, 8, 8), uni(24, 32, 1, 1), nrm(4, 24, 8, 8)
+    got = hip_conv(ctx, X, W)
+    for b in range(4):
+        g = hip_gemm(ctx, W.reshape(24, 32), X[b].reshape(32, 64))
+        assert_close_max(got[b].reshape(24, 64), g, 1e-6, "1x1 == gemm, in place")
+    fused = hip_conv(ctx, X, W, epilogue="relu", R=R)
+    assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "1x1 conv + residual + relu")
 
 
 # ------------------------------------------------------------------ elementwise

@@ -91,7 +91,11 @@ constexpr int MC_PAD = 8;    // MC tile row stride = extent + 8 (floats)
 
 // B_IM2COL32 / B_IM2COL64: at most 31 / 63 taps and X below 2 GiB, read through
 // a buffer descriptor; B_IM2COL_BIG: anything else, read with flat loads.
-enum BMode { B_KC = 0, B_MC = 1, B_IM2COL32 = 2, B_IM2COL64 = 3, B_IM2COL_BIG = 4 };
+// B_PIXELS: a 1x1, stride-1, unpadded conv.  Its B matrix is X itself, k rows of
+// h*w contiguous pixels per image, so it is fetched like B_MC (16-byte pieces)
+// with the image jump folded into each thread's column offset; the host picks it
+// only when every tile and K slab is whole (n % BN == 0, k % BK == 0, h*w % 4 == 0).
+enum BMode { B_KC = 0, B_MC = 1, B_IM2COL32 = 2, B_IM2COL64 = 3, B_IM2COL_BIG = 4, B_PIXELS = 5 };
 
 struct ConvGeom {
   int c_in_g;        // input channels per group
@@ -396,6 +400,8 @@ template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE_, bool VEC>
 __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kernel(Params p) {
   constexpr bool IM2COL_FAST = BMODE_ == B_IM2COL32 || BMODE_ == B_IM2COL64;
   constexpr bool IM2COL = IM2COL_FAST || BMODE_ == B_IM2COL_BIG;
+  constexpr bool PIXELS = BMODE_ == B_PIXELS;
+  constexpr bool CONV = IM2COL || PIXELS;  // Y is NCHW, the bias is per row
   constexpr bool B_IS_KC = BMODE_ == B_KC;
   static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
   constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
@@ -446,7 +452,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   // clamped, their products are never stored); an operand that is contiguous
   // along M or N takes it on tiles that lie fully inside the matrix.
   const bool a_fast = p.fast && (A_KC || (VEC && row0 + BM <= p.m));
-  const bool b_fast = p.fast && (B_IS_KC || IM2COL_FAST || (VEC && col0 + BN <= p.n));
+  const bool b_fast = p.fast && (B_IS_KC || IM2COL_FAST || PIXELS || (VEC && col0 + BN <= p.n));
   int voff_a[BM / 64], voff_b[BN / 64];
   if (A_KC) {
 #pragma unroll
@@ -470,9 +476,16 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     }
   } else if (!IM2COL) {
     constexpr int TPR = BN / 4, RPP = NTHREADS / TPR;
+    // B_PIXELS: column = pixel index over the batch; its four pixels share an image
+    long long colpos = col0 + (tid % TPR) * 4;
+    if (PIXELS) {
+      const unsigned plane = (unsigned)(p.cv.h * p.cv.w);
+      const unsigned img = (unsigned)colpos / plane;
+      colpos = (long long)img * p.cv.c_total * plane + ((unsigned)colpos - img * plane);
+    }
 #pragma unroll
     for (int i = 0; i < BN / 64; i++)
-      voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + col0 + (tid % TPR) * 4) * 4);
+      voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + colpos) * 4);
   }
   const rsrc_t rsrc_a = make_rsrc(A, p.a_bytes);
 
@@ -516,7 +529,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   }
   // conv: p.b_bytes is group 0's window, later groups start further into X
   const int b_window =
-      IM2COL ? p.b_bytes - (int)((long long)bz * p.cv.c_in_g * p.cv.h * p.cv.w * 4) : p.b_bytes;
+      CONV ? p.b_bytes - (int)((long long)bz * p.cv.c_in_g * p.cv.h * p.cv.w * 4) : p.b_bytes;
   const rsrc_t rsrc_b = make_rsrc(bbase, b_window);
   // first of the L consecutive k rows this wavefront gathers in each slab
   const int kgroup0 = IM2COL ? __builtin_amdgcn_readfirstlane(tid / BN) * (BK / (NTHREADS / BN)) : 0;
@@ -558,7 +571,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
       fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(rsrc_b, p.cv.ktab, pf, k0 + kgroup0, st.b);
     } else if (IM2COL) {
       st.ok = fetch_im2col<BN>(p.cv, px, k0, kend, tid, st.b);
-    } else if (b_fast && full) {
+    } else if ((b_fast && full) || PIXELS) {
       fetch_rows_fast<BN, VEC>(rsrc_b, voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * ldb * 4), st.b);
     } else if (B_IS_KC) {
       fetch_kc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
@@ -685,7 +698,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     const int colc = col_ok ? col : p.n - 1;
     long long ybase;     // offset of (row 0, this column) in Y
     long long ystride;   // distance between consecutive rows in Y
-    if (IM2COL) {
+    if (CONV) {
       const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
       const unsigned img = (unsigned)colc / ohw;
       const unsigned q = (unsigned)colc - img * ohw;
@@ -707,7 +720,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
           for (int j = 0; j < 8; j++) {
             int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
             row = row < p.m ? row : p.m - 1;
-            cv[j] = IM2COL ? p.C[bz * p.cv.cout_g + row]
+            cv[j] = CONV ? p.C[bz * p.cv.cout_g + row]
                            : p.C[(long long)row * p.sC0 + (long long)colc * p.sC1];
           }
         }
@@ -1143,6 +1156,26 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   const long long x_bytes = ((long long)n * c * h * w + (long long)pt * w + pl) * 4;
   const long long w_bytes = (long long)cout_g * kdim * 4;
   const bool small = x_bytes < 0x7fffffffLL && w_bytes < 0x7fffffffLL;
+  const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
+  // 1x1, stride 1, no padding: X is the B matrix as it lies (B_PIXELS), provided every tile
+  // and K slab is whole; a forced tile may be up to 256 columns wide
+  const long long plane = (long long)h * w;
+  if (small && vec && ntaps == 1 && sh == 1 && sw == 1 && pt == 0 && pl == 0 && pb == 0 && pr == 0 &&
+      plane % 4 == 0 && kdim % BK == 0 && aligned16(p.B) &&
+      npix % (g_forced_tile >= 0 ? 256 : 64) == 0) {
+    p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
+    p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
+    p.sBb = (long long)c_in_g * plane; p.sB0 = plane; p.sB1 = 1;
+    p.alpha = 1.0f; p.beta = 1.0f; p.epilogue = epilogue;
+    p.cv.c_in_g = c_in_g; p.cv.h = h; p.cv.w = w; p.cv.oh = oh; p.cv.ow = ow;
+    p.cv.sh = p.cv.sw = p.cv.kh = p.cv.kw = p.cv.dh = p.cv.dw = 1;
+    p.cv.c_total = c; p.cv.cout_total = cout; p.cv.cout_g = cout_g;
+    p.cv.ntaps = 1; p.cv.npix = npix;
+    p.fast = 1;
+    p.a_bytes = (int)w_bytes;
+    p.b_bytes = (int)x_bytes;  // window of group 0; the kernel shortens it per group
+    return launch<true, B_PIXELS>(p, group, true);
+  }
   const int mode = !small || ntaps > 63 ? B_IM2COL_BIG : (ntaps > 31 ? B_IM2COL64 : B_IM2COL32);
   KtabKey key;
   memset(&key, 0, sizeof(key));
@@ -1194,7 +1227,6 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.ntaps = ntaps;
   p.cv.npix = npix; p.cv.ktab = it->second.ktab;
   p.cv.kh = kh; p.cv.kw = kw; p.cv.dh = dh; p.cv.dw = dw;
-  const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
   p.fast = small ? 1 : 0;
   p.a_bytes = small ? (int)w_bytes : 0;
   // a group's window runs from its first byte (shifted down by the padding) to the end of X

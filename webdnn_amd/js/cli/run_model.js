@@ -4,7 +4,7 @@
 //
 //   node run_model.js --model DIR [--onnx model.onnx | --optimized] [--backend hip|cpu]
 //        --inputs a.bin[,b.bin...] --output out.bin
-//        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure]
+//        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
 //        [--graph] [--alt-inputs a2.bin[,b2.bin...]]
 //
@@ -47,6 +47,8 @@ function parseArgs(argv) {
     else if (a === "--no-fuse") args.noFuse = true;
     else if (a === "--warmup") args.warmup = parseInt(next(), 10);
     else if (a === "--runs") args.runs = parseInt(next(), 10);
+    else if (a === "--queue-ahead") args.queueAhead = parseFloat(next());
+    else if (a === "--measure-all") args.measureAll = true;
     else if (a === "--measure") args.measure = true;
     else if (a === "--cpu-entries") args.cpuEntries = next();
     else if (a === "--tile") args.tile = parseInt(next(), 10);
@@ -105,11 +107,34 @@ async function main() {
   for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, { graph: !!args.graph });
   const times = [];
   let outputs = null;
+  let queueAhead = null;
+  const deviceTimes = [];
   for (let i = 0; i < args.runs; i++) {
+    // --queue-ahead MS (with --measure): put about MS milliseconds of streaming kernels on the
+    // device queue first, so that the measured run's launches are all queued before the device
+    // reaches them.  Its kernels then run back to back and the per-node events time the device
+    // alone, not the host's enqueue rate.
+    if (args.queueAhead && args.measure && i === args.runs - 1 && runner.backendName === "hip") {
+      const hip = runner.backendContexts.hip;
+      const n = 128 * 1024 * 1024; // floats: 0.5 GiB in, 0.5 GiB out per launch
+      const a = hip.emptyTensor([n], "float32"), b = hip.emptyTensor([n], "float32");
+      hip.native.unary(0, 0, a.handle, b.handle, n); // touch both buffers once
+      hip.sync();
+      const reps = Math.max(1, Math.ceil(args.queueAhead / 0.2));
+      hip.native.eventRecord(4094);
+      for (let r = 0; r < reps; r++) hip.native.unary(0, 0, a.handle, b.handle, n);
+      hip.native.eventRecord(4095);
+      queueAhead = { launches: reps, tensors: [a, b] };
+    }
     const t0 = process.hrtime.bigint();
     outputs = await runner.run(altInputs && i % 2 === 1 ? altInputs : runInputs,
-      { measurePerformance: !!args.measure && i === args.runs - 1, graph: !!args.graph });
+      { measurePerformance: !!args.measureAll || (!!args.measure && i === args.runs - 1), graph: !!args.graph });
     times.push(Number(process.hrtime.bigint() - t0) / 1e6);
+    // --measure-all: device time of every timed run (HIP events on the library's stream; a replayed
+    // graph is bracketed by one pair, an eager run has one event per node boundary)
+    if (args.measureAll && runner.lastPerformance) {
+      deviceTimes.push(runner.lastPerformance.reduce((acc, p) => acc + (p.deviceElapsed || 0), 0));
+    }
   }
   if (args.output) {
     const fd = fs.openSync(args.output, "w");
@@ -123,12 +148,18 @@ async function main() {
     backend: runner.backendName,
     outputs: outputs.map((t, i) => ({ name: runner.getOutputNames()[i], dims: t.dims, dataType: t.dataType })),
     msPerRun: times,
+    deviceMsPerRun: args.measureAll ? deviceTimes : undefined,
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
     node: process.version,
     graph: args.graph ? { captured: !!runner.graphState, unsupported: runner.graphUnsupported } : undefined,
   };
   runner.disposeGraph();
+  if (queueAhead) {
+    // the queued work must have outlasted the host's enqueue of the measured run
+    report.queueAhead = { launches: queueAhead.launches, deviceMs: runner.backendContexts.hip.native.eventElapsedMs(4094, 4095) };
+    for (const t of queueAhead.tensors) t.dispose();
+  }
   if (args.measure && runner.lastPerformance) {
     report.performance = runner.lastPerformance.map((p) => ({
       name: p.name, opType: p.opType, backend: p.backend, outputDims: p.outputDims,
