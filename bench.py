@@ -277,6 +277,7 @@ def main():
         report_only = bench_report_only(workdir, max(3, args.steps // 2), min(args.warmup, 3))
         baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
     kernels = bench_kernels(args.steps, args.warmup)
+    bandwidth = bench_bandwidth(args.steps, args.warmup)
 
     # The timed steps are graph replays: one HIP event pair brackets each replay on the library's
     # stream.  That device time covers the 54 contraction launches with their reduce passes plus the
@@ -325,6 +326,8 @@ def main():
             "conv_c3": kernels["conv_c3"],
             "ffn_c2": report_only["ffn_c2"],
             "detr_r50_b1": report_only["detr_r50_b1"],
+            "bandwidth_kernels": {"unit": "GB/s of algorithmic bytes (HIP events around back-to-back launches)",
+                                  "peak": 8000.0, "kernels": bandwidth},
             "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
             "resnet50_ms_per_step_eager": round(resnet["ms_per_step_eager"], 4),
             "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),

@@ -448,11 +448,14 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   const int kend = whole ? p.k : (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k);
 
   // ---- descriptor fetch plans: one byte offset per 16-byte piece -------------
-  // A row-major-in-K operand may always take this path (rows past the edge are
-  // clamped, their products are never stored); an operand that is contiguous
-  // along M or N takes it on tiles that lie fully inside the matrix.
-  const bool a_fast = p.fast && (A_KC || (VEC && row0 + BM <= p.m));
-  const bool b_fast = p.fast && (B_IS_KC || IM2COL_FAST || PIXELS || (VEC && col0 + BN <= p.n));
+  // Every operand below 2 GiB takes this path, edge tiles included.  Rows of a
+  // row-major-in-K operand past the edge are clamped; an operand that is
+  // contiguous along M or N simply reads on past its last row or column, into
+  // the next k row (or, past the end of the matrix, zeros from the descriptor's
+  // bounds check).  Either way the surplus rows and columns only feed products
+  // that are never stored.
+  const bool a_fast = p.fast;
+  const bool b_fast = p.fast && BMODE_ != B_IM2COL_BIG;
   int voff_a[BM / 64], voff_b[BN / 64];
   if (A_KC) {
 #pragma unroll
@@ -830,7 +833,7 @@ struct WorkPlan {
 // sooner than `solo` times the longest single workgroup (the slow-down of a
 // workgroup that runs alone on a CU); every workgroup adds a start-up/epilogue
 // cost and a split adds the reduce pass over the partial sums.
-WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
+WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather) {
   const long long cus = wdh::compute_units();
   const int slabs = (k + BK - 1) / BK;
   WorkPlan w = {tiles, 0, 1, 0};
@@ -852,8 +855,11 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
   const double area = (double)bm * bn / (64.0 * 64.0);
   const double slab_us = 0.30 * area;
   const double start_us = 0.9 * (area > 1.0 ? 2.0 : 1.0);
-  const double solo = 2.5;
   const double tile_bytes = (double)bm * bn * 4.0;
+  // A launch cannot finish sooner than its longest workgroup, and with the CU mostly to
+  // itself a workgroup is bound by the latency of its loads, slab after slab: about 2.5
+  // times its nominal time (measured inside whole graphs, where operands arrive cold).
+  auto floor_us = [](double longest) { return 2.5 * longest; };
   auto cost = [&](long long tail, int s) {
     const long long full_rounds = (tiles - tail) / cus;  // tiles - tail is a multiple of cus or 0
     const long long tail_rounds = (tail * s + cus - 1) / cus;
@@ -861,10 +867,11 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
     const double whole_us = slabs * slab_us + start_us;
     const double work = full_rounds * whole_us + tail_rounds * chunk_us;
     const double longest = full_rounds > 0 ? whole_us : chunk_us;
-    double t = work > solo * longest ? work : solo * longest;
-    // reduce pass: a launch plus the partial sums written and read back (mostly
-    // through the last-level cache, ~8 TB/s)
-    if (s > 1) t += 6.0 + 2.0 * tail * s * tile_bytes / 8.0e6;
+    double t = work > floor_us(longest) ? work : floor_us(longest);
+    // reduce pass: a launch, a serial walk over the s partial sums of each element (what
+    // the deep splits of small Gemms feel; convs split at most ~8 ways), and the partial
+    // sums written and read back (mostly through the last-level cache, ~8 TB/s)
+    if (s > 1) t += (gather ? 6.0 : 4.0 + 0.26 * s) + 2.0 * tail * s * tile_bytes / 8.0e6;
     return t;
   };
   const long long rem = tiles % cus;
@@ -875,7 +882,7 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn) {
     const long long rounds = (tiles + cus - 1) / cus;
     const double whole_us = slabs * slab_us + start_us;
     const double work = rounds * whole_us;
-    best = work > solo * whole_us ? work : solo * whole_us;
+    best = work > floor_us(whole_us) ? work : floor_us(whole_us);
   }
   long long best_tail = 0;
   int best_s = 1;
@@ -895,7 +902,7 @@ int launch_tile(Params &p, int nz, bool vec) {
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   const long long tiles = (long long)p.tiles_m * p.tiles_n * nz;
-  const WorkPlan w = plan_work(tiles, p.k, BM, BN);
+  const WorkPlan w = plan_work(tiles, p.k, BM, BN, BMODE >= B_IM2COL32);
   const long long blocks = w.full + w.tail * w.split;
   if (blocks > 0x7fffffffLL)
     return wdh::fail(WDH_EINVAL, "contraction: %lld workgroups exceed the grid limit", blocks);
@@ -1060,7 +1067,8 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   // clamped edge row plus a 16-byte piece may reach 12 bytes past the span).
   const long long a_bytes = k ? span(1, 0, m, p.sA0, k, p.sA1) * 4 : 0;
   const long long b_bytes = k ? span(1, 0, k, p.sB0, n, p.sB1) * 4 : 0;
-  p.fast = a_bytes < 0x7fffffffLL && b_bytes < 0x7fffffffLL;
+  // (the margin covers the columns an edge tile reads past the matrix)
+  p.fast = a_bytes < 0x7fffffffLL - 4096 && b_bytes < 0x7fffffffLL - 4096;
   p.a_bytes = p.fast ? (int)a_bytes : 0;
   p.b_bytes = p.fast ? (int)b_bytes : 0;
   if (useA_kc && useB_kc) return launch<true, B_KC>(p, batch, vec);
