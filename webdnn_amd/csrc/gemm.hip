@@ -83,6 +83,9 @@ __device__ __forceinline__ float buf_load(rsrc_t r, int voff, int soff) {
 __device__ __forceinline__ f32x4 buf_load4(rsrc_t r, int voff, int soff) {
   return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
+__device__ __forceinline__ void buf_store(rsrc_t r, float v, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+}
 
 constexpr int BK = 16;
 constexpr int NTHREADS = 256;
@@ -145,6 +148,8 @@ struct Params {
   int fast;         // every operand spans less than 2 GiB: descriptor loads allowed
   int a_bytes;      // fast: bytes of one z of A / of B (conv: of X from the first byte
   int b_bytes;      //       of a group to the end of the tensor, plus the padding shift)
+  int y_bytes;      // > 0: bytes of one z of Y (conv: of all of Y), below 2 GiB, and C spans
+  int c_bytes;      //      c_bytes (< 2 GiB): whole tiles may use the descriptor epilogue
   ConvGeom cv;
 };
 
@@ -690,10 +695,67 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
         }
     return;  // splitk_reduce_kernel adds the chunks up
   }
-  // Bias and residual values of a 32x32 block are all requested before the
-  // first is used, so the block pays one memory round trip, not thirty-two.
-  // Loads use clamped indices (always inside the tensors); only the store is
-  // conditional.
+  // Whole tiles of results below 2 GiB: every address is one per-lane byte
+  // offset (column, plus the four rows by which the two halves of a wavefront
+  // differ) and one scalar offset per accumulator row, so a stored element costs
+  // no address arithmetic, no bounds test and no change of the execution mask.
+  if (p.y_bytes > 0 && row0 + BM <= p.m && col0 + BN <= p.n) {
+    const long long zoff = CONV ? 0 : (long long)bz * p.m * p.n;
+    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, p.y_bytes);
+    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, p.y_bytes);
+    const rsrc_t rsrc_c = make_rsrc(p.C ? p.C : p.Y, p.C ? p.c_bytes : 0);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = col0 + wcol + nt * 32 + li;
+      int ybase, ystride, voff_c, cstride;  // in elements; byte offsets stay below 2^31
+      if (CONV) {
+        const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+        const unsigned img = (unsigned)col / ohw;
+        ybase = (int)((img * (unsigned)p.cv.cout_total + (unsigned)(bz * p.cv.cout_g)) * ohw +
+                      ((unsigned)col - img * ohw));
+        ystride = (int)ohw;
+        voff_c = (bz * p.cv.cout_g + 4 * half) * 4;
+        cstride = 1;
+      } else {
+        ybase = col;
+        ystride = p.n;
+        voff_c = (int)((4 * half * p.sC0 + col * p.sC1) * 4);
+        cstride = (int)p.sC0;
+      }
+      const int voff_y = (ybase + 4 * half * ystride) * 4;
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int rbase = __builtin_amdgcn_readfirstlane(row0 + wrow + mt * 32);
+#pragma unroll
+        for (int hb = 0; hb < 2; hb++) {
+          float cv[8], rv[8];
+          if (p.C) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              cv[j] = buf_load(rsrc_c, voff_c, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * cstride * 4);
+          }
+          if (p.R) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              rv[j] = buf_load(rsrc_r, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
+          }
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            float y = p.alpha * acc[mt][nt][8 * hb + j];
+            if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+            if (p.R) y = y + rv[j];
+            if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+            buf_store(rsrc_y, y, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
+          }
+        }
+      }
+    }
+    return;
+  }
+  // Edge tiles and larger results.  Bias and residual values of a 32x32 block
+  // are all requested before the first is used, so the block pays one memory
+  // round trip, not thirty-two.  Loads use clamped indices (always inside the
+  // tensors); only the store is conditional.
 #pragma unroll
   for (int nt = 0; nt < NT; nt++) {
     const int col = col0 + wcol + nt * 32 + li;
@@ -1071,6 +1133,13 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   p.fast = a_bytes < 0x7fffffffLL - 4096 && b_bytes < 0x7fffffffLL - 4096;
   p.a_bytes = p.fast ? (int)a_bytes : 0;
   p.b_bytes = p.fast ? (int)b_bytes : 0;
+  {
+    const long long y_bytes = (long long)m * n * 4;
+    const long long c_bytes = p.C ? span(1, 0, m, p.sC0, n, p.sC1) * 4 : 0;
+    const bool ok = y_bytes < 0x7fffffffLL && c_bytes < 0x7fffffffLL;
+    p.y_bytes = ok ? (int)y_bytes : 0;
+    p.c_bytes = ok ? (int)c_bytes : 0;
+  }
   if (useA_kc && useB_kc) return launch<true, B_KC>(p, batch, vec);
   if (useA_kc && !useB_kc) return launch<true, B_MC>(p, batch, vec);
   if (!useA_kc && useB_kc) return launch<false, B_KC>(p, batch, vec);
@@ -1182,6 +1251,8 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.fast = 1;
     p.a_bytes = (int)w_bytes;
     p.b_bytes = (int)x_bytes;  // window of group 0; the kernel shortens it per group
+    p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+    p.c_bytes = cout * 4;
     return launch<true, B_PIXELS>(p, group, true);
   }
   const int mode = !small || ntaps > 63 ? B_IM2COL_BIG : (ntaps > 31 ? B_IM2COL64 : B_IM2COL32);
@@ -1239,6 +1310,8 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.a_bytes = small ? (int)w_bytes : 0;
   // a group's window runs from its first byte (shifted down by the padding) to the end of X
   p.b_bytes = small ? (int)x_bytes : 0;  // window of group 0; the kernel shortens it per group
+  p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+  p.c_bytes = cout * 4;
   if (mode == B_IM2COL32) return launch<true, B_IM2COL32>(p, group, vec);
   if (mode == B_IM2COL64) return launch<true, B_IM2COL64>(p, group, vec);
   return launch<true, B_IM2COL_BIG>(p, group, vec);
