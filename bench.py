@@ -43,7 +43,7 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 # HBM-side bytes per contraction-kernel launch of the ResNet-50 step, averaged over its 54 launches:
 # rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB device copy;
 # recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read counters itself).
-TRAFFIC_BYTES_PER_LAUNCH = 78.5e6
+TRAFFIC_BYTES_PER_LAUNCH = 78.6e6
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 
