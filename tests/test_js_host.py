@@ -233,6 +233,21 @@ def test_graph_replay_on_the_host_path(tmp_path):
     assert rep["liveBuffers"] == rep["initializerCopies"]          # the graph's buffers are gone after disposeGraph
 
 
+def test_cli_reports_device_time_of_every_run(tmp_path):
+    """--measure-all: one device time per timed run, eager (an event per node boundary) and replayed
+    (one event pair around the graph launch)."""
+    data, _ = modelgen.resnet50_model(batch=1, image=32, width=4, blocks=(1, 1, 1, 1), classes=5)
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(4).standard_normal((1, 3, 32, 32)).astype(np.float32)
+    _, eager = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=3, extra=["--measure-all"])
+    assert len(eager["deviceMsPerRun"]) == 3 and "performance" not in eager
+    _, replay = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=4, warmup=2,
+                                      extra=["--graph", "--measure-all"])
+    assert replay["graph"]["captured"] and len(replay["deviceMsPerRun"]) == 4
+    _, plain = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=2)
+    assert "deviceMsPerRun" not in plain
+
+
 def test_graph_mode_falls_back_when_the_run_needs_device_data_on_the_host(tmp_path):
     """The glue graph computes a Reshape shape on the device; reading it back cannot be recorded."""
     data, _ = modelgen.glue_model(11)
