@@ -233,6 +233,48 @@ def test_graph_replay_on_the_host_path(tmp_path):
     assert rep["liveBuffers"] == rep["initializerCopies"]          # the graph's buffers are gone after disposeGraph
 
 
+def test_exporter_shaped_model_bytes_decode_and_run(tmp_path):
+    """A ModelProto laid out the way the PyTorch exporter writes one (the shape of the reference's
+    example/minimum/model/model.onnx: ir_version, producer name and version, then the graph with its
+    node before its name, value infos with TypeProto.Tensor shapes, opset_import last), assembled here
+    byte by byte from the field numbers of onnx.proto rather than by this package's own encoder.  The
+    decoder must skip the fields it has no use for and find the rest; the one Relu node then has to
+    reproduce the reference's own vector (test/unit/cpuOperator.test.ts:15-18) on both backends."""
+    def varint(v):
+        out = bytearray()
+        while True:
+            out.append((v & 0x7F) | (0x80 if v > 0x7F else 0))
+            v >>= 7
+            if not v:
+                return bytes(out)
+
+    def field(number, payload):            # wire type 2: length-delimited
+        return varint(number << 3 | 2) + varint(len(payload)) + payload
+
+    def scalar(number, value):             # wire type 0: varint
+        return varint(number << 3 | 0) + varint(value)
+
+    def value_info(name, dims):            # ValueInfoProto{name=1, type=2{tensor_type=1{elem_type=1, shape=2{dim=1{dim_value=1}}}}}
+        shape = b"".join(field(1, scalar(1, d)) for d in dims)
+        return field(1, name) + field(2, field(1, scalar(1, 1) + field(2, shape)))
+
+    node = field(1, b"in0") + field(2, b"out0") + field(3, b"Relu_0") + field(4, b"Relu")
+    graph = field(1, node) + field(2, b"exported-graph") + field(11, value_info(b"in0", [2, 3])) + \
+        field(12, value_info(b"out0", [2, 3]))
+    model = scalar(1, 6) + field(2, b"pytorch") + field(3, b"1.7") + field(7, graph) + field(8, scalar(2, 9))
+    assert len(model) == 112 and model[:2] == b"\x08\x06"      # ir_version = 6 comes first
+    (tmp_path / "model.onnx").write_bytes(model)
+    parsed = modelgen.parse_model(model)
+    assert parsed["opset"] == 9 and [n["op_type"] for n in parsed["nodes"]] == ["Relu"]
+    assert parsed["inputs"] == [("in0", [2, 3])] and parsed["outputs"] == [("out0", [2, 3])]
+    x = np.array([[-2, -0.5, 0], [1, 3, -0.0]], np.float32)
+    want = np.array([[0, 0, 0], [1, 3, 0]], np.float32)
+    for backend, kw in (("cpu", dict(oracle_cpu=True)), ("hip", dict(fake_native=True))):
+        out, rep = node_runner.run_model(str(tmp_path), [x], backend, **kw)
+        assert rep["outputs"][0]["name"] == "out0" and rep["outputs"][0]["dims"] == [2, 3]
+        assert_bit_exact(out[0], want, "Relu through %s" % backend)
+
+
 def test_cli_reports_device_time_of_every_run(tmp_path):
     """--measure-all: one device time per timed run, eager (an event per node boundary) and replayed
     (one event pair around the graph launch)."""
