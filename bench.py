@@ -254,8 +254,8 @@ def bench_bandwidth(steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["all", "kernels", "bandwidth"], default="all",
                     help="kernels: only the in-process Gemm 4096 / Conv C3 launches plus one device-to-device "
