@@ -292,7 +292,8 @@ def test_unary(ctx):
 
 # ------------------------------------------------------------------ row reductions
 @pytest.mark.parametrize("shape", [(8, 850, 850), (8, 100, 850), (8, 100, 100), (3, 4, 5, 6), (7, 1), (5, 64), (3, 129),
-                                   (4, 1025), (2, 2049), (3, 5000), (1, 1), (5, 256), (3, 1024), (2, 2048), (4, 852), (9, 132)])
+                                   (4, 1025), (2, 2049), (3, 5000), (1, 1), (5, 256), (3, 1024), (2, 2048), (4, 852), (9, 132),
+                                   (9001, 100), (8195, 260), (8193, 513), (8200, 1024)])   # more rows than resident wavefronts
 def test_softmax(ctx, shape):
     x = nrm(*shape, std=3.0)
     got = H.softmax(ctx, ctx.move_tensor(x)).get_data()
@@ -308,7 +309,8 @@ def test_softmax_edges(ctx):
 
 
 @pytest.mark.parametrize("shape", [(850, 1, 256), (100, 1, 256), (6, 2048), (3, 5000), (4, 7), (2, 3, 1), (9, 1000),
-                                   (5, 250), (7, 1024), (3, 132)])
+                                   (5, 250), (7, 1024), (3, 132),
+                                   (27200, 256), (8195, 250), (8193, 1000), (8194, 1028)])       # more rows than resident wavefronts
 def test_layernorm(ctx, shape):
     x, g, b = nrm(*shape, std=2.0), nrm(shape[-1]), nrm(shape[-1])
     got = H.layer_normalization(ctx, ctx.move_tensor(x), ctx.move_tensor(g), ctx.move_tensor(b)).get_data()
