@@ -87,6 +87,30 @@ __device__ __forceinline__ void buf_store(rsrc_t r, float v, int voff, int soff)
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
 
+// Division of a non-negative 32-bit integer by a divisor fixed for the launch: the
+// host turns the divisor into a multiplier and a shift, the kernel pays one
+// multiply-high and one shift instead of the ~40 instructions of a hardware-less
+// integer division.  Exact for 0 <= n < 2^31.
+struct FastDiv {
+  unsigned mul;    // 0: the divisor is 1
+  unsigned shift;
+  int d;
+};
+inline FastDiv make_fastdiv(long long divisor) {
+  FastDiv f = {0u, 0u, (int)divisor};
+  if (divisor <= 1) return f;
+  unsigned lg = 0;
+  while ((1ll << lg) < divisor) lg++;
+  const unsigned pw = 31 + lg;
+  f.mul = (unsigned)((((unsigned long long)1 << pw) + (unsigned long long)divisor - 1) /
+                     (unsigned long long)divisor);
+  f.shift = pw - 32;
+  return f;
+}
+__device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
+  return f.mul ? (int)(__umulhi((unsigned)n, f.mul) >> f.shift) : n;
+}
+
 constexpr int BK = 16;
 constexpr int NTHREADS = 256;
 constexpr int LDK = BK + 4;  // KC tile row stride (floats)
@@ -119,6 +143,13 @@ struct ConvGeom {
   // carry tap 31 (B_IM2COL32) or 63 (B_IM2COL64), which no pixel has.
   // B_IM2COL_BIG: x = the same offset in elements, y = (ky*dh)<<16 | kx*dw.
   const int2 *ktab;
+  // conv3x3_halo_kernel only: the input rows a tile needs are staged in LDS as
+  // rows of `pitch` floats, `slots` of them per channel, the first input column in
+  // LDS column col0; pb/pr = bottom / right padding
+  int pitch, slots, col0;
+  FastDiv fd_ow, fd_oh, fd_ohw;      // output width, height, plane
+  FastDiv fd_plane;                  // h*w
+  FastDiv fd_oh2, fd_upc, fd_pg;     // oh+2, pieces per channel, pieces per row (halo kernel)
 };
 
 struct Params {
@@ -134,6 +165,7 @@ struct Params {
   float alpha, beta;
   int epilogue;
   int tiles_m, tiles_n;
+  FastDiv fd_tiles_per_z, fd_tail_tiles, fd_group, fd_last_rows;  // see decode_work / tile_coords
   // Work decomposition.  Tiles are numbered tile + z * tiles_m * tiles_n (z =
   // batch entry or conv group).  The first full_tiles of them are computed by
   // one workgroup each; every remaining ("tail") tile is cut along K into
@@ -170,16 +202,45 @@ __device__ __forceinline__ int xcd_contiguous(int pid, int total) {
 
 // Tile number within one z -> tile coordinates, visiting tiles in groups of 8
 // tile-rows so that the panels a group touches stay resident in L2.
-__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n,
-                                            int *tm, int *tn) {
-  constexpr int GROUP = 8;
-  const int per_group = GROUP * tiles_n;
-  const int group = id / per_group;
-  const int first_m = group * GROUP;
-  const int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
-  const int in_group = id % per_group;
-  *tm = first_m + in_group % rows;
-  *tn = in_group / rows;
+constexpr int TILE_GROUP = 8;
+__device__ __forceinline__ void tile_coords(const Params &p, int id, int *tm, int *tn) {
+  const int per_group = TILE_GROUP * p.tiles_n;
+  const int group = fdiv(id, p.fd_group);
+  const int first_m = group * TILE_GROUP;
+  const int in_group = id - group * per_group;
+  if (p.tiles_m - first_m >= TILE_GROUP) {
+    *tn = in_group / TILE_GROUP;
+    *tm = first_m + in_group % TILE_GROUP;
+  } else {
+    // the last, shorter group
+    *tn = fdiv(in_group, p.fd_last_rows);
+    *tm = first_m + in_group - *tn * p.fd_last_rows.d;
+  }
+}
+
+// Which tile a workgroup computes and, for a chunk workgroup, which part of K.
+struct TileWork {
+  bool whole;
+  int lin, chunk, bz, tm, tn;
+};
+__device__ __forceinline__ TileWork decode_work(const Params &p) {
+  TileWork t;
+  const int pid = blockIdx.x;
+  t.whole = pid < p.full_tiles;
+  t.chunk = 0;
+  if (t.whole) {
+    t.lin = xcd_contiguous(pid, p.full_tiles);
+  } else {
+    // chunk workgroups: an XCD takes a contiguous run of (chunk, tile) pairs with the
+    // tile varying fastest, so that tiles which share a slice of B meet in one L2
+    const int v = xcd_contiguous(pid - p.full_tiles, p.tail_tiles * p.tail_split);
+    t.chunk = fdiv(v, p.fd_tail_tiles);
+    t.lin = p.full_tiles + (v - t.chunk * p.tail_tiles);
+  }
+  const int tiles_per_z = p.tiles_m * p.tiles_n;
+  t.bz = fdiv(t.lin, p.fd_tiles_per_z);  // batch entry (gemm) or group (conv)
+  tile_coords(p, t.lin - t.bz * tiles_per_z, &t.tm, &t.tn);
+  return t;
 }
 
 // ---- global -> register fetch of one K slab ------------------------------
@@ -347,13 +408,16 @@ __device__ __forceinline__ void stash_im2col(float *tile, int tid,
     tile[(kgroup * L + i) * LD + pix] = ((okbits >> i) & 1u) ? reg[i >> 2][i & 3] : 0.0f;
 }
 
+// The descriptor gather leaves a thread with L consecutive k of one pixel: they go
+// to LDS as they are, tile[pixel][k] (the KC layout), L/4 16-byte stores.
 template <int EXT>
 __device__ __forceinline__ void stash_im2col_fast(float *tile, int tid,
                                                   const f32x4 (&reg)[EXT / 64]) {
-  constexpr int G = NTHREADS / EXT, L = BK / G, LD = EXT + MC_PAD;
+  constexpr int G = NTHREADS / EXT, L = BK / G;
   const int kgroup = tid / EXT, pix = tid % EXT;
 #pragma unroll
-  for (int i = 0; i < L; i++) tile[(kgroup * L + i) * LD + pix] = reg[i >> 2][i & 3];
+  for (int i = 0; i < L / 4; i++)
+    *reinterpret_cast<f32x4 *>(tile + pix * LDK + kgroup * L + 4 * i) = reg[i];
 }
 
 constexpr int tile_floats(bool kc, int ext) { return kc ? ext * LDK : BK * (ext + MC_PAD); }
@@ -380,7 +444,7 @@ __device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int
     long long off;
     if (CONV) {
       const int ohw = p.cv.oh * p.cv.ow;
-      const int img = col / ohw, q = col - img * ohw;
+      const int img = fdiv(col, p.cv.fd_ohw), q = col - img * ohw;
       off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
       if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
     } else {
@@ -390,6 +454,154 @@ __device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int
     if (p.R) y = y + p.R[off];
     if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
     p.Y[off] = y;
+  }
+}
+
+// ---- epilogue shared by the contraction kernels ----------------------------------
+// A lane holds column (li) of each 32x32 block of its wavefront's part of the tile,
+// rows 8*(r/4) + 4*half + r%4 for accumulator register r.  Chunk workgroups store raw
+// sums for splitk_reduce_kernel; whole tiles apply alpha, the C/bias term, the
+// residual and Relu and store to Y (NCHW for CONV).
+template <int BM, int BN, int WM, int WN, bool CONV>
+__device__ __forceinline__ void finish_tile(const Params &p,
+                                            f32x16 (&acc)[BM / (WM * 32)][BN / (WN * 32)],
+                                            bool whole, int lin, int chunk, int bz, int row0,
+                                            int col0) {
+  constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int li = lane & 31, half = lane >> 5;
+  const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
+  if (!whole) {
+    // raw sums of the whole tile (edge rows and columns included), tile-local
+    float *part = p.partial +
+                  ((long long)(lin - p.full_tiles) * p.tail_split + chunk) * (BM * BN);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int lr = wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          part[lr * BN + wcol + nt * 32 + li] = acc[mt][nt][r];
+        }
+    return;  // splitk_reduce_kernel adds the chunks up
+  }
+  // Whole tiles of results below 2 GiB: every address is one per-lane byte
+  // offset (column, plus the four rows by which the two halves of a wavefront
+  // differ) and one scalar offset per accumulator row, so a stored element costs
+  // no address arithmetic, no bounds test and no change of the execution mask.
+  if (p.y_bytes > 0 && row0 + BM <= p.m && col0 + BN <= p.n) {
+    const long long zoff = CONV ? 0 : (long long)bz * p.m * p.n;
+    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, p.y_bytes);
+    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, p.y_bytes);
+    const rsrc_t rsrc_c = make_rsrc(p.C ? p.C : p.Y, p.C ? p.c_bytes : 0);
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = col0 + wcol + nt * 32 + li;
+      int ybase, ystride, voff_c, cstride;  // in elements; byte offsets stay below 2^31
+      if (CONV) {
+        const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+        const unsigned img = (unsigned)fdiv(col, p.cv.fd_ohw);
+        ybase = (int)((img * (unsigned)p.cv.cout_total + (unsigned)(bz * p.cv.cout_g)) * ohw +
+                      ((unsigned)col - img * ohw));
+        ystride = (int)ohw;
+        voff_c = (bz * p.cv.cout_g + 4 * half) * 4;
+        cstride = 1;
+      } else {
+        ybase = col;
+        ystride = p.n;
+        voff_c = (int)((4 * half * p.sC0 + col * p.sC1) * 4);
+        cstride = (int)p.sC0;
+      }
+      const int voff_y = (ybase + 4 * half * ystride) * 4;
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int rbase = __builtin_amdgcn_readfirstlane(row0 + wrow + mt * 32);
+#pragma unroll
+        for (int hb = 0; hb < 2; hb++) {
+          float cv[8], rv[8];
+          if (p.C) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              cv[j] = buf_load(rsrc_c, voff_c, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * cstride * 4);
+          }
+          if (p.R) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              rv[j] = buf_load(rsrc_r, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
+          }
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            float y = p.alpha * acc[mt][nt][8 * hb + j];
+            if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+            if (p.R) y = y + rv[j];
+            if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+            buf_store(rsrc_y, y, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
+          }
+        }
+      }
+    }
+    return;
+  }
+  // Edge tiles and larger results.  Bias and residual values of a 32x32 block
+  // are all requested before the first is used, so the block pays one memory
+  // round trip, not thirty-two.  Loads use clamped indices (always inside the
+  // tensors); only the store is conditional.
+#pragma unroll
+  for (int nt = 0; nt < NT; nt++) {
+    const int col = col0 + wcol + nt * 32 + li;
+    const bool col_ok = col < p.n;
+    const int colc = col_ok ? col : p.n - 1;
+    long long ybase;     // offset of (row 0, this column) in Y
+    long long ystride;   // distance between consecutive rows in Y
+    if (CONV) {
+      const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+      const unsigned img = (unsigned)fdiv(colc, p.cv.fd_ohw);
+      const unsigned q = (unsigned)colc - img * ohw;
+      ybase = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g) * ohw + q;
+      ystride = ohw;
+    } else {
+      ybase = (long long)bz * p.m * p.n + colc;
+      ystride = p.n;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+      const int rfirst = row0 + wrow + mt * 32 + 4 * half;
+      // eight rows at a time keeps the 64-register tiles from spilling
+#pragma unroll
+      for (int hb = 0; hb < 2; hb++) {
+        float cv[8], rv[8];
+        if (p.C) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+            row = row < p.m ? row : p.m - 1;
+            cv[j] = CONV ? p.C[bz * p.cv.cout_g + row]
+                           : p.C[(long long)row * p.sC0 + (long long)colc * p.sC1];
+          }
+        }
+        if (p.R) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+            row = row < p.m ? row : p.m - 1;
+            rv[j] = p.R[ybase + (long long)row * ystride];
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
+          float y = p.alpha * acc[mt][nt][8 * hb + j];
+          if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+          if (p.R) y = y + rv[j];
+          if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+          if (col_ok && row < p.m) p.Y[ybase + (long long)row * ystride] = y;
+        }
+      }
+    }
   }
 }
 
@@ -408,11 +620,14 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   constexpr bool PIXELS = BMODE_ == B_PIXELS;
   constexpr bool CONV = IM2COL || PIXELS;  // Y is NCHW, the bias is per row
   constexpr bool B_IS_KC = BMODE_ == B_KC;
+  // layout of the B tile in LDS: tile[column][k] for a k-contiguous B and for the
+  // descriptor gather (whose threads hold consecutive k of one pixel)
+  constexpr bool B_LDS_KC = B_IS_KC || IM2COL_FAST;
   static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
   constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
   static_assert(MT >= 1 && NT >= 1, "tile too small for the wavefront grid");
   constexpr int A_FLOATS = tile_floats(A_KC, BM);
-  constexpr int B_FLOATS = tile_floats(B_IS_KC, BN);
+  constexpr int B_FLOATS = tile_floats(B_LDS_KC, BN);
   constexpr int LDA = BM + MC_PAD, LDB = BN + MC_PAD;
   __shared__ __attribute__((aligned(16))) float lds_a[2][A_FLOATS];
   __shared__ __attribute__((aligned(16))) float lds_b[2][B_FLOATS];
@@ -425,23 +640,10 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
   const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
 
   // which tile, and which part of K
-  const int pid = blockIdx.x;
-  const bool whole = pid < p.full_tiles;
-  int lin, chunk = 0;
-  if (whole) {
-    lin = xcd_contiguous(pid, p.full_tiles);
-  } else {
-    // chunk workgroups: an XCD takes a contiguous run of (chunk, tile) pairs with the
-    // tile varying fastest, so that tiles which share a slice of B meet in one L2
-    const int v = xcd_contiguous(pid - p.full_tiles, p.tail_tiles * p.tail_split);
-    chunk = v / p.tail_tiles;
-    lin = p.full_tiles + (v - chunk * p.tail_tiles);
-  }
-  const int tiles_per_z = p.tiles_m * p.tiles_n;
-  const int bz = lin / tiles_per_z;  // batch entry (gemm) or group (conv)
-  int tm, tn;
-  tile_coords(lin - bz * tiles_per_z, p.tiles_m, p.tiles_n, &tm, &tn);
-  const int row0 = tm * BM, col0 = tn * BN;
+  const TileWork tw = decode_work(p);
+  const bool whole = tw.whole;
+  const int lin = tw.lin, chunk = tw.chunk, bz = tw.bz;
+  const int row0 = tw.tm * BM, col0 = tw.tn * BN;
 
   const float *A = p.A + (long long)bz * p.sAb;
   const float *B = p.B + (long long)bz * p.sBb;
@@ -488,7 +690,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     long long colpos = col0 + (tid % TPR) * 4;
     if (PIXELS) {
       const unsigned plane = (unsigned)(p.cv.h * p.cv.w);
-      const unsigned img = (unsigned)colpos / plane;
+      const unsigned img = (unsigned)fdiv((int)colpos, p.cv.fd_plane);
       colpos = (long long)img * p.cv.c_total * plane + ((unsigned)colpos - img * plane);
     }
 #pragma unroll
@@ -509,9 +711,9 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     bbase = px.xbase - bias;
     if (P < (unsigned)p.cv.npix) {
       const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
-      const unsigned img = P / ohw;
+      const unsigned img = (unsigned)fdiv((int)P, p.cv.fd_ohw);
       const unsigned q = P - img * ohw;
-      const int oy = (int)(q / (unsigned)p.cv.ow), ox = (int)q - oy * p.cv.ow;
+      const int oy = fdiv((int)q, p.cv.fd_ow), ox = (int)q - oy * p.cv.ow;
       const long long img_off = (long long)img * p.cv.c_total * plane;
       px.iy0 = oy * p.cv.sh - p.cv.pt;
       px.ix0 = ox * p.cv.sw - p.cv.pl;
@@ -614,7 +816,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
           av[mt][j] = *reinterpret_cast<const f32x4 *>(
               ta + (wrow + mt * 32 + li) * LDK + 8 * j + 4 * half);
     }
-    if (B_IS_KC) {
+    if (B_LDS_KC) {
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
 #pragma unroll
@@ -631,7 +833,7 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
         a_el[mt] = A_KC ? av[mt][st >> 2][st & 3] : ta[kk * LDA + wrow + mt * 32 + li];
 #pragma unroll
       for (int nt = 0; nt < NT; nt++)
-        b_el[nt] = B_IS_KC ? bv[nt][st >> 2][st & 3] : tb[kk * LDB + wcol + nt * 32 + li];
+        b_el[nt] = B_LDS_KC ? bv[nt][st >> 2][st & 3] : tb[kk * LDB + wcol + nt * 32 + li];
 #pragma unroll
       for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -678,137 +880,215 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     __syncthreads();
   }
 
-  // ---- epilogue: lane holds column (li) of each 32x32 tile, rows
-  // 8*(r/4) + 4*half + r%4 for accumulator register r.
-  if (!whole) {
-    // raw sums of the whole tile (edge rows and columns included), tile-local
-    float *part = p.partial +
-                  ((long long)(lin - p.full_tiles) * p.tail_split + chunk) * (BM * BN);
-#pragma unroll
-    for (int nt = 0; nt < NT; nt++)
-#pragma unroll
-      for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int lr = wrow + mt * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          part[lr * BN + wcol + nt * 32 + li] = acc[mt][nt][r];
-        }
-    return;  // splitk_reduce_kernel adds the chunks up
+  finish_tile<BM, BN, WM, WN, CONV>(p, acc, whole, lin, chunk, bz, row0, col0);
+}
+
+// ---- 3x3, stride 1, dilation 1: taps read from an input tile staged in LDS -------
+// Same contraction as the gathered form (M = output channels, N = pixels in
+// (image, oy, ox) order, K = (channel, ky, kx)), same tiles, same work plan and
+// epilogue.  What differs is how B reaches the matrix cores.  K advances in blocks of
+// 8 input channels (72 k).  For a block, the workgroup copies the input rows its BN
+// pixels touch -- whole rows, as they lie in X, with 16-, 8- or 4-byte loads -- into
+// LDS: xs[channel][slot][column], where consecutive output rows of an image share
+// slots (output row R of the tile, tap row ky -> slot (R - R0) + ky + 2 * (images
+// after the tile's first)), columns left and right of the row and rows above and
+// below the image are zero (requested through offsets outside the descriptor, so they
+// cost no memory traffic).  A lane then reads tap (ky, kx) of channel c of its pixel at
+// a fixed distance from its pixel's corner: one LDS address per tap and lane, computed
+// once per tile, plus an immediate per channel.  No tap table, no padding masks, no
+// address arithmetic in the loop; each input element is fetched once per tile and
+// block instead of once per tap, and a block (36 MFMA steps) costs two barriers.
+// The weights of a block, a[row][72 k] in the order they lie in W, are read with
+// 16-byte LDS loads: the lower half of a wavefront multiplies channels 0-3 of the
+// block (k 0..35), the upper half channels 4-7 (k 36..71), so the two k of one MFMA
+// step are (c, tap) and (c + 4, tap).
+constexpr int HALO_CB = 8;                 // channels per K block
+constexpr int HALO_KB = HALO_CB * 9;       // k per block
+constexpr int HALO_ROWA = HALO_KB + 4;     // weight tile row stride (floats)
+constexpr int HALO_AROWS = 14;             // weight rows per pass: 256 threads = 14 rows x 18 pieces
+// floats per channel of the input tile; 32 mod 64 so that the two halves of a
+// wavefront (channels c and c + 4) fall on different LDS banks
+constexpr int halo_plane(int bn) { return bn <= 64 ? 480 : 544; }
+// 16/8/4-byte pieces of the input tile per thread and block
+constexpr int halo_units(int vecw) { return vecw == 1 ? 5 : 4; }
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+template <int VECW> struct HaloPiece;
+template <> struct HaloPiece<4> {
+  typedef f32x4 type;
+  static __device__ __forceinline__ type load(rsrc_t r, int voff, int soff) {
+    return buf_load4(r, voff, soff);
   }
-  // Whole tiles of results below 2 GiB: every address is one per-lane byte
-  // offset (column, plus the four rows by which the two halves of a wavefront
-  // differ) and one scalar offset per accumulator row, so a stored element costs
-  // no address arithmetic, no bounds test and no change of the execution mask.
-  if (p.y_bytes > 0 && row0 + BM <= p.m && col0 + BN <= p.n) {
-    const long long zoff = CONV ? 0 : (long long)bz * p.m * p.n;
-    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, p.y_bytes);
-    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, p.y_bytes);
-    const rsrc_t rsrc_c = make_rsrc(p.C ? p.C : p.Y, p.C ? p.c_bytes : 0);
+};
+template <> struct HaloPiece<2> {
+  typedef f32x2 type;
+  static __device__ __forceinline__ type load(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(f32x2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+  }
+};
+template <> struct HaloPiece<1> {
+  typedef float type;
+  static __device__ __forceinline__ type load(rsrc_t r, int voff, int soff) {
+    return buf_load(r, voff, soff);
+  }
+};
+
+template <int BM, int BN, int WM, int WN, int VECW>
+__global__ __launch_bounds__(NTHREADS, BM * BN <= 64 * 64 ? 4 : 2) void conv3x3_halo_kernel(Params p) {
+  static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
+  constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
+  constexpr int PLANE = halo_plane(BN);
+  constexpr int AU = (BM + HALO_AROWS - 1) / HALO_AROWS;  // weight pieces per thread and block
+  constexpr int XU = halo_units(VECW);
+  typedef typename HaloPiece<VECW>::type xpiece;
+  __shared__ __attribute__((aligned(16))) float as[AU * HALO_AROWS * HALO_ROWA];
+  __shared__ __attribute__((aligned(16))) float xs[HALO_CB * PLANE + 4];  // + a dump cell for idle pieces
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int li = lane & 31, half = lane >> 5;
+  const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
+
+  const TileWork t = decode_work(p);
+  const int row0 = t.tm * BM, col0 = t.tn * BN;
+  const int kbeg = t.whole ? 0 : t.chunk * p.kchunk;
+  const int kend = t.whole ? p.k : (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k);
+
+  const ConvGeom &cv = p.cv;
+  const int plane_in = cv.h * cv.w;
+  // first output row of the tile (rows numbered through the batch) and its image
+  const int R0 = fdiv(col0, cv.fd_ow);
+  const int img0 = fdiv(R0, cv.fd_oh);
+
+  // ---- weights: piece (row r0 + 14 i, k 4q .. 4q+3) of the block -----------------
+  // (threads 252..255 repeat pieces of row 13: same values to the same cells)
+  const int q = tid % 18, r0 = tid / 18 < HALO_AROWS ? tid / 18 : HALO_AROWS - 1;
+  int voff_a[AU];
 #pragma unroll
-    for (int nt = 0; nt < NT; nt++) {
-      const int col = col0 + wcol + nt * 32 + li;
-      int ybase, ystride, voff_c, cstride;  // in elements; byte offsets stay below 2^31
-      if (CONV) {
-        const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
-        const unsigned img = (unsigned)col / ohw;
-        ybase = (int)((img * (unsigned)p.cv.cout_total + (unsigned)(bz * p.cv.cout_g)) * ohw +
-                      ((unsigned)col - img * ohw));
-        ystride = (int)ohw;
-        voff_c = (bz * p.cv.cout_g + 4 * half) * 4;
-        cstride = 1;
-      } else {
-        ybase = col;
-        ystride = p.n;
-        voff_c = (int)((4 * half * p.sC0 + col * p.sC1) * 4);
-        cstride = (int)p.sC0;
-      }
-      const int voff_y = (ybase + 4 * half * ystride) * 4;
+  for (int i = 0; i < AU; i++) {
+    int r = row0 + r0 + HALO_AROWS * i;
+    r = r < p.m ? r : p.m - 1;  // rows past the edge are never stored
+    voff_a[i] = (r * p.k + 4 * q) * 4;
+  }
+  const int lds_a_w = (r0 * HALO_ROWA + 4 * q) * 4;
+  const rsrc_t rsrc_a = make_rsrc(p.A + (long long)t.bz * p.sAb, p.a_bytes);
+
+  // ---- input rows: piece u = tid + 256 i -> (channel, slot, column group) ---------
+  const int pg = cv.pitch / VECW;       // pieces per row
+  const int upc = cv.slots * pg;        // pieces per channel
+  const int first_rows = (img0 + 1) * cv.oh - R0;  // output rows from R0 to the end of its image
+  int voff_x[XU], lds_x_w[XU];
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) {
-        const int rbase = __builtin_amdgcn_readfirstlane(row0 + wrow + mt * 32);
-#pragma unroll
-        for (int hb = 0; hb < 2; hb++) {
-          float cv[8], rv[8];
-          if (p.C) {
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-              cv[j] = buf_load(rsrc_c, voff_c, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * cstride * 4);
-          }
-          if (p.R) {
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-              rv[j] = buf_load(rsrc_r, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
-          }
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            float y = p.alpha * acc[mt][nt][8 * hb + j];
-            if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
-            if (p.R) y = y + rv[j];
-            if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
-            buf_store(rsrc_y, y, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
-          }
-        }
-      }
+  for (int i = 0; i < XU; i++) {
+    const int u = tid + NTHREADS * i;
+    const int c = fdiv(u, cv.fd_upc), rem = u - c * upc;
+    const int slot = fdiv(rem, cv.fd_pg), cg = rem - slot * pg;
+    // which input row the slot holds
+    int d, iy;
+    if (slot < first_rows + 2) {
+      d = 0;
+      iy = (R0 - img0 * cv.oh) - cv.pt + slot;
+    } else {
+      const int s2 = slot - first_rows - 2;
+      const int dd = fdiv(s2, cv.fd_oh2);
+      d = 1 + dd;
+      iy = s2 - dd * (cv.oh + 2) - cv.pt;
     }
-    return;
+    const int img = img0 + d;
+    const int ix = cg * VECW - cv.col0;
+    const bool live = c < HALO_CB;
+    const bool data = live && (long long)img * cv.oh * cv.ow < cv.npix && iy >= 0 && iy < cv.h &&
+                      ix >= 0 && ix + VECW <= cv.w;
+    voff_x[i] = data ? (((img * cv.c_total + c) * cv.h + iy) * cv.w + ix) * 4 : BUF_OOB;
+    lds_x_w[i] = live ? (c * PLANE + slot * cv.pitch + cg * VECW) * 4 : HALO_CB * PLANE * 4;
   }
-  // Edge tiles and larger results.  Bias and residual values of a 32x32 block
-  // are all requested before the first is used, so the block pays one memory
-  // round trip, not thirty-two.  Loads use clamped indices (always inside the
-  // tensors); only the store is conditional.
+  const long long group_off = (long long)t.bz * cv.c_in_g * plane_in;
+  const rsrc_t rsrc_x = make_rsrc(p.B + group_off, p.b_bytes - (int)(group_off * 4));
+
+  // ---- where a lane finds its operands in LDS -------------------------------------
+  int lds_a_r[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++)
+    lds_a_r[mt] = ((wrow + mt * 32 + li) * HALO_ROWA + 36 * half) * 4;
+  int lds_b_r[NT][9];
 #pragma unroll
   for (int nt = 0; nt < NT; nt++) {
-    const int col = col0 + wcol + nt * 32 + li;
-    const bool col_ok = col < p.n;
-    const int colc = col_ok ? col : p.n - 1;
-    long long ybase;     // offset of (row 0, this column) in Y
-    long long ystride;   // distance between consecutive rows in Y
-    if (CONV) {
-      const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
-      const unsigned img = (unsigned)colc / ohw;
-      const unsigned q = (unsigned)colc - img * ohw;
-      ybase = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g) * ohw + q;
-      ystride = ohw;
-    } else {
-      ybase = (long long)bz * p.m * p.n + colc;
-      ystride = p.n;
-    }
+    int P = col0 + wcol + nt * 32 + li;
+    P = P < (int)cv.npix ? P : (int)cv.npix - 1;  // lanes past the edge are never stored
+    const int R = fdiv(P, cv.fd_ow), ox = P - R * cv.ow;
+    const int slot0 = (R - R0) + 2 * (fdiv(R, cv.fd_oh) - img0);
+    const int corner = (4 * half * PLANE + slot0 * cv.pitch + cv.col0 - cv.pl + ox) * 4;
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-      const int rfirst = row0 + wrow + mt * 32 + 4 * half;
-      // eight rows at a time keeps the 64-register tiles from spilling
+    for (int tap = 0; tap < 9; tap++)
+      lds_b_r[nt][tap] = corner + ((tap / 3) * cv.pitch + tap % 3) * 4;
+  }
+
+  f32x16 acc[MT][NT];
 #pragma unroll
-      for (int hb = 0; hb < 2; hb++) {
-        float cv[8], rv[8];
-        if (p.C) {
+  for (int a = 0; a < MT; a++)
 #pragma unroll
-          for (int j = 0; j < 8; j++) {
-            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
-            row = row < p.m ? row : p.m - 1;
-            cv[j] = CONV ? p.C[bz * p.cv.cout_g + row]
-                           : p.C[(long long)row * p.sC0 + (long long)colc * p.sC1];
-          }
-        }
-        if (p.R) {
+    for (int b = 0; b < NT; b++)
 #pragma unroll
-          for (int j = 0; j < 8; j++) {
-            int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
-            row = row < p.m ? row : p.m - 1;
-            rv[j] = p.R[ybase + (long long)row * ystride];
-          }
-        }
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+
+  f32x4 ra[AU];
+  xpiece rx[XU];
+  auto fetch = [&](int k0) {
+    const int soff_a = k0 * 4;
+    const int soff_x = (k0 / 9) * plane_in * 4;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-          const int row = rfirst + 16 * hb + 8 * (j >> 2) + (j & 3);
-          float y = p.alpha * acc[mt][nt][8 * hb + j];
-          if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
-          if (p.R) y = y + rv[j];
-          if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
-          if (col_ok && row < p.m) p.Y[ybase + (long long)row * ystride] = y;
-        }
+    for (int i = 0; i < AU; i++) ra[i] = buf_load4(rsrc_a, voff_a[i], soff_a);
+#pragma unroll
+    for (int i = 0; i < XU; i++) rx[i] = HaloPiece<VECW>::load(rsrc_x, voff_x[i], soff_x);
+  };
+  auto stash = [&]() {
+    char *const as_b = reinterpret_cast<char *>(as);
+    char *const xs_b = reinterpret_cast<char *>(xs);
+#pragma unroll
+    for (int i = 0; i < AU; i++)
+      *reinterpret_cast<f32x4 *>(as_b + lds_a_w + i * (HALO_AROWS * HALO_ROWA * 4)) = ra[i];
+#pragma unroll
+    for (int i = 0; i < XU; i++) *reinterpret_cast<xpiece *>(xs_b + lds_x_w[i]) = rx[i];
+  };
+  auto compute = [&]() {
+    const char *const as_b = reinterpret_cast<const char *>(as);
+    const char *const xs_b = reinterpret_cast<const char *>(xs);
+#pragma unroll
+    for (int j = 0; j < 9; j++) {
+      f32x4 av[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++)
+        av[mt] = *reinterpret_cast<const f32x4 *>(as_b + lds_a_r[mt] + 16 * j);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int kk = 4 * j + e, c = kk / 9, tap = kk % 9;
+        float b_el[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++)
+          b_el[nt] = *reinterpret_cast<const float *>(xs_b + lds_b_r[nt][tap] + c * (PLANE * 4));
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+          for (int nt = 0; nt < NT; nt++)
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mt][e], b_el[nt], acc[mt][nt], 0, 0, 0);
       }
     }
+  };
+
+  // One LDS buffer: block b+1 travels global -> registers while block b runs through
+  // the matrix cores, and is written to LDS once every wavefront has finished reading.
+  fetch(kbeg);
+  for (int k0 = kbeg; k0 < kend; k0 += HALO_KB) {
+    if (k0 != kbeg) __syncthreads();
+    stash();
+    __syncthreads();
+    if (k0 + HALO_KB < kend) fetch(k0 + HALO_KB);
+    __builtin_amdgcn_sched_barrier(0);
+    compute();
   }
+  finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0);
 }
 
 // Reference-order scalar kernel for operands that are dense in neither index
@@ -840,9 +1120,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(Params p, int bm, in
   const int j = blockIdx.x;
   const int lin = p.full_tiles + j;
   const int tiles_per_z = p.tiles_m * p.tiles_n;
-  const int bz = lin / tiles_per_z;
+  const int bz = fdiv(lin, p.fd_tiles_per_z);
   int tm, tn;
-  tile_coords(lin - bz * tiles_per_z, p.tiles_m, p.tiles_n, &tm, &tn);
+  tile_coords(p, lin - bz * tiles_per_z, &tm, &tn);
   reduce_quad<CONV>(p, bm, bn, j, bz, tm, tn, ((int)blockIdx.y * 256 + (int)threadIdx.x) * 4);
 }
 
@@ -859,11 +1139,14 @@ const int kTileN[] = {128, 256, 128, 64, 64};
 // reachable through wdh_set_option.
 TileId pick_tile(int m, int n, int nz) {
   const long long tiles128 = (long long)((m + 127) / 128) * ((n + 127) / 128) * nz;
-  return tiles128 >= 2LL * wdh::compute_units() ? T128x128 : T64x64;
+  // a 128-row tile over 64 rows (or 128 columns over 64) would compute mostly padding
+  const double filled = (double)m * n * nz / ((double)tiles128 * 128.0 * 128.0);
+  return tiles128 >= 2LL * wdh::compute_units() && filled >= 0.8 ? T128x128 : T64x64;
 }
 
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
+int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
 
 // How the tiles of one launch are spread over the chip.
 struct WorkPlan {
@@ -882,13 +1165,16 @@ struct WorkPlan {
 // sooner than `solo` times the longest single workgroup (the slow-down of a
 // workgroup that runs alone on a CU); every workgroup adds a start-up/epilogue
 // cost and a split adds the reduce pass over the partial sums.
-WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather) {
+WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather, int kgran = BK) {
+  // kgran: the K loop advances in units of this many elements (a chunk is a whole number of them);
+  // the model's constants are per 16 elements
   const long long cus = wdh::compute_units();
-  const int slabs = (k + BK - 1) / BK;
+  const int slabs = (k + kgran - 1) / kgran;
+  const double per16 = kgran / 16.0;
   WorkPlan w = {tiles, 0, 1, 0};
   auto with_split = [&](long long tail, int s) {
     WorkPlan r;
-    r.kchunk = ((slabs + s - 1) / s) * BK;
+    r.kchunk = ((slabs + s - 1) / s) * kgran;
     r.split = (k + r.kchunk - 1) / r.kchunk;
     if (r.split < 1) r.split = 1;
     r.tail = r.split > 1 ? tail : 0;
@@ -900,9 +1186,9 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather) {
     const int s = g_forced_split < slabs ? g_forced_split : (slabs > 0 ? slabs : 1);
     return s > 1 ? with_split(tiles, s) : w;
   }
-  if (slabs < 8) return w;
+  if (slabs * per16 < 8) return w;
   const double area = (double)bm * bn / (64.0 * 64.0);
-  const double slab_us = 0.30 * area;
+  const double slab_us = 0.30 * area * per16;
   const double start_us = 0.9 * (area > 1.0 ? 2.0 : 1.0);
   const double tile_bytes = (double)bm * bn * 4.0;
   // A launch cannot finish sooner than its longest workgroup, and with the CU mostly to
@@ -924,7 +1210,9 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather) {
     return t;
   };
   const long long rem = tiles % cus;
-  const int max_s = slabs / 4 < 32 ? slabs / 4 : 32;  // at least 4 slabs per chunk
+  // at least 64 elements of K per chunk
+  const int min_units = per16 >= 4.0 ? 1 : (int)(4.0 / per16 + 0.999);
+  const int max_s = slabs / min_units < 32 ? slabs / min_units : 32;
   double best;
   // unsplit: the remainder tiles make one more (partial) round of whole tiles
   {
@@ -946,12 +1234,14 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather) {
   return best_s > 1 ? with_split(best_tail, best_s) : w;
 }
 
-template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE>
-int launch_tile(Params &p, int nz, bool vec) {
+// Plans the work of one launch, provides the partial-sum workspace, starts the main
+// kernel through `start(grid)` and, if tiles were cut along K, the reduce pass.
+template <int BM, int BN, typename Start>
+int launch_planned(Params &p, int nz, bool conv, int kgran, Start start) {
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   const long long tiles = (long long)p.tiles_m * p.tiles_n * nz;
-  const WorkPlan w = plan_work(tiles, p.k, BM, BN, BMODE >= B_IM2COL32);
+  const WorkPlan w = plan_work(tiles, p.k, BM, BN, conv, kgran);
   const long long blocks = w.full + w.tail * w.split;
   if (blocks > 0x7fffffffLL)
     return wdh::fail(WDH_EINVAL, "contraction: %lld workgroups exceed the grid limit", blocks);
@@ -960,23 +1250,21 @@ int launch_tile(Params &p, int nz, bool vec) {
   p.tail_tiles = (int)w.tail;
   p.tail_split = w.split;
   p.kchunk = w.kchunk;
+  p.fd_tiles_per_z = make_fastdiv((long long)p.tiles_m * p.tiles_n);
+  p.fd_tail_tiles = make_fastdiv(w.tail > 0 ? w.tail : 1);
+  p.fd_group = make_fastdiv((long long)TILE_GROUP * p.tiles_n);
+  p.fd_last_rows = make_fastdiv(p.tiles_m % TILE_GROUP ? p.tiles_m % TILE_GROUP : 1);
   wdh_buf scratch = 0;
   if (w.tail > 0) {
     scratch = wdh_alloc((size_t)w.tail * w.split * BM * BN * sizeof(float));
     if (!scratch) return WDH_ENOMEM;
     p.partial = (float *)wdh::resolve(scratch, nullptr);
   }
-  dim3 grid((unsigned)blocks);
-  if (vec)
-    hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, true>), grid,
-                       dim3(NTHREADS), 0, wdh::stream(), p);
-  else
-    hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, false>), grid,
-                       dim3(NTHREADS), 0, wdh::stream(), p);
+  start(dim3((unsigned)blocks));
   hipError_t e = hipGetLastError();
   if (e == hipSuccess && w.tail > 0) {
     dim3 rgrid((unsigned)w.tail, (unsigned)(BM * BN / 1024));
-    if (BMODE >= B_IM2COL32)
+    if (conv)
       hipLaunchKernelGGL(splitk_reduce_kernel<true>, rgrid, dim3(256), 0, wdh::stream(), p,
                          BM, BN);
     else
@@ -990,6 +1278,52 @@ int launch_tile(Params &p, int nz, bool vec) {
   if (e != hipSuccess)
     return wdh::fail(WDH_EHIP, "contraction launch failed: %s", hipGetErrorString(e));
   return WDH_OK;
+}
+
+template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE>
+int launch_tile(Params &p, int nz, bool vec) {
+  return launch_planned<BM, BN>(p, nz, BMODE >= B_IM2COL32, BK, [&](dim3 grid) {
+    if (vec)
+      hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, true>), grid,
+                         dim3(NTHREADS), 0, wdh::stream(), p);
+    else
+      hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, false>), grid,
+                         dim3(NTHREADS), 0, wdh::stream(), p);
+  });
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_halo_tile(Params &p, int nz, int vecw) {
+  return launch_planned<BM, BN>(p, nz, true, HALO_KB, [&](dim3 grid) {
+    if (vecw == 4)
+      hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4>), grid, dim3(NTHREADS), 0,
+                         wdh::stream(), p);
+    else if (vecw == 2)
+      hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 2>), grid, dim3(NTHREADS), 0,
+                         wdh::stream(), p);
+    else
+      hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 1>), grid, dim3(NTHREADS), 0,
+                         wdh::stream(), p);
+  });
+}
+
+// Fills in the LDS layout of the input tile for BN-pixel tiles; false if the geometry
+// does not fit the kernel's LDS budget (the gathered form serves it then).
+bool halo_fits(ConvGeom &cv, int bn, int nimg, int vecw, int pr) {
+  const int up = [](int v, int to) { return (v + to - 1) / to * to; }(cv.pl, vecw);
+  cv.col0 = up;
+  cv.pitch = up + cv.w + (pr + vecw - 1) / vecw * vecw;
+  int rows = 2 + (bn - 2) / cv.ow;
+  int imgs = 2 + (bn - 2) / (cv.oh * cv.ow);
+  if (imgs > nimg) imgs = nimg;
+  if (rows > nimg * cv.oh) rows = nimg * cv.oh;
+  cv.slots = rows + 2 * imgs;
+  cv.fd_oh2 = make_fastdiv(cv.oh + 2);
+  cv.fd_pg = make_fastdiv(cv.pitch / vecw);
+  cv.fd_upc = make_fastdiv((long long)cv.slots * (cv.pitch / vecw));
+  const long long pieces = (long long)HALO_CB * cv.slots * (cv.pitch / vecw);
+  return (long long)cv.slots * cv.pitch <= halo_plane(bn) &&
+         pieces <= (long long)halo_units(vecw) * NTHREADS;
 }
 
 template <bool A_KC, int BMODE>
@@ -1036,6 +1370,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     if (value < -1 || value == 0 || value > 64)
       return fail(WDH_EINVAL, "wdh_set_option: split_k %d (use -1 or 1..64)", value);
     g_forced_split = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "conv3x3_halo") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: conv3x3_halo %d (use 0 or 1)", value);
+    g_halo = value;
     return WDH_OK;
   }
   return fail(WDH_EINVAL, "wdh_set_option: unknown option \"%s\"", name);
@@ -1214,6 +1554,11 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   if (!wdh::operand(hY, out_bytes, "wdh_conv2d: Y", &ptr)) return WDH_EINVAL;
   p.Y = (float *)ptr;
 
+  p.cv.fd_ow = make_fastdiv(ow);
+  p.cv.fd_oh = make_fastdiv(oh);
+  p.cv.fd_ohw = make_fastdiv((long long)oh * ow);
+  p.cv.fd_plane = make_fastdiv((long long)h * w);
+
   const int ntaps = kh * kw;
   // Descriptor loads need every byte offset formed in the kernel (X, shifted up
   // by the top-left padding, and one group's weights) to stay below 2^31.
@@ -1241,6 +1586,29 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
     p.c_bytes = cout * 4;
     return launch<true, B_PIXELS>(p, group, true);
+  }
+  // 3x3, stride 1, no dilation, input channels in blocks of 8: taps read from an input
+  // tile staged in LDS (conv3x3_halo_kernel)
+  if (g_halo && small && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 &&
+      c_in_g % HALO_CB == 0 && aligned16(p.A)) {
+    const int vecw = (w % 4 == 0 && aligned16(p.B)) ? 4 : ((w % 2 == 0 && ((uintptr_t)p.B & 7) == 0) ? 2 : 1);
+    p.cv.h = h; p.cv.w = w; p.cv.oh = oh; p.cv.ow = ow; p.cv.pt = pt; p.cv.pl = pl;
+    const int bn = g_forced_tile == T64x128 ? 128 : 64;
+    if (halo_fits(p.cv, bn, n, vecw, pr)) {
+      p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
+      p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
+      p.alpha = 1.0f; p.beta = 1.0f; p.epilogue = epilogue;
+      p.cv.c_in_g = c_in_g; p.cv.sh = p.cv.sw = p.cv.dh = p.cv.dw = 1; p.cv.kh = p.cv.kw = 3;
+      p.cv.c_total = c; p.cv.cout_total = cout; p.cv.cout_g = cout_g;
+      p.cv.ntaps = 9; p.cv.npix = npix;
+      p.fast = 1;
+      p.a_bytes = (int)w_bytes;
+      p.b_bytes = (int)((long long)n * c * h * w * 4);
+      p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+      p.c_bytes = cout * 4;
+      if (bn == 128) return launch_halo_tile<64, 128, 1, 4>(p, group, vecw);
+      return launch_halo_tile<64, 64, 2, 2>(p, group, vecw);
+    }
   }
   const int mode = !small || ntaps > 63 ? B_IM2COL_BIG : (ntaps > 31 ? B_IM2COL64 : B_IM2COL32);
   KtabKey key;
