@@ -72,7 +72,18 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *   "split_k"           -1 = choose per problem (default); n >= 1 = cut the
  *                       K loop of every tile of wdh_gemm / wdh_conv2d into n
  *                       chunks whose partial sums are added in chunk order
- *                       by a second kernel (1 = never split). */
+ *                       by a second kernel (1 = never split).
+ *   "conv3x3_halo"      1 (default) = 3x3, stride-1, undilated convolutions whose
+ *                       input channels per group are a multiple of 8 stage the
+ *                       input rows of a tile in LDS and read the taps from there;
+ *                       0 = they gather taps from global memory like every other
+ *                       geometry (both forms compute the same sums).
+ *   "descriptor_loads"  1 (default) = operands below 2 GiB are read and written
+ *                       through buffer descriptors with 32-bit offsets; 0 = every
+ *                       operand is treated as if it spanned 2 GiB or more (64-bit
+ *                       addresses, bounds-checked stores, the gather form for every
+ *                       convolution).  A test hook: it runs the large-operand code
+ *                       on ordinary sizes. */
 int wdh_set_option(const char *name, int value);
 
 /* ---- buffers --------------------------------------------------------- */

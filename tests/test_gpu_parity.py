@@ -774,3 +774,165 @@ def test_split_k_auto_on_deep_small_layers(ctx):
                      "3x3 512 @7x7")
     A, B = uni(64, 4096), uni(4096, 48)
     assert_close_max(hip_gemm(ctx, A, B), ref.gemm(A, B), GEMM_TOL, "skinny gemm")
+
+
+# ------------------------------------------------------------------ every contraction path
+BIG_KERNEL_CONVS = [
+    # n, cin, h, w, cout, kh, kw, pads, strides, dil, group: more than 63 taps -> the flat-load gather
+    (2, 6, 30, 31, 10, 9, 9, [4, 4, 4, 4], [1, 1], [1, 1], 1),
+    (1, 8, 40, 37, 12, 11, 11, [5, 3, 2, 5], [2, 3], [1, 1], 2),
+    (2, 4, 45, 45, 6, 9, 9, [8, 8, 8, 8], [2, 2], [2, 2], 1),
+    (1, 3, 64, 50, 5, 11, 9, [0, 0, 0, 0], [1, 2], [1, 1], 1),
+    (1, 16, 26, 26, 16, 9, 9, [4, 4, 4, 4], [1, 1], [1, 1], 16),   # depthwise
+    (3, 5, 23, 29, 70, 8, 9, [3, 4, 4, 4], [1, 1], [1, 1], 1),     # two row tiles, ragged K (360)
+]
+
+
+@pytest.mark.parametrize("shape", BIG_KERNEL_CONVS)
+def test_conv_kernels_of_more_than_63_taps(ctx, shape):
+    n, cin, h, w, cout, kh, kw, pads, strides, dil, group = shape
+    X, B = uni(n, cin, h, w, lo=0), nrm(cout)
+    W = nrm(cout, cin // group, kh, kw, std=float(np.sqrt(2.0 / (cin // group * kh * kw))))
+    want = ref.conv(X, W, B, dil, group, None, pads, strides)
+    got = hip_conv(ctx, X, W, B, dil, group, pads, strides)
+    assert_close_max(got, want, GEMM_TOL, "conv %s" % (shape,))
+    R = nrm(*want.shape)
+    fused = hip_conv(ctx, X, W, B, dil, group, pads, strides, epilogue="relu", R=R)
+    assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "big-kernel conv + residual + relu")
+
+
+def test_conv_reference_large_im2col_case(ctx):
+    """The reference's conv11 (test/model_test/make_models.py:641-643): Conv2d(1, 1, 4, 1, 1) on
+    (32, 1, 1027, 1027), the case that makes its CPU backend split the im2col buffer."""
+    X, W, B = uni(32, 1, 1027, 1027), nrm(1, 1, 4, 4, std=0.25), nrm(1)
+    got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])
+    assert got.shape == (32, 1, 1026, 1026)
+    for img in (0, 17, 31):
+        want = ref.conv(X[img:img + 1], W, B, pads=[1, 1, 1, 1])
+        assert_close_max(got[img:img + 1], want, GEMM_TOL, "conv11 image %d" % img)
+
+
+@pytest.mark.parametrize("ta,tb", list(itertools.product([0, 1], [0, 1])))
+def test_flat_load_loop_and_checked_epilogue_on_ordinary_sizes(ctx, ta, tb):
+    """descriptor_loads = 0 sends ordinary operands down the paths that 2 GiB operands take: flat
+    loads in the general loop, the bounds-checked epilogue, the flat-load conv gather."""
+    m, n, k = 150, 203, 77
+    A, B, C = (uni(k, m) if ta else uni(m, k)), (uni(n, k) if tb else uni(k, n)), uni(n)
+    A2, B2 = (uni(64, 256) if ta else uni(256, 64)), (uni(128, 64) if tb else uni(64, 128))
+    X, W, Bv, R = uni(3, 16, 19, 21, lo=0), he(40, 16, 3), nrm(40), nrm(3, 40, 19, 21)
+    X1, W1 = uni(4, 32, 8, 8), uni(24, 32, 1, 1)
+    want = {}
+    for mode in (1, 0):
+        try:
+            ctx.set_option("descriptor_loads", mode)
+            got = {
+                "gemm": hip_gemm(ctx, A, B, C, 0.5, 2.0, ta, tb, epilogue="relu"),
+                "gemm whole tiles": hip_gemm(ctx, A2, B2, None, 1.0, 1.0, ta, tb),
+                "conv 3x3": hip_conv(ctx, X, W, Bv, pads=[1, 1, 1, 1], epilogue="relu", R=R),
+                "conv 3x3 s2": hip_conv(ctx, X, W, Bv, pads=[1, 0, 1, 2], strides=[2, 1]),
+                "conv 1x1": hip_conv(ctx, X1, W1),
+            }
+        finally:
+            ctx.set_option("descriptor_loads", 1)
+        if mode == 1:
+            want = got
+            continue
+        assert_close_max(got["gemm"], ref.unary("Relu", ref.gemm(A, B, C, 0.5, 2.0, ta, tb)), GEMM_TOL, "flat gemm")
+        assert_close_max(got["gemm whole tiles"], ref.gemm(A2, B2, None, 1.0, 1.0, ta, tb), GEMM_TOL, "flat gemm 2")
+        assert_close_max(got["conv 3x3"], ref.unary("Relu", ref.binary("Add", ref.conv(X, W, Bv, pads=[1, 1, 1, 1]), R)),
+                         GEMM_TOL, "flat conv")
+        assert_close_max(got["conv 3x3 s2"], ref.conv(X, W, Bv, pads=[1, 0, 1, 2], strides=[2, 1]), GEMM_TOL, "flat conv s2")
+        assert_close_max(got["conv 1x1"], ref.conv(X1, W1), GEMM_TOL, "flat conv 1x1")
+        for key in got:
+            # the two forms add the same products; only the order inside a K slab may differ
+            assert_close_max(got[key], want[key], 1e-5, "descriptor vs flat: " + key)
+    with pytest.raises(capi.HipError):
+        ctx.set_option("descriptor_loads", 2)
+
+
+def test_gemm_with_strides_dense_in_neither_index(ctx):
+    """wdh_gemm called directly with operands that are contiguous in neither index (a view with a
+    step along both axes): the scalar kernel that follows the reference's loop order."""
+    m, n, k, batch = 37, 29, 53, 3
+    Abig, Bbig = uni(batch, m, 2 * k), uni(batch, k, 3 * n)   # A[b, i, 2x], B[b, x, 3j]
+    C, R = uni(m, 1), nrm(batch, m, n)
+    A, B = Abig[:, :, ::2], Bbig[:, :, ::3]
+    ta, tb, tc, tr = (ctx.move_tensor(v) for v in (Abig, Bbig, C, R))
+    y = ctx.empty_tensor([batch, m, n])
+    capi.call("wdh_gemm", ta.handle, tb.handle, tc.handle, y.handle, batch, m, n, k,
+              m * 2 * k, 2 * k, 2, k * 3 * n, 3 * n, 3, 1, 0, 0.75, 1.5, 1, tr.handle)
+    want = np.stack([ref.gemm(A[b], B[b], C, 0.75, 1.5) for b in range(batch)])
+    want = ref.unary("Relu", ref.binary("Add", want, R))
+    assert_close_max(y.get_data(), want, GEMM_TOL, "strided gemm")
+    # both operands transposed views with a step
+    At = np.ascontiguousarray(np.swapaxes(Abig, 1, 2))        # [b, 2k, m]
+    ta2 = ctx.move_tensor(At)
+    y2 = ctx.empty_tensor([batch, m, n])
+    capi.call("wdh_gemm", ta2.handle, tb.handle, 0, y2.handle, batch, m, n, k,
+              2 * k * m, 1, 2 * m, k * 3 * n, 3 * n, 3, 0, 0, 1.0, 1.0, 0, 0)
+    want2 = np.stack([ref.gemm(A[b], B[b]) for b in range(batch)])
+    assert_close_max(y2.get_data(), want2, GEMM_TOL, "strided gemm, A transposed")
+
+
+def test_gemm_operand_of_more_than_2_gib(ctx):
+    """A [528384, 1024] spans 2.16 GB: 32-bit byte offsets cannot address it, so the kernel takes
+    the flat-load loop.  The oracle runs on sampled rows."""
+    m, k, n = 528384, 1024, 64
+    rng = np.random.default_rng(7)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    ta, tb, tc = ctx.move_tensor(A), ctx.move_tensor(B), ctx.move_tensor(C)
+    y = H.gemm(ctx, ta, tb, tc)
+    got = y.get_data()
+    rows = np.concatenate([np.arange(0, 64), rng.integers(0, m, 192), np.arange(m - 64, m),
+                           np.arange(524288 - 8, 524288 + 8)])   # around the 2 GiB line of A
+    want = ref.gemm(A[rows], B, C)
+    assert_close_max(got[rows], want, GEMM_TOL, "2 GiB gemm, sampled rows")
+    # every row, against the BLAS product in double
+    full = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float32)
+    assert_close_max(got, full, GEMM_TOL, "2 GiB gemm, all rows vs float64 BLAS")
+    for t in (ta, tb, tc, y):
+        t.dispose()
+    capi.call("wdh_trim", 0)   # hand the 2 GiB block back to the driver
+
+
+HALO_CONVS = [
+    # n, cin, h, w, cout, pads, group: 3x3 stride 1, channels in blocks of 8 -> the LDS-tile kernel
+    (2, 8, 56, 56, 16, [1, 1, 1, 1], 1),       # 16-byte row pieces
+    (3, 16, 28, 28, 70, [1, 1, 1, 1], 1),      # 64-pixel tiles straddle images (784 each); two row tiles
+    (5, 24, 14, 14, 40, [1, 1, 1, 1], 1),      # 8-byte pieces
+    (7, 32, 7, 7, 33, [1, 1, 1, 1], 1),        # 4-byte pieces, a tile spans three images
+    (2, 8, 12, 20, 9, [0, 0, 0, 0], 1),        # no padding
+    (2, 16, 9, 12, 12, [2, 1, 0, 2], 1),       # unequal pads, wider than the kernel's reach
+    (1, 8, 5, 8, 8, [1, 1, 1, 1], 1),          # 40 pixels: a single partial tile
+    (2, 32, 10, 16, 24, [1, 1, 1, 1], 4),      # groups
+    (1, 64, 3, 3, 64, [1, 1, 1, 1], 1),        # plane smaller than the kernel's halo
+    (2, 8, 6, 120, 8, [1, 1, 1, 1], 1),        # rows too wide for the LDS tile: falls back to the gather
+    (33, 8, 2, 2, 8, [1, 1, 1, 1], 1),         # 4-pixel images: too many rows per tile, falls back
+]
+
+
+@pytest.mark.parametrize("shape", HALO_CONVS)
+def test_conv3x3_lds_tile_kernel(ctx, shape):
+    n, cin, h, w, cout, pads, group = shape
+    X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin // group, 3), nrm(cout)
+    want = ref.conv(X, W, B, None, group, None, pads, None)
+    R = nrm(*want.shape)
+    got = {}
+    for halo in (1, 0):
+        try:
+            ctx.set_option("conv3x3_halo", halo)
+            got[halo] = hip_conv(ctx, X, W, B, None, group, pads)
+            fused = hip_conv(ctx, X, W, B, None, group, pads, epilogue="relu", R=R)
+            for split in (2, 64):
+                ctx.set_option("split_k", split)
+                cut = hip_conv(ctx, X, W, B, None, group, pads)
+                ctx.set_option("split_k", -1)
+                assert_close_max(cut, want, GEMM_TOL, "halo %d split %d %s" % (halo, split, shape))
+        finally:
+            ctx.set_option("conv3x3_halo", 1)
+            ctx.set_option("split_k", -1)
+        assert_close_max(got[halo], want, GEMM_TOL, "halo %d %s" % (halo, shape))
+        assert_bit_exact(fused, np.maximum(got[halo] + R, 0) + 0.0, "halo %d + residual + relu" % halo)
+    assert_close_max(got[1], got[0], 1e-5, "LDS-tile form vs gathered form")

@@ -1146,6 +1146,7 @@ TileId pick_tile(int m, int n, int nz) {
 
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
+int g_descriptors = 1;    // 0: every operand is treated as if it spanned 2 GiB or more
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
 
 // How the tiles of one launch are spread over the chip.
@@ -1372,6 +1373,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     g_forced_split = value;
     return WDH_OK;
   }
+  if (strcmp(name, "descriptor_loads") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: descriptor_loads %d (use 0 or 1)", value);
+    g_descriptors = value;
+    return WDH_OK;
+  }
   if (strcmp(name, "conv3x3_halo") == 0) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: conv3x3_halo %d (use 0 or 1)", value);
@@ -1431,7 +1438,11 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   const bool b_kc = (sB0 == 1 || k == 1), b_mc = (sB1 == 1 || n == 1);
   if (!(a_kc || a_mc) || !(b_kc || b_mc) ||
       ((long long)(m + 63) / 64) * ((n + 63) / 64) > 0x7fffffffLL) {
-    dim3 grid((unsigned)(((long long)m * n + 255) / 256), (unsigned)batch);
+    const long long sblocks = ((long long)m * n + 255) / 256;
+    if (sblocks > 0x7fffffffLL)
+      return fail(WDH_EINVAL, "wdh_gemm: %lld x %lld results exceed the grid limit of the strided form",
+                  (long long)m, (long long)n);
+    dim3 grid((unsigned)sblocks, (unsigned)batch);
     hipLaunchKernelGGL(contraction_strided_kernel, grid, dim3(256), 0,
                        wdh::stream(), p);
     WDH_LAUNCH_CHECK();
@@ -1457,13 +1468,13 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   const long long a_bytes = k ? span(1, 0, m, p.sA0, k, p.sA1) * 4 : 0;
   const long long b_bytes = k ? span(1, 0, k, p.sB0, n, p.sB1) * 4 : 0;
   // (the margin covers the columns an edge tile reads past the matrix)
-  p.fast = a_bytes < 0x7fffffffLL - 4096 && b_bytes < 0x7fffffffLL - 4096;
+  p.fast = g_descriptors && a_bytes < 0x7fffffffLL - 4096 && b_bytes < 0x7fffffffLL - 4096;
   p.a_bytes = p.fast ? (int)a_bytes : 0;
   p.b_bytes = p.fast ? (int)b_bytes : 0;
   {
     const long long y_bytes = (long long)m * n * 4;
     const long long c_bytes = p.C ? span(1, 0, m, p.sC0, n, p.sC1) * 4 : 0;
-    const bool ok = y_bytes < 0x7fffffffLL && c_bytes < 0x7fffffffLL;
+    const bool ok = g_descriptors && y_bytes < 0x7fffffffLL && c_bytes < 0x7fffffffLL;
     p.y_bytes = ok ? (int)y_bytes : 0;
     p.c_bytes = ok ? (int)c_bytes : 0;
   }
@@ -1564,7 +1575,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   // by the top-left padding, and one group's weights) to stay below 2^31.
   const long long x_bytes = ((long long)n * c * h * w + (long long)pt * w + pl) * 4;
   const long long w_bytes = (long long)cout_g * kdim * 4;
-  const bool small = x_bytes < 0x7fffffffLL && w_bytes < 0x7fffffffLL;
+  const bool small = g_descriptors && x_bytes < 0x7fffffffLL && w_bytes < 0x7fffffffLL;
   const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
   // 1x1, stride 1, no padding: X is the B matrix as it lies (B_PIXELS), provided every tile
   // and K slab is whole; a forced tile may be up to 256 columns wide
@@ -1583,7 +1594,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.fast = 1;
     p.a_bytes = (int)w_bytes;
     p.b_bytes = (int)x_bytes;  // window of group 0; the kernel shortens it per group
-    p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+    p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
     p.c_bytes = cout * 4;
     return launch<true, B_PIXELS>(p, group, true);
   }
@@ -1604,7 +1615,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       p.fast = 1;
       p.a_bytes = (int)w_bytes;
       p.b_bytes = (int)((long long)n * c * h * w * 4);
-      p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+      p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
       p.c_bytes = cout * 4;
       if (bn == 128) return launch_halo_tile<64, 128, 1, 4>(p, group, vecw);
       return launch_halo_tile<64, 64, 2, 2>(p, group, vecw);
@@ -1665,7 +1676,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.a_bytes = small ? (int)w_bytes : 0;
   // a group's window runs from its first byte (shifted down by the padding) to the end of X
   p.b_bytes = small ? (int)x_bytes : 0;  // window of group 0; the kernel shortens it per group
-  p.y_bytes = out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
+  p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
   p.c_bytes = cout * 4;
   if (mode == B_IM2COL32) return launch<true, B_IM2COL32>(p, group, vec);
   if (mode == B_IM2COL64) return launch<true, B_IM2COL64>(p, group, vec);
