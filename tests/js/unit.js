@@ -320,6 +320,98 @@ test("load(): unknown backend throws, empty order has no backend, hip failure fa
   fs.rmdirSync(dir, { recursive: true });
 });
 
+test("runner: an operator that throws after allocating leaves no device buffer behind", async () => {
+  const WebDNN = require(path.join(JS, "index"));
+  const dir = fs.mkdtempSync(path.join(os.tmpdir(), "webdnn_unit_"));
+  writeReluModel(dir);
+  WebDNN.resetDefaultContexts();
+  table.clearOperators();
+  const runner = await WebDNN.load(dir, { backendOrder: ["hip", "cpu"], backendOptions: { hip: { native: fakeNative, strict: true } } });
+  // the Relu entry becomes one that allocates its output and two temporaries, then fails
+  // (the first matching entry wins, so the registry is rebuilt around it)
+  table.clearOperators();
+  table.registerOperators([{
+    opType: "Relu", backend: "hip", opsetMin: 1,
+    factory: () => ({
+      backend: "hip",
+      initialize() {},
+      getTensorBackendRequirement(nIn) { return new Array(nIn).fill("hip"); },
+      async run(context, inputs) {
+        context.emptyTensor(inputs[0].dims, "float32");
+        const tmp = context.emptyTensor([16], "float32");
+        tmp.dispose();
+        context.emptyTensor([3], "int32");
+        throw new Error("kernel refused");
+      },
+    }),
+  }]);
+  const live0 = fakeNative.__liveBuffers();
+  const x = new WebDNN.CPUTensor([5], "float32", new Float32Array([-2, -0.5, 0, 1, 3]));
+  await assert.rejects(() => runner.run([x]), /kernel refused/);
+  assert.strictEqual(fakeNative.__liveBuffers(), live0);
+  assert.strictEqual(runner.backendContexts.hip.tracked, null);
+  fs.rmdirSync(dir, { recursive: true });
+});
+
+test("runner: graph replays read runner-owned input buffers, never the caller's device tensors", async () => {
+  const WebDNN = require(path.join(JS, "index"));
+  const dir = fs.mkdtempSync(path.join(os.tmpdir(), "webdnn_unit_"));
+  writeReluModel(dir);
+  WebDNN.resetDefaultContexts();
+  table.clearOperators();
+  const runner = await WebDNN.load(dir, { backendOrder: ["hip", "cpu"], backendOptions: { hip: { native: fakeNative, strict: true } } });
+  const hip = runner.backendContexts.hip;
+  const A = await hip.moveTensor(new WebDNN.CPUTensor([5], "float32", new Float32Array([-2, -1, 0, 1, 2])), {});
+  const B = await hip.moveTensor(new WebDNN.CPUTensor([5], "float32", new Float32Array([5, -6, 7, -8, 9])), {});
+  const want = { A: [0, 0, 0, 1, 2], B: [5, 0, 7, 0, 9] };
+  const order = ["A", "A", "B", "A", "B", "B", "A"]; // eager, capture, replays
+  for (const which of order) {
+    const [y] = await runner.run([which === "A" ? A : B], { graph: true });
+    assert.deepStrictEqual(Array.from(y.data), want[which], `run with ${which}`);
+  }
+  assert.ok(runner.graphState && runner.graphState.inputs[0] !== A && runner.graphState.inputs[0] !== B);
+  // the caller's tensors are untouched and may be disposed while the graph lives on
+  assert.deepStrictEqual(Array.from(await A.getData()), [-2, -1, 0, 1, 2]);
+  assert.deepStrictEqual(Array.from(await B.getData()), [5, -6, 7, -8, 9]);
+  A.dispose();
+  const [y] = await runner.run([B], { graph: true });
+  assert.deepStrictEqual(Array.from(y.data), want.B);
+  // other shapes: the graph is dropped and the next run warms up eagerly before a new capture
+  assert.strictEqual(runner.graphWarm, true);
+  B.dispose();
+  runner.disposeGraph();
+  fs.rmdirSync(dir, { recursive: true });
+});
+
+test("runner: loading another model frees the device copies of the old initializers", async () => {
+  const WebDNN = require(path.join(JS, "index"));
+  const dir = fs.mkdtempSync(path.join(os.tmpdir(), "webdnn_unit_"));
+  const model = {
+    irVersion: 7, opsetImport: [{ domain: "", version: 13 }], metadataProps: [],
+    graph: {
+      name: "g", node: [{ input: ["x", "w"], output: ["y"], name: "a", opType: "Add", attribute: [] }],
+      initializer: [{ name: "w", dims: [5], dataType: 1, floatData: [1, 1, 1, 1, 1] }],
+      input: [{ name: "x", type: { tensorType: { elemType: 1, shape: { dim: [{ dimValue: 5 }] } } } }],
+      output: [{ name: "y", type: { tensorType: { elemType: 1, shape: { dim: [{ dimValue: 5 }] } } } }],
+      valueInfo: [],
+    },
+  };
+  fs.writeFileSync(path.join(dir, "model.onnx"), onnx.encodeModel(model));
+  WebDNN.resetDefaultContexts();
+  table.clearOperators();
+  const live0 = fakeNative.__liveBuffers();
+  const runner = await WebDNN.load(dir, { backendOrder: ["hip", "cpu"], backendOptions: { hip: { native: fakeNative, strict: true } } });
+  const x = new WebDNN.CPUTensor([5], "float32", new Float32Array([1, 2, 3, 4, 5]));
+  const [y] = await runner.run([x]);
+  assert.deepStrictEqual(Array.from(y.data), [2, 3, 4, 5, 6]);
+  assert.strictEqual(fakeNative.__liveBuffers(), live0 + 1); // the weight's device copy
+  await runner.loadModel(dir, "model.onnx");
+  assert.strictEqual(fakeNative.__liveBuffers(), live0);
+  const [y2] = await runner.run([x]);
+  assert.deepStrictEqual(Array.from(y2.data), [2, 3, 4, 5, 6]);
+  fs.rmdirSync(dir, { recursive: true });
+});
+
 (async () => {
   let passed = 0, failed = 0;
   for (const [name, fn] of tests) {

@@ -164,14 +164,14 @@ def test_optimized_model_directory(tmp_path):
     assert_close_max(got8[0], ref8[out_name], 1e-3, "8-bit coded weights")
 
 
-def _graph_runs(tmp_path, data, a, b, runs):
+def _graph_runs(tmp_path, data, a, b, runs, resident=False):
     alt = []
     for i, arr in enumerate(b):
         p = tmp_path / ("alt_%d.bin" % i)
         np.ascontiguousarray(arr).tofile(str(p))
         alt.append(str(p))
     return node_runner.run_model(str(tmp_path), a, "hip", strict=True, runs=runs,
-                                 extra=["--graph", "--alt-inputs", ",".join(alt)])
+                                 extra=["--graph", "--alt-inputs", ",".join(alt)] + (["--resident-inputs"] if resident else []))
 
 
 def test_graph_replay_equals_eager_runs(tmp_path):
@@ -189,6 +189,24 @@ def test_graph_replay_equals_eager_runs(tmp_path):
         assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
         assert rep["stats"]["graphReplay"] is True
         assert_bit_exact(got[0], want[0], "run %d of a graph-mode session" % runs)
+
+
+def test_graph_replay_with_two_resident_device_inputs(tmp_path):
+    """The caller hands over tensors that already live on the device and alternates between two of
+    them: run(A) eager, run(B) captured, then A, B, A ... replayed.  The graph reads from buffers of
+    its own, so every run must equal the eager run of the tensor it was given, and the caller's
+    tensors must come through unchanged (the last run reads A or B again after several replays)."""
+    data, _ = modelgen.resnet50_model(batch=4, image=64, width=16, blocks=(1, 1, 1, 1), classes=10)
+    Xa = np.random.default_rng(12).standard_normal((4, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(13).standard_normal((4, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    ea, _ = node_runner.run_model(str(tmp_path), [Xa], "hip", strict=True)
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True)
+    assert np.abs(ea[0] - eb[0]).max() > 0
+    for runs, want in ((2, eb), (3, ea), (4, eb), (5, ea), (8, eb)):
+        got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs, resident=True)
+        assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
+        assert_bit_exact(got[0], want[0], "run %d with resident inputs" % runs)
 
 
 def test_graph_replay_detr_style(tmp_path):

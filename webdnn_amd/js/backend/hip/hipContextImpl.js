@@ -17,6 +17,7 @@ class WebDNNHipContextImpl {
     this.option = option || {};
     this.native = null;
     this.initialized = false;
+    this.tracked = null;
   }
 
   // Throws when the addon, the library or the GPU is missing; load() then skips
@@ -45,7 +46,25 @@ class WebDNNHipContextImpl {
   }
 
   emptyTensor(dims, dataType) {
-    return new HipTensorImpl(this, dims, dataType);
+    const t = new HipTensorImpl(this, dims, dataType);
+    if (this.tracked) this.tracked.push(t);
+    return t;
+  }
+
+  // The runner brackets every operator.run with trackAllocations / stopTracking; when the
+  // operator throws, releaseTracked frees what it had allocated (its outputs and
+  // temporaries), which nobody else holds a reference to.
+  trackAllocations() {
+    this.tracked = [];
+  }
+
+  releaseTracked() {
+    for (const t of this.tracked || []) t.dispose();
+    this.tracked = null;
+  }
+
+  stopTracking() {
+    this.tracked = null;
   }
 
   // eslint-disable-next-line no-unused-vars

@@ -98,10 +98,15 @@ async function main() {
   const altInputs = args.altInputs ? readInputs(args.altInputs) : null;
 
   // --resident-inputs: upload the inputs once; the timed runs then start with their data in HBM
-  let runInputs = inputs;
+  let runInputs = inputs,
+    runAltInputs = altInputs;
   if (args.residentInputs && runner.backendName === "hip") {
     runInputs = [];
     for (const t of inputs) runInputs.push(await runner.backendContexts.hip.moveTensor(t, {}));
+    if (altInputs) {
+      runAltInputs = [];
+      for (const t of altInputs) runAltInputs.push(await runner.backendContexts.hip.moveTensor(t, {}));
+    }
     runner.backendContexts.hip.sync();
   }
   for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, { graph: !!args.graph });
@@ -127,7 +132,7 @@ async function main() {
       queueAhead = { launches: reps, tensors: [a, b] };
     }
     const t0 = process.hrtime.bigint();
-    outputs = await runner.run(altInputs && i % 2 === 1 ? altInputs : runInputs,
+    outputs = await runner.run(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs,
       { measurePerformance: !!args.measureAll || (!!args.measure && i === args.runs - 1), graph: !!args.graph });
     times.push(Number(process.hrtime.bigint() - t0) / 1e6);
     // --measure-all: device time of every timed run (HIP events on the library's stream; a replayed

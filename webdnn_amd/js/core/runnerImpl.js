@@ -44,6 +44,7 @@ class RunnerImpl {
     this.graphState = null;
     this.graphWarm = false;
     this.graphUnsupported = null; // reason, once a capture has failed for this model
+    this.graphRetries = 0; // captures given up for a reason an eager run cures
     // Operator instances by node and by where its inputs live.  The reference builds
     // and initializes a new instance per node per run (runnerImpl.ts:441-452);
     // instances here keep no state beyond their attributes, so later runs reuse them.
@@ -54,6 +55,7 @@ class RunnerImpl {
     this.disposeGraph();
     this.graphWarm = false;
     this.graphUnsupported = null;
+    this.graphRetries = 0;
     const bytes = fs.readFileSync(path.join(directory, onnxBasename));
     this.loadModelFromBytes(bytes, directory);
   }
@@ -74,6 +76,9 @@ class RunnerImpl {
     }
     for (const [name, tensor] of this.loadExternalInitializerTensor(directory).entries()) {
       this.initializerTensors.set(name, tensor);
+    }
+    for (const kv of (this.copiedInitializerTensors || new Map()).values()) {
+      for (const t of kv.values()) t.dispose();
     }
     this.copiedInitializerTensors = new Map();
     for (const backend of this.backendOrder) {
@@ -166,22 +171,33 @@ class RunnerImpl {
       cpu = this.backendContexts.cpu;
     if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
     const signature = inputs.map((t) => `${t.dataType}[${t.dims.join(",")}]`).join(";");
-    if (this.graphState && this.graphState.signature !== signature) this.disposeGraph();
+    if (this.graphState && this.graphState.signature !== signature) {
+      // other shapes: other buffers, maybe conv geometries not seen yet -- warm up again
+      this.disposeGraph();
+      this.graphWarm = false;
+    }
     if (!this.graphState) {
       if (!this.graphWarm) {
         this.graphWarm = true;
         return this.runEager(inputs, opts);
       }
-      const graphInputs = [],
-        ownedInputs = [];
-      for (const t of inputs) {
-        if (t.backend === "hip") {
-          graphInputs.push(t);
-        } else {
-          const moved = await hip.moveTensor(t, {});
-          graphInputs.push(moved);
-          ownedInputs.push(moved);
+      // The graph reads its inputs from buffers the runner owns: a caller's device tensor
+      // is copied in like a host tensor is uploaded, so the caller may overwrite or dispose
+      // it afterwards and later replays never write into caller memory.
+      const graphInputs = [];
+      try {
+        for (const t of inputs) {
+          if (t.backend === "hip") {
+            const own = hip.emptyTensor(t.dims, t.dataType);
+            graphInputs.push(own);
+            hip.native.copy(own.handle, 0, t.handle, 0, own.length * 4);
+          } else {
+            graphInputs.push(await hip.moveTensor(t, {}));
+          }
         }
+      } catch (error) {
+        for (const t of graphInputs) t.dispose();
+        throw error;
       }
       let outputs = null,
         failure = null;
@@ -200,18 +216,25 @@ class RunnerImpl {
       if (failure) {
         if (id >= 0) hip.native.graphDestroy(id);
         for (const t of outputs || []) if (t.backend === "hip") t.dispose();
-        for (const t of ownedInputs) t.dispose();
-        this.graphUnsupported = failure.message;
+        for (const t of graphInputs) t.dispose();
+        // A geometry met for the first time while recording (its tables need a blocking
+        // copy) is cured by the eager run below; anything else will fail the same way again.
+        const transient = /run it once before capturing/.test(failure.message) && this.graphRetries < 3;
+        if (transient) {
+          this.graphRetries++;
+        } else {
+          this.graphUnsupported = failure.message;
+        }
         logger.warn(`run could not be captured into a graph (${failure.message}); running eagerly`);
         return this.runEager(inputs, opts);
       }
-      this.graphState = { id, inputs: graphInputs, ownedInputs, outputs, signature, stats: this.lastRunStats };
+      this.graphRetries = 0;
+      this.graphState = { id, inputs: graphInputs, ownedInputs: graphInputs, outputs, signature, stats: this.lastRunStats };
     } else {
       const state = this.graphState;
       for (let i = 0; i < inputs.length; i++) {
         const src = inputs[i],
           dst = state.inputs[i];
-        if (src === dst) continue;
         if (src.backend === "hip") hip.native.copy(dst.handle, 0, src.handle, 0, dst.length * 4);
         else await dst.setData(await src.getData());
       }
@@ -343,7 +366,17 @@ class RunnerImpl {
             // one event per node boundary: node i's device time runs from event i to event i+1
             // (every event costs the stream a small bubble, so as few as possible)
             if (useEvents) hip.native.eventRecord(i);
-            const operatorOutputs = await operator.run(context, operatorInputs, node.output.length);
+            // tensors an operator allocates before it throws would otherwise never be freed
+            if (context.trackAllocations) context.trackAllocations();
+            let operatorOutputs;
+            try {
+              operatorOutputs = await operator.run(context, operatorInputs, node.output.length);
+            } catch (error) {
+              if (context.releaseTracked) context.releaseTracked();
+              throw error;
+            } finally {
+              if (context.stopTracking) context.stopTracking();
+            }
             actualInputDims = operatorInputs.map((t) => t.dims);
             actualOutputDims = operatorOutputs.map((t) => t.dims);
             for (let j = 0; j < node.output.length; j++) {
