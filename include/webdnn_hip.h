@@ -168,6 +168,26 @@ int wdh_gemm(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
              int64_t sB0, int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
              float beta, int epilogue, wdh_buf R);
 
+/* wdh_gemm for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results as wdh_gemm; the one difference is where the partial sums of tiles cut
+ * along K live: in a workspace of WDH_STATIC_SCRATCH_BYTES inside the library's
+ * own device image (one copy per GPU, held until the process ends) instead of a
+ * block from the pool.  The call performs no hipMalloc / hipFree and takes nothing
+ * from the pool.  A problem whose plan needs more workspace than that fails with
+ * WDH_EINVAL and touches nothing (wdh_set_option("split_k", 1) makes every size fit:
+ * unsplit launches use no workspace).  All calls on a GPU share the one workspace,
+ * which keeps the previous call's contents: the kernels write every partial sum
+ * they later read, so nothing has to be cleared, but two such calls that overlap
+ * on one GPU (other streams, other threads) race; the library's single stream
+ * orders them. */
+#define WDH_STATIC_SCRATCH_BYTES (16u << 20)
+int wdh_gemm_static(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
+                    int n, int k, int64_t sAb, int64_t sA0, int64_t sA1,
+                    int64_t sBb, int64_t sB0, int64_t sB1, int64_t sC0,
+                    int64_t sC1, float alpha, float beta, int epilogue, wdh_buf R);
+
 /* ---- Conv (2-D, NCHW) ------------------------------------------------
  * Replaces CpuConv.run = im2col + matmul + transpose + bias
  * (operators/cpu/operators/standard/conv.ts:134-333) and the four WebGPU

@@ -18,6 +18,10 @@ bool capturing();        // a graph capture is open on the stream
 void poison_capture();   // the open capture cannot be completed (wdh_graph_end will fail)
 hipStream_t stream();
 int compute_units();
+int device();           // the device wdh_init selected
+// Looks up the device address of the static workspace of wdh_gemm_static for `device`,
+// which must be the current device (called by wdh_init).
+int init_static_scratch(int device);
 
 // Handle -> device pointer.  Returns nullptr (and records WDH_EINVAL) for an
 // unknown handle.  A zero-byte buffer resolves to a non-null dummy pointer.

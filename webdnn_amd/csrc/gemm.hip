@@ -59,6 +59,36 @@
 
 #include "common.h"
 
+// Workspace of wdh_gemm_static: the partial sums of tiles cut along K, held in the
+// library's own image instead of pool memory so that the call allocates nothing.
+// Every GPU the library runs on holds one copy until the process ends.
+#define WDH_STATIC_SCRATCH_FLOATS (4u << 20) /* 16 MiB */
+static __device__ __align__(256) float scratch[WDH_STATIC_SCRATCH_FLOATS];
+static_assert(sizeof(float) * WDH_STATIC_SCRATCH_FLOATS == WDH_STATIC_SCRATCH_BYTES,
+              "the header states the workspace size");
+// In host code `scratch` is only a stand-in for the symbol: the array's device address is
+// looked up once per device (wdh_init, with that device current) and kept here.
+constexpr int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices] = {};
+
+namespace wdh {
+int init_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    return fail(WDH_ENODEV, "wdh_init: device %d beyond the %d this library keeps a workspace for",
+                device, kMaxDevices);
+  if (g_scratch_ptr[device]) return WDH_OK;
+  float *ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) {
+    (void)hipGetLastError();
+    return fail(WDH_EHIP, "wdh_init: address of the static workspace on device %d: %s", device,
+                e == hipSuccess ? "null" : hipGetErrorString(e));
+  }
+  g_scratch_ptr[device] = ptr;
+  return WDH_OK;
+}
+}  // namespace wdh
+
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1147,6 +1177,7 @@ TileId pick_tile(int m, int n, int nz) {
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
 int g_descriptors = 1;    // 0: every operand is treated as if it spanned 2 GiB or more
+bool g_static_scratch = false;  // set for the duration of a wdh_gemm_static call
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
 
 // How the tiles of one launch are spread over the chip.
@@ -1255,11 +1286,25 @@ int launch_planned(Params &p, int nz, bool conv, int kgran, Start start) {
   p.fd_tail_tiles = make_fastdiv(w.tail > 0 ? w.tail : 1);
   p.fd_group = make_fastdiv((long long)TILE_GROUP * p.tiles_n);
   p.fd_last_rows = make_fastdiv(p.tiles_m % TILE_GROUP ? p.tiles_m % TILE_GROUP : 1);
-  wdh_buf scratch = 0;
+  wdh_buf pooled = 0;
   if (w.tail > 0) {
-    scratch = wdh_alloc((size_t)w.tail * w.split * BM * BN * sizeof(float));
-    if (!scratch) return WDH_ENOMEM;
-    p.partial = (float *)wdh::resolve(scratch, nullptr);
+    const size_t need = (size_t)w.tail * w.split * BM * BN * sizeof(float);
+    if (g_static_scratch) {
+      // the caller cannot allocate: the chunks' sums go to the library's static workspace,
+      // through its device address (every element a reduce pass reads is written first by
+      // the launch before it, so nothing has to be cleared between calls)
+      if (need > WDH_STATIC_SCRATCH_BYTES)
+        return wdh::fail(WDH_EINVAL,
+                         "wdh_gemm_static: this problem is cut into %lld x %d partial tiles of %d x %d, "
+                         "%zu bytes; the static workspace holds %zu (set split_k to 1 to run it unsplit)",
+                         w.tail, w.split, BM, BN, need, (size_t)WDH_STATIC_SCRATCH_BYTES);
+      p.partial = g_scratch_ptr[wdh::device()];
+      if (!p.partial) return wdh::fail(WDH_ESTATE, "wdh_gemm_static: no static workspace on device %d", wdh::device());
+    } else {
+      pooled = wdh_alloc(need);
+      if (!pooled) return WDH_ENOMEM;
+      p.partial = (float *)wdh::resolve(pooled, nullptr);
+    }
   }
   start(dim3((unsigned)blocks));
   hipError_t e = hipGetLastError();
@@ -1275,7 +1320,7 @@ int launch_planned(Params &p, int nz, bool conv, int kgran, Start start) {
   }
   // The scratch block goes back to the pool right away: whoever gets it next
   // touches it through the same stream, behind the two kernels above.
-  if (scratch) (void)wdh_free(scratch);
+  if (pooled) (void)wdh_free(pooled);
   if (e != hipSuccess)
     return wdh::fail(WDH_EHIP, "contraction launch failed: %s", hipGetErrorString(e));
   return WDH_OK;
@@ -1386,6 +1431,19 @@ extern "C" int wdh_set_option(const char *name, int value) {
     return WDH_OK;
   }
   return fail(WDH_EINVAL, "wdh_set_option: unknown option \"%s\"", name);
+}
+
+extern "C" int wdh_gemm_static(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
+                               int batch, int m, int n, int k, int64_t sAb,
+                               int64_t sA0, int64_t sA1, int64_t sBb, int64_t sB0,
+                               int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
+                               float beta, int epilogue, wdh_buf hR) {
+  WDH_REQUIRE_INIT();
+  g_static_scratch = true;
+  const int rc = wdh_gemm(hA, hB, hC, hY, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1,
+                          alpha, beta, epilogue, hR);
+  g_static_scratch = false;
+  return rc;
 }
 
 extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,

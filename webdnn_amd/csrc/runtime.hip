@@ -119,6 +119,7 @@ bool capturing() { return g.capturing != 0; }
 void poison_capture() { g.capture_failed = true; }
 hipStream_t stream() { return g.stream; }
 int compute_units() { return g.prop.multiProcessorCount; }
+int device() { return g.device; }
 
 void *resolve(wdh_buf h, size_t *bytes) {
   if (h <= 0 || (size_t)h > g.slots.size() || g.slots[h - 1].ptr == nullptr) {
@@ -188,6 +189,10 @@ int wdh_init(int device) {
     g.stage_busy[i] = false;
   }
   WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
+  {
+    const int rc = wdh::init_static_scratch(device);
+    if (rc != WDH_OK) return rc;
+  }
   g.device = device;
   g.ready = true;
   wdh::clear_error();
