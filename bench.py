@@ -85,14 +85,18 @@ def bench_resnet(steps, warmup, workdir):
                          if p["opType"] in ("Conv", "WebDNNHipFusedConv", "Gemm"))
     launches = sum(1 for p in prof["performance"] if p["opType"] in ("Conv", "WebDNNHipFusedConv", "Gemm"))
     all_ms = sum(p["deviceElapsed"] or 0.0 for p in prof["performance"])
-    # PCIe-inclusive: the input is a host tensor, uploaded by the run
+    # PCIe-inclusive: the input is a host tensor (runner.run([CPUTensor]), as in the reference), uploaded
+    # by every run: 19.3 MB through the pinned staging buffers, then the same graph replay / node loop
     host_in = node_run(workdir, inp, "hip", max(3, steps // 4), 2, ["--strict"])
+    host_in_graph = node_run(workdir, inp, "hip", steps, max(warmup, 2), ["--strict", "--graph"])
+    assert host_in_graph["graph"]["captured"], host_in_graph["graph"]
     return {
         "batch": batch, "flops": g.flops, "nodes": timed["nodes"], "ms_per_step": total_ms / steps,
         "images_per_s": batch * steps / total_ms * 1e3, "contraction_ms": contraction_ms,
         "contraction_launches": launches, "device_ms": all_ms,
         "graph_device_ms": sum(timed["deviceMsPerRun"]) / len(timed["deviceMsPerRun"]),
         "images_per_s_host_input": batch / (sum(host_in["msPerRun"]) / len(host_in["msPerRun"])) * 1e3,
+        "ms_per_step_host_input_graph": sum(host_in_graph["msPerRun"]) / len(host_in_graph["msPerRun"]),
         "ms_per_step_eager": sum(eager["msPerRun"]) / len(eager["msPerRun"]),
         "device": timed.get("device"), "node_version": timed["node"],
     }
@@ -115,15 +119,21 @@ def bench_report_only(workdir, steps, warmup):
             f.write(data)
         inp = os.path.join(d, "input.bin")
         np.random.default_rng(11).standard_normal(shape).astype(np.float32).tofile(inp)
-        rep = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--graph"])
+        rep = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--graph", "--measure-all"])
         assert list(rep["stats"]["nodesByBackend"]) == ["hip"], rep["stats"]
         ms = sum(rep["msPerRun"]) / len(rep["msPerRun"])
+        dev_ms = sum(rep["deviceMsPerRun"]) / len(rep["deviceMsPerRun"])
         eager = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs"])
         out[key] = {"workload": label, "nodes": rep["nodes"], "ms_per_run": round(ms, 4),
                     "graph_replay": bool(rep["graph"]["captured"]),
                     "ms_per_run_eager": round(sum(eager["msPerRun"]) / len(eager["msPerRun"]), 4),
                     "gflops": round(g.flops / ms / 1e6, 1),
-                    "frac_mfma_peak": round(g.flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
+                    "frac_mfma_peak": round(g.flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+                    # device time of a replay (HIP events around the graph launch): the kernels alone,
+                    # without the input upload, the output download and the host's share of runner.run
+                    "device_ms": round(dev_ms, 4),
+                    "device_gflops": round(g.flops / dev_ms / 1e6, 1),
+                    "device_frac_mfma_peak": round(g.flops / dev_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
     return out
 
 
@@ -198,6 +208,91 @@ def bench_kernels(steps, warmup, calibrate_copy=False):
     }
 
 
+def bench_resnet_layers(steps, warmup, batch=32):
+    """Every distinct Conv / Gemm launch of the ResNet-50 step, through the C ABI with back-to-back
+    launches (operands hot in the caches, unlike inside the graph): shape, how often the step runs
+    it, microseconds, TFLOP/s, and how the launch was laid out (tile, whole / K-split tiles, form)."""
+    from webdnn_amd import hostops as H
+    from webdnn_amd import modelgen
+
+    ctx = H.HipContext(0).initialize()
+    rng = np.random.default_rng(0)
+    data, _ = modelgen.resnet50_model(batch=batch)
+    model = modelgen.parse_model(data)
+    shapes = {name: list(dims) for name, dims in model["inputs"]}
+    shapes.update({name: list(a.shape) for name, a in model["initializers"].items()})
+    consumers = {}
+    for nd in model["nodes"]:
+        for i in nd["inputs"]:
+            consumers.setdefault(i, []).append(nd)
+    layers = {}
+    for nd in model["nodes"]:
+        ins, out = nd["inputs"], nd["outputs"][0]
+        if nd["op_type"] == "Conv":
+            x, w = shapes[ins[0]], shapes[ins[1]]
+            a = nd["attrs"]
+            s = H.conv_shape(x, w, a.get("dilations"), a.get("group", 1), a.get("kernel_shape"), a.get("pads"),
+                             a.get("strides"))
+            shapes[out] = [x[0], w[0], s["out_shape"][0], s["out_shape"][1]]
+            nxt = consumers.get(out, [])
+            residual = len(nxt) == 1 and nxt[0]["op_type"] == "Add"      # what the fusion pass absorbs
+            key = (tuple(x), tuple(w), tuple(s["pads"]), tuple(s["strides"]), residual)
+            layers.setdefault(key, {"count": 0, "kind": "Conv"})["count"] += 1
+        elif nd["op_type"] == "Gemm":
+            key = (tuple(shapes[ins[0]]), tuple(shapes[ins[1]]), (), (), False)
+            layers.setdefault(key, {"count": 0, "kind": "Gemm"})["count"] += 1
+            shapes[out] = [shapes[ins[0]][0], shapes[ins[1]][0]]
+        elif nd["op_type"] in ("Relu", "Add"):
+            shapes[out] = shapes[ins[0]]
+        elif nd["op_type"] == "MaxPool":
+            a = nd["attrs"]
+            x = shapes[ins[0]]
+            s = H.maxpool_shape(x, a["kernel_shape"], pads=a.get("pads"), strides=a.get("strides"))
+            shapes[out] = [x[0], x[1], s["out_shape"][0], s["out_shape"][1]]
+        elif nd["op_type"] == "GlobalAveragePool":
+            shapes[out] = shapes[ins[0]][:2] + [1, 1]
+        elif nd["op_type"] == "Flatten":
+            shapes[out] = [shapes[ins[0]][0], int(np.prod(shapes[ins[0]][1:]))]
+    rows = []
+    for (x, w, pads, strides, residual), info in layers.items():
+        if info["kind"] == "Conv":
+            X = ctx.move_tensor(rng.uniform(0, 1, x).astype(np.float32))
+            W = ctx.move_tensor((rng.standard_normal(w) * np.sqrt(2.0 / (w[1] * w[2] * w[3]))).astype(np.float32))
+            B = ctx.move_tensor(np.zeros(w[0], np.float32))
+            probe = H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu")
+            plan, odims = ctx.last_plan(), probe.dims
+            R = ctx.move_tensor(rng.uniform(0, 1, odims).astype(np.float32)) if residual else None
+            probe.dispose()
+            ms = timed_steps(ctx, lambda: H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu",
+                                                 residual=R).dispose(), steps, warmup)
+            m, n, k = w[0], odims[0] * odims[2] * odims[3], w[1] * w[2] * w[3]
+            label = "Conv %dx%d s%d %d->%d @%dx%d%s" % (w[2], w[3], strides[0], x[1], w[0], x[2], x[3],
+                                                         " +residual" if residual else "")
+            for t in (X, W, B) + ((R,) if R is not None else ()):
+                t.dispose()
+        else:
+            A = ctx.move_tensor(rng.standard_normal(x).astype(np.float32))
+            Wt = ctx.move_tensor((rng.standard_normal(w) * 0.01).astype(np.float32))
+            Bv = ctx.move_tensor(np.zeros(w[0], np.float32))
+            H.gemm(ctx, A, Wt, Bv, trans_b=1).dispose()
+            plan = ctx.last_plan()
+            ms = timed_steps(ctx, lambda: H.gemm(ctx, A, Wt, Bv, trans_b=1).dispose(), steps, warmup)
+            m, n, k = x[0], w[0], x[1]
+            label = "Gemm [%d,%d] x [%d,%d]^T" % (x[0], x[1], w[0], w[1])
+            for t in (A, Wt, Bv):
+                t.dispose()
+        flops = 2.0 * m * n * k
+        rows.append({"layer": label, "count": info["count"], "m": m, "n": n, "k": k, "us": round(ms * 1e3, 1),
+                     "tflops": round(flops / ms / 1e9, 1),
+                     "frac_mfma_peak": round(flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 3), **plan})
+    total_us = sum(r["us"] * r["count"] for r in rows)
+    total_flops = sum(2.0 * r["m"] * r["n"] * r["k"] * r["count"] for r in rows)
+    return {"note": "back-to-back launches of each distinct layer with its fused bias/residual/Relu epilogue and "
+                    "its K-split reduce pass; us = HIP events / launches",
+            "launches": sum(r["count"] for r in rows), "sum_us": round(total_us, 1),
+            "tflops": round(total_flops / total_us / 1e6, 1), "layers": rows}
+
+
 def bench_bandwidth(steps, warmup):
     """GB/s of the HBM-bound kernels at the shapes the configs use: algorithmic bytes (every input and
     output element once) over the average launch time, against the 8 TB/s peak."""
@@ -257,7 +352,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "kernels", "bandwidth"], default="all",
+    ap.add_argument("--only", choices=["all", "kernels", "bandwidth", "layers"], default="all",
                     help="kernels: only the in-process Gemm 4096 / Conv C3 launches plus one device-to-device "
                          "copy of known size (the unit for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
@@ -269,6 +364,9 @@ def main():
         print(json.dumps({"bandwidth_kernels": bench_bandwidth(args.steps, args.warmup),
                           "unit": "GB/s of algorithmic bytes", "peak": 8000.0}))
         return
+    if args.only == "layers":
+        print(json.dumps({"resnet50_layers": bench_resnet_layers(args.steps, args.warmup)}))
+        return
     if args.only == "kernels":
         print(json.dumps({"kernels": bench_kernels(args.steps, args.warmup, calibrate_copy=True)}))
         return
@@ -279,6 +377,7 @@ def main():
         baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
     kernels = bench_kernels(args.steps, args.warmup)
     bandwidth = bench_bandwidth(args.steps, args.warmup)
+    layers = bench_resnet_layers(args.steps, min(args.warmup, 5))
 
     # The timed steps are graph replays: one HIP event pair brackets each replay on the library's
     # stream.  That device time covers the 54 contraction launches with their reduce passes plus the
@@ -332,6 +431,12 @@ def main():
             "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
             "resnet50_ms_per_step_eager": round(resnet["ms_per_step_eager"], 4),
             "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),
+            "resnet50_host_input_graph": {
+                "note": "the same step with the batch handed over as a host tensor on every run "
+                        "(runner.run([CPUTensor]), 19.3 MB over PCIe inside the timed region), graph replay",
+                "ms_per_step": round(resnet["ms_per_step_host_input_graph"], 4),
+                "images_per_s": round(resnet["batch"] / resnet["ms_per_step_host_input_graph"] * 1e3, 1)},
+            "resnet50_layers": layers,
             "device": resnet["device"],
         },
     }

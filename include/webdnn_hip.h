@@ -86,6 +86,21 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       on ordinary sizes. */
 int wdh_set_option(const char *name, int value);
 
+/* How the most recent wdh_gemm / wdh_conv2d launch was laid out (for per-layer
+ * reports; cf. the per-node records of measurePerformance,
+ * core/runnerImpl.ts:533-541): workgroup tile, the number of tiles computed whole
+ * and of tiles cut along K, chunks per cut tile (1 = none), and which form of the
+ * kernel ran: WDH_FORM_* below.  Any pointer may be NULL. */
+#define WDH_FORM_GEMM_KC 0        /* B k-contiguous (transB)                    */
+#define WDH_FORM_GEMM_MC 1        /* B n-contiguous                             */
+#define WDH_FORM_CONV_GATHER32 2  /* taps gathered from X, at most 31 taps      */
+#define WDH_FORM_CONV_GATHER64 3  /* ... 32 to 63 taps                          */
+#define WDH_FORM_CONV_GATHER_FLAT 4 /* ... more taps or X of 2 GiB or more      */
+#define WDH_FORM_CONV_PIXELS 5    /* 1x1 stride 1: X read in place              */
+#define WDH_FORM_CONV3X3_LDS 6    /* 3x3 stride 1: taps read from an LDS tile   */
+int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles,
+                  int64_t *split_tiles, int *split, int *form);
+
 /* ---- buffers --------------------------------------------------------- */
 
 /* Replaces the `alloc` message, wasmContextImpl.ts:128-134 and

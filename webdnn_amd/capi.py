@@ -26,6 +26,8 @@ SIGNATURES = {
     "wdh_device_info": (_c.c_int, [_c.c_char_p, _c.c_int, _c.POINTER(_c.c_int),
                                    _c.POINTER(_c.c_int), _u64p]),
     "wdh_set_option": (_c.c_int, [_c.c_char_p, _c.c_int]),
+    "wdh_last_plan": (_c.c_int, [_c.POINTER(_c.c_int), _c.POINTER(_c.c_int), _i64p, _i64p,
+                                 _c.POINTER(_c.c_int), _c.POINTER(_c.c_int)]),
     "wdh_alloc": (c_buf, [_c.c_size_t]),
     "wdh_free": (_c.c_int, [c_buf]),
     "wdh_write": (_c.c_int, [c_buf, _c.c_size_t, _c.c_void_p, _c.c_size_t]),

@@ -1177,6 +1177,9 @@ TileId pick_tile(int m, int n, int nz) {
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
 int g_descriptors = 1;    // 0: every operand is treated as if it spanned 2 GiB or more
+// what launch_planned decided for the most recent launch (wdh_last_plan)
+struct LastPlan { int bm, bn, split, form; long long full, tail; } g_last_plan = {};
+int g_last_form = 0;
 bool g_static_scratch = false;  // set for the duration of a wdh_gemm_static call
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
 
@@ -1282,6 +1285,7 @@ int launch_planned(Params &p, int nz, bool conv, int kgran, Start start) {
   p.tail_tiles = (int)w.tail;
   p.tail_split = w.split;
   p.kchunk = w.kchunk;
+  g_last_plan = {BM, BN, w.split, g_last_form, w.full, w.tail};
   p.fd_tiles_per_z = make_fastdiv((long long)p.tiles_m * p.tiles_n);
   p.fd_tail_tiles = make_fastdiv(w.tail > 0 ? w.tail : 1);
   p.fd_group = make_fastdiv((long long)TILE_GROUP * p.tiles_n);
@@ -1328,6 +1332,7 @@ int launch_planned(Params &p, int nz, bool conv, int kgran, Start start) {
 
 template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE>
 int launch_tile(Params &p, int nz, bool vec) {
+  g_last_form = BMODE;
   return launch_planned<BM, BN>(p, nz, BMODE >= B_IM2COL32, BK, [&](dim3 grid) {
     if (vec)
       hipLaunchKernelGGL((contraction_kernel<BM, BN, WM, WN, A_KC, BMODE, true>), grid,
@@ -1340,6 +1345,7 @@ int launch_tile(Params &p, int nz, bool vec) {
 
 template <int BM, int BN, int WM, int WN>
 int launch_halo_tile(Params &p, int nz, int vecw) {
+  g_last_form = WDH_FORM_CONV3X3_LDS;
   return launch_planned<BM, BN>(p, nz, true, HALO_KB, [&](dim3 grid) {
     if (vecw == 4)
       hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4>), grid, dim3(NTHREADS), 0,
@@ -1431,6 +1437,17 @@ extern "C" int wdh_set_option(const char *name, int value) {
     return WDH_OK;
   }
   return fail(WDH_EINVAL, "wdh_set_option: unknown option \"%s\"", name);
+}
+
+extern "C" int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles, int64_t *split_tiles,
+                             int *split, int *form) {
+  if (tile_m) *tile_m = g_last_plan.bm;
+  if (tile_n) *tile_n = g_last_plan.bn;
+  if (whole_tiles) *whole_tiles = g_last_plan.full;
+  if (split_tiles) *split_tiles = g_last_plan.tail;
+  if (split) *split = g_last_plan.split;
+  if (form) *form = g_last_plan.form;
+  return WDH_OK;
 }
 
 extern "C" int wdh_gemm_static(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,

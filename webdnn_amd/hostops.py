@@ -152,6 +152,18 @@ class HipContext:
     def set_option(self, name, value):
         call("wdh_set_option", name.encode(), int(value))
 
+    FORMS = ("gemm, B k-contiguous", "gemm, B n-contiguous", "conv, gathered taps", "conv, gathered taps (32-63)",
+             "conv, gathered taps (flat loads)", "conv 1x1, X in place", "conv 3x3, LDS tile")
+
+    def last_plan(self):
+        """Layout of the most recent Gemm / Conv launch: tile, whole tiles, tiles cut along K, chunks, form."""
+        bm, bn, split, form = (ctypes.c_int() for _ in range(4))
+        whole, cut = ctypes.c_int64(), ctypes.c_int64()
+        call("wdh_last_plan", ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(whole), ctypes.byref(cut),
+             ctypes.byref(split), ctypes.byref(form))
+        return {"tile": "%dx%d" % (bm.value, bn.value), "whole_tiles": whole.value, "split_tiles": cut.value,
+                "split": split.value, "form": self.FORMS[form.value]}
+
     def empty_tensor(self, dims, data_type="float32"):
         return HipTensor(self, dims, data_type)
 
