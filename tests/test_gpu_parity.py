@@ -936,3 +936,23 @@ def test_conv3x3_lds_tile_kernel(ctx, shape):
         assert_close_max(got[halo], want, GEMM_TOL, "halo %d %s" % (halo, shape))
         assert_bit_exact(fused, np.maximum(got[halo] + R, 0) + 0.0, "halo %d + residual + relu" % halo)
     assert_close_max(got[1], got[0], 1e-5, "LDS-tile form vs gathered form")
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+def test_conv3x3_lds_tile_kernel_every_tile_shape(ctx, tile):
+    """The LDS-tile kernel exists for the same five workgroup tiles as the gathered form."""
+    cases = [(3, 16, 28, 28, 70, [1, 1, 1, 1], 1), (5, 24, 14, 14, 200, [1, 1, 1, 1], 1),
+             (9, 32, 7, 7, 33, [1, 0, 1, 2], 1), (2, 32, 20, 56, 24, [1, 1, 1, 1], 2)]
+    for n, cin, h, w, cout, pads, group in cases:
+        X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin // group, 3), nrm(cout)
+        want = ref.conv(X, W, B, None, group, None, pads, None)
+        try:
+            ctx.set_option("contraction_tile", tile)
+            got = hip_conv(ctx, X, W, B, None, group, pads)
+            ctx.set_option("split_k", 3)
+            cut = hip_conv(ctx, X, W, B, None, group, pads, epilogue="relu")
+        finally:
+            ctx.set_option("contraction_tile", -1)
+            ctx.set_option("split_k", -1)
+        assert_close_max(got, want, GEMM_TOL, "tile %d %s" % (tile, (n, cin, h, w, cout)))
+        assert_close_max(cut, ref.unary("Relu", want), GEMM_TOL, "tile %d split 3" % tile)

@@ -176,7 +176,7 @@ struct ConvGeom {
   // conv3x3_halo_kernel only: the input rows a tile needs are staged in LDS as
   // rows of `pitch` floats, `slots` of them per channel, the first input column in
   // LDS column col0; pb/pr = bottom / right padding
-  int pitch, slots, col0;
+  int pitch, slots, col0, units;
   FastDiv fd_ow, fd_oh, fd_ohw;      // output width, height, plane
   FastDiv fd_plane;                  // h*w
   FastDiv fd_oh2, fd_upc, fd_pg;     // oh+2, pieces per channel, pieces per row (halo kernel)
@@ -938,9 +938,13 @@ constexpr int HALO_ROWA = HALO_KB + 4;     // weight tile row stride (floats)
 constexpr int HALO_AROWS = 14;             // weight rows per pass: 256 threads = 14 rows x 18 pieces
 // floats per channel of the input tile; 32 mod 64 so that the two halves of a
 // wavefront (channels c and c + 4) fall on different LDS banks
-constexpr int halo_plane(int bn) { return bn <= 64 ? 480 : 544; }
-// 16/8/4-byte pieces of the input tile per thread and block
-constexpr int halo_units(int vecw) { return vecw == 1 ? 5 : 4; }
+constexpr int halo_plane(int bn) { return bn <= 64 ? 480 : (bn <= 128 ? 544 : 672); }
+// most 16/8/4-byte pieces of the input tile a thread fetches per block (the launch says
+// how many of them a geometry needs)
+constexpr int halo_units(int vecw, int bn) {
+  return vecw == 4 ? (bn <= 64 ? 4 : (bn <= 128 ? 5 : 6))
+                   : (vecw == 2 ? (bn <= 64 ? 4 : (bn <= 128 ? 6 : 8)) : (bn <= 64 ? 5 : (bn <= 128 ? 8 : 12)));
+}
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 template <int VECW> struct HaloPiece;
@@ -964,12 +968,12 @@ template <> struct HaloPiece<1> {
 };
 
 template <int BM, int BN, int WM, int WN, int VECW>
-__global__ __launch_bounds__(NTHREADS, BM * BN <= 64 * 64 ? 4 : 2) void conv3x3_halo_kernel(Params p) {
+__global__ __launch_bounds__(NTHREADS, BM == 64 ? (BN == 64 ? 4 : (BN == 128 ? 3 : 2)) : 2) void conv3x3_halo_kernel(Params p) {
   static_assert(WM * WN == NTHREADS / 64, "four wavefronts");
   constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
   constexpr int PLANE = halo_plane(BN);
   constexpr int AU = (BM + HALO_AROWS - 1) / HALO_AROWS;  // weight pieces per thread and block
-  constexpr int XU = halo_units(VECW);
+  constexpr int XU = halo_units(VECW, BN);
   typedef typename HaloPiece<VECW>::type xpiece;
   __shared__ __attribute__((aligned(16))) float as[AU * HALO_AROWS * HALO_ROWA];
   __shared__ __attribute__((aligned(16))) float xs[HALO_CB * PLANE + 4];  // + a dump cell for idle pieces
@@ -1009,6 +1013,7 @@ __global__ __launch_bounds__(NTHREADS, BM * BN <= 64 * 64 ? 4 : 2) void conv3x3_
   const int pg = cv.pitch / VECW;       // pieces per row
   const int upc = cv.slots * pg;        // pieces per channel
   const int first_rows = (img0 + 1) * cv.oh - R0;  // output rows from R0 to the end of its image
+  const int xu = cv.units;  // pieces per thread this geometry needs (<= XU)
   int voff_x[XU], lds_x_w[XU];
 #pragma unroll
   for (int i = 0; i < XU; i++) {
@@ -1071,7 +1076,8 @@ __global__ __launch_bounds__(NTHREADS, BM * BN <= 64 * 64 ? 4 : 2) void conv3x3_
 #pragma unroll
     for (int i = 0; i < AU; i++) ra[i] = buf_load4(rsrc_a, voff_a[i], soff_a);
 #pragma unroll
-    for (int i = 0; i < XU; i++) rx[i] = HaloPiece<VECW>::load(rsrc_x, voff_x[i], soff_x);
+    for (int i = 0; i < XU; i++)
+      if (i < xu) rx[i] = HaloPiece<VECW>::load(rsrc_x, voff_x[i], soff_x);
   };
   auto stash = [&]() {
     char *const as_b = reinterpret_cast<char *>(as);
@@ -1080,7 +1086,8 @@ __global__ __launch_bounds__(NTHREADS, BM * BN <= 64 * 64 ? 4 : 2) void conv3x3_
     for (int i = 0; i < AU; i++)
       *reinterpret_cast<f32x4 *>(as_b + lds_a_w + i * (HALO_AROWS * HALO_ROWA * 4)) = ra[i];
 #pragma unroll
-    for (int i = 0; i < XU; i++) *reinterpret_cast<xpiece *>(xs_b + lds_x_w[i]) = rx[i];
+    for (int i = 0; i < XU; i++)
+      if (i < xu) *reinterpret_cast<xpiece *>(xs_b + lds_x_w[i]) = rx[i];
   };
   auto compute = [&]() {
     const char *const as_b = reinterpret_cast<const char *>(as);
@@ -1374,8 +1381,8 @@ bool halo_fits(ConvGeom &cv, int bn, int nimg, int vecw, int pr) {
   cv.fd_pg = make_fastdiv(cv.pitch / vecw);
   cv.fd_upc = make_fastdiv((long long)cv.slots * (cv.pitch / vecw));
   const long long pieces = (long long)HALO_CB * cv.slots * (cv.pitch / vecw);
-  return (long long)cv.slots * cv.pitch <= halo_plane(bn) &&
-         pieces <= (long long)halo_units(vecw) * NTHREADS;
+  cv.units = (int)((pieces + NTHREADS - 1) / NTHREADS);
+  return (long long)cv.slots * cv.pitch <= halo_plane(bn) && cv.units <= halo_units(vecw, bn);
 }
 
 template <bool A_KC, int BMODE>
@@ -1679,7 +1686,12 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       c_in_g % HALO_CB == 0 && aligned16(p.A)) {
     const int vecw = (w % 4 == 0 && aligned16(p.B)) ? 4 : ((w % 2 == 0 && ((uintptr_t)p.B & 7) == 0) ? 2 : 1);
     p.cv.h = h; p.cv.w = w; p.cv.oh = oh; p.cv.ow = ow; p.cv.pt = pt; p.cv.pl = pl;
-    const int bn = g_forced_tile == T64x128 ? 128 : 64;
+    // tile: 64x128 (each wavefront 64 rows x 32 pixels: one LDS read of the input feeds two
+    // matrix-core steps) where the pixel count fills the chip with such tiles, 64x64 below
+    TileId tile = g_forced_tile >= 0 ? (TileId)g_forced_tile : T64x64;
+    if (g_forced_tile < 0 && (npix + 127) / 128 * ((cout_g + 63) / 64) * group >= 2LL * wdh::compute_units())
+      tile = T64x128;
+    const int bn = kTileN[tile];
     if (halo_fits(p.cv, bn, n, vecw, pr)) {
       p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
       p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
@@ -1692,8 +1704,13 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       p.b_bytes = (int)((long long)n * c * h * w * 4);
       p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
       p.c_bytes = cout * 4;
-      if (bn == 128) return launch_halo_tile<64, 128, 1, 4>(p, group, vecw);
-      return launch_halo_tile<64, 64, 2, 2>(p, group, vecw);
+      switch (tile) {
+        case T128x128: return launch_halo_tile<128, 128, 2, 2>(p, group, vecw);
+        case T64x256: return launch_halo_tile<64, 256, 1, 4>(p, group, vecw);
+        case T64x128: return launch_halo_tile<64, 128, 1, 4>(p, group, vecw);
+        case T128x64: return launch_halo_tile<128, 64, 2, 2>(p, group, vecw);
+        default: return launch_halo_tile<64, 64, 2, 2>(p, group, vecw);
+      }
     }
   }
   const int mode = !small || ntaps > 63 ? B_IM2COL_BIG : (ntaps > 31 ? B_IM2COL64 : B_IM2COL32);
