@@ -1,26 +1,16 @@
 "use strict";
-// CPU tensor: a typed array plus dims.  The I/O type of runner.run().
-// Reference: src/descriptor_runner/backend/cpu/cpuTensorImpl.ts:14-89.
+// Host tensor: a typed array plus dims; what runner.run() takes and returns.
+// Interface after src/descriptor_runner/backend/cpu/cpuTensorImpl.ts:14-89 (data,
+// useExternalBuffer, getData / setData / getDataSync, getValue / setValue, dispose, isCPUTensor).
 const { TensorImpl } = require("../../core/tensorImpl");
 const { DataArrayConstructor } = require("../../interface/constants");
 
 class CPUTensorImpl extends TensorImpl {
+  // `data`: wrap the caller's typed array instead of allocating a zero-filled one
   constructor(dims, dataType, data) {
     super(dims, dataType || "float32", "cpu");
-    this.data = data || new DataArrayConstructor[this.dataType](this.length);
-    this.useExternalBuffer = !!data;
-  }
-
-  async getData() {
-    return this.data;
-  }
-
-  async setData(data) {
-    this.data.set(data);
-  }
-
-  dispose() {
-    this.data = new Float32Array(1);
+    this.useExternalBuffer = data != null;
+    this.data = this.useExternalBuffer ? data : new DataArrayConstructor[this.dataType](this.length);
   }
 
   static isCPUTensor(tensor) {
@@ -31,18 +21,31 @@ class CPUTensorImpl extends TensorImpl {
     return this.data;
   }
 
-  getValue(idxs) {
-    if (idxs.length !== this.ndim) throw new Error("length of idxs does not match tensor.ndim");
-    let ofs = 0;
-    for (let i = 0; i < this.ndim; i++) ofs += this.strides[i] * idxs[i];
-    return this.data[ofs];
+  async getData() {
+    return this.data;
   }
 
-  setValue(value, idxs) {
-    if (idxs.length !== this.ndim) throw new Error("length of idxs does not match tensor.ndim");
-    let ofs = 0;
-    for (let i = 0; i < this.ndim; i++) ofs += this.strides[i] * idxs[i];
-    this.data[ofs] = value;
+  async setData(values) {
+    this.data.set(values);
+  }
+
+  // Drops the (possibly large) array; the object stays valid but empty.
+  dispose() {
+    this.data = new Float32Array(1);
+  }
+
+  // Position of an element named by one index per axis.
+  offsetOf(indices) {
+    if (indices.length !== this.ndim) throw new Error("length of idxs does not match tensor.ndim");
+    return indices.reduce((offset, index, axis) => offset + index * this.strides[axis], 0);
+  }
+
+  getValue(indices) {
+    return this.data[this.offsetOf(indices)];
+  }
+
+  setValue(value, indices) {
+    this.data[this.offsetOf(indices)] = value;
   }
 }
 

@@ -1,7 +1,8 @@
 "use strict";
-// Reference: src/descriptor_runner/operators/base/transpose.ts:7-35.
+// Contract after src/descriptor_runner/operators/base/transpose.ts:7-35.
 const { OperatorImpl } = require("../operatorImpl");
 const { getAttrInts } = require("../operatorUtil");
+const { permutedView } = require("../shapes");
 
 class Transpose extends OperatorImpl {
   initialize(attribute) {
@@ -9,18 +10,9 @@ class Transpose extends OperatorImpl {
     this.perm = getAttrInts(attribute, "perm", []);
   }
 
+  // -> {outShape, inStrides}: the output is the input read through permuted strides
   calcShape(input) {
-    // default perm: reversed axes
-    const perm = this.perm.length > 0 ? this.perm : Array.from({ length: input.ndim }, (v, i) => input.ndim - 1 - i);
-    if (perm.length !== input.ndim) throw new Error("Transpose: perm length differs from rank");
-    const outShape = new Array(input.ndim),
-      inStrides = new Array(input.ndim);
-    for (let outAxis = 0; outAxis < input.ndim; outAxis++) {
-      const inAxis = perm[outAxis];
-      outShape[outAxis] = input.dims[inAxis];
-      inStrides[outAxis] = input.strides[inAxis];
-    }
-    return { outShape, inStrides };
+    return permutedView(input.dims, input.strides, this.perm);
   }
 }
 module.exports = { Transpose };

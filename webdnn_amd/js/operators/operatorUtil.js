@@ -1,6 +1,6 @@
 "use strict";
-// Attribute getters, strides and broadcasting shared by every backend's operators.
-// Reference: src/descriptor_runner/operators/operatorUtil.ts:8-245.
+// Attribute getters shared by every backend's operators.
+// Reference: src/descriptor_runner/operators/operatorUtil.ts:8-125.
 const { clipToInt32 } = require("../util");
 const { DataType } = require("../core/onnxProto");
 
@@ -83,55 +83,10 @@ function tensorProtoToArray(t) {
   }
 }
 
-function calcStrides(dims) {
-  const strides = [];
-  let length = 1;
-  for (let i = dims.length - 1; i >= 0; i--) {
-    strides.unshift(length);
-    length *= dims[i];
-  }
-  return strides;
-}
-
-// Strides of B when broadcast (unidirectionally) to A's shape.
-function broadcastUni(dimsA, dimsB) {
-  if (dimsA.length < dimsB.length) {
-    throw new Error(`Unidirectional broadcast error: ${dimsA}, ${dimsB}`);
-  }
-  const expandedDimsB = Array.prototype.slice.call(dimsB);
-  while (expandedDimsB.length < dimsA.length) expandedDimsB.unshift(1);
-  const stridesB = calcStrides(expandedDimsB);
-  for (let i = 0; i < dimsA.length; i++) {
-    if (dimsA[i] !== expandedDimsB[i]) {
-      if (expandedDimsB[i] === 1) stridesB[i] = 0;
-      else throw new Error(`Unidirectional broadcast error: ${dimsA}, ${dimsB}`);
-    }
-  }
-  return stridesB;
-}
-
-// Multidirectional broadcast of several shapes: result dims + strides of every input.
-function broadcastMulti(allDims) {
-  const ndim = Math.max(...allDims.map((d) => d.length));
-  const expandedAll = allDims.map((dims) => {
-    const e = Array.prototype.slice.call(dims);
-    while (e.length < ndim) e.unshift(1);
-    return e;
-  });
-  const dims = [];
-  for (let i = 0; i < ndim; i++) dims.push(Math.max(...expandedAll.map((e) => e[i])));
-  const allStrides = expandedAll.map((e) => {
-    const strides = calcStrides(e);
-    for (let i = 0; i < ndim; i++) {
-      if (e[i] !== dims[i]) {
-        if (e[i] === 1) strides[i] = 0;
-        else throw new Error(`Multidirectional broadcasting error: ${allDims.map((d) => `[${d}]`)}`);
-      }
-    }
-    return strides;
-  });
-  return { dims, allStrides };
-}
+// Strides and the two broadcasting rules live with the rest of the shape arithmetic
+// (operators/shapes.js); operator files import them from here under the names the
+// reference's operators use (operatorUtil.ts:169-245).
+const { denseStrides: calcStrides, broadcastOnto: broadcastUni, broadcastTogether: broadcastMulti } = require("./shapes");
 
 module.exports = {
   getAttrFloat, getAttrInt, getAttrInts, getAttrString, getAttrTensor, tensorProtoToArray,
