@@ -261,6 +261,13 @@ int wdh_layernorm(wdh_buf X, wdh_buf Gamma, wdh_buf Beta, wdh_buf Y,
 /* ReduceMean over the trailing `len` elements of each of `outer` rows;
  * replaces ReduceMean (reduce.ts:369-405) for trailing-axes reductions. */
 int wdh_reduce_mean(wdh_buf X, wdh_buf Y, int64_t outer, int len);
+/* One pass of ReduceMean over an arbitrary set of axes: the reference reduces the
+ * axes one after the other in ascending order (ReduceOp.runCore, reduce.ts:40-100),
+ * each pass a sum in double stored as fp32, the last pass divided by the product of
+ * all reduced extents (reduce.ts:369-405).  X viewed as [outer, red, inner]:
+ *   Y[o, i] = f32( (sum_r X[o, r, i]) / divisor ),  divisor = 1 for all passes but the last. */
+int wdh_reduce_axis(wdh_buf X, wdh_buf Y, int64_t outer, int red, int64_t inner,
+                    int64_t divisor);
 
 /* ---- pooling -------------------------------------------------------------
  * Replaces CpuMaxPool.maxpool (operators/cpu/operators/standard/maxpool.ts:58-112);

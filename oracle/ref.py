@@ -223,6 +223,27 @@ def reduce_mean_last(X):
     return Y
 
 
+def reduce_mean(X, axes=(), keepdims=1):
+    """ReduceMean over any set of axes (all axes when `axes` is empty): one pass per axis in
+    ascending order, fp32 between the passes (reduce.ts:40-100, 114-131, 369-405)."""
+    X = _f32(X)
+    nd = X.ndim
+    ax = sorted(a + nd if a < 0 else a for a in axes) if len(axes) else list(range(nd))
+    shape, data, total = list(X.shape), np.ascontiguousarray(X).reshape(-1), 1
+    for i, a in enumerate(ax):
+        red = shape[a]
+        total *= red
+        outer = int(np.prod(shape[:a], dtype=np.int64))
+        inner = int(np.prod(shape[a + 1:], dtype=np.int64))
+        out = np.empty(outer * inner, dtype=np.float32)
+        divisor = float(total) if i == len(ax) - 1 else 1.0
+        _check(_lib.ref_reduce_axis(_ptr(data), ctypes.c_int64(outer), ctypes.c_int64(red), ctypes.c_int64(inner),
+                                    ctypes.c_double(divisor), _ptr(out)), "ReduceMean")
+        shape[a], data = 1, out
+    final = shape if keepdims else [d for i, d in enumerate(shape) if i not in ax]
+    return data.reshape(final)
+
+
 def gather(data, indices, axis=0):
     data = np.asarray(data, order="C")
     indices = np.asarray(indices, dtype=np.int32, order="C")

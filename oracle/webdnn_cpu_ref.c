@@ -539,13 +539,29 @@ int ref_transpose(const uint32_t *dI, const int64_t *dims, int ndim,
  * operators/cpu/operators/standard/reduce.ts:369-405 restricted to a reduction
  * over the single last axis: X viewed as [outer, len]; sum in double in index
  * order, divided by len, stored as fp32.  (Several axes are reduced one after
- * the other there with an fp32 store in between; that form is not restated.) */
+ * the other there with an fp32 store in between: ref_reduce_axis below.) */
 int ref_reduce_mean_trailing(const float *X, int64_t outer, int64_t len, float *Y) {
 #pragma omp parallel for num_threads(g_threads) schedule(static)
   for (int64_t o = 0; o < outer; o++) {
     double s = 0;
     for (int64_t r = 0; r < len; r++) s += (double)X[o * len + r];
     Y[o] = (float)(s / (double)len);
+  }
+  return REF_OK;
+}
+
+/* One pass of the general form (ReduceOp.runCore, reduce.ts:40-100, with the ReduceMean
+ * kernels of reduce.ts:369-405): X viewed as [outer, red, inner]; every result is the sum
+ * of its `red` elements in index order in double, divided by `divisor` (1 for every pass
+ * but the last, the product of all reduced extents for the last) and stored as fp32. */
+int ref_reduce_axis(const float *X, int64_t outer, int64_t red, int64_t inner, double divisor, float *Y) {
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t o = 0; o < outer; o++) {
+    for (int64_t n = 0; n < inner; n++) {
+      double s = 0;
+      for (int64_t r = 0; r < red; r++) s += (double)X[(o * red + r) * inner + n];
+      Y[o * inner + n] = divisor == 1.0 ? (float)s : (float)(s / divisor);
+    }
   }
   return REF_OK;
 }

@@ -45,8 +45,7 @@ def run_graph(model, feeds, keep=None):
             y = ref.layernorm_decomposed(x[0], x[1] if len(x) > 1 else None, x[2] if len(x) > 2 else None,
                                          a.get("epsilon", 1e-5))
         elif op == "ReduceMean":
-            assert a.get("axes") in ([-1], [x[0].ndim - 1]) and a.get("keepdims", 1) == 1
-            y = ref.reduce_mean_last(x[0])
+            y = ref.reduce_mean(x[0], a.get("axes", []), a.get("keepdims", 1))
         elif op == "Squeeze":
             y = ref.squeeze(x[0], x[1].reshape(-1) if len(x) > 1 else a.get("axes", []))
         elif op == "Unsqueeze":

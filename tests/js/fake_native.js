@@ -188,6 +188,18 @@ const native = {
     }
   },
 
+  reduceAxis(X, Y, outer, red, inner, divisor) {
+    count("reduceAxis");
+    const x = f32(X), y = f32(Y);
+    for (let o = 0; o < outer; o++) {
+      for (let n = 0; n < inner; n++) {
+        let s = 0;
+        for (let r = 0; r < red; r++) s += x[(o * red + r) * inner + n];
+        y[o * inner + n] = s / divisor;
+      }
+    }
+  },
+
   reduceMean(X, Y, outer, len) {
     count("reduceMean");
     const x = f32(X), y = f32(Y);
@@ -284,7 +296,7 @@ const native = {
 // Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
 // alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
 // calls that need device data on the host throw and spoil the capture.
-const RECORDED = ["copy", "gemm", "conv2d", "binary", "unary", "softmax", "layernorm", "reduceMean", "maxpool2d",
+const RECORDED = ["copy", "gemm", "conv2d", "binary", "unary", "softmax", "layernorm", "reduceMean", "reduceAxis", "maxpool2d",
   "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
 const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
 const graphs = new Map();

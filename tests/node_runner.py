@@ -9,6 +9,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_ENTRIES = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 FAKE_NATIVE = os.path.join(ROOT, "tests", "js", "fake_native.js")
+RETRY_ENTRIES = os.path.join(ROOT, "tests", "js", "retry_entries.js")
 
 
 def run_model(model_dir, inputs, backend, strict=True, fuse=True, oracle_cpu=False, runs=1, warmup=0,

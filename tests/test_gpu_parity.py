@@ -334,6 +334,29 @@ def test_global_average_pool_and_reduce_mean(ctx, shape):
     assert ulp_diff(rm, ref.reduce_mean_last(flat)).max() <= 1
 
 
+@pytest.mark.parametrize("shape,axes,keep", [
+    ((6, 7, 8), [0], 1), ((6, 7, 8), [1], 0), ((6, 7, 8), [2], 1), ((6, 7, 8), [0, 2], 0), ((6, 7, 8), [], 1),
+    ((3, 4, 5, 6), [1, 2], 1), ((3, 4, 5, 6), [-1, 0], 0), ((2, 850, 256), [1], 1), ((32, 64, 56, 56), [0], 0),
+    ((4, 2048, 7, 7), [2, 3], 1), ((1, 100, 1, 256), [3, 1], 0), ((5,), [0], 0), ((300, 1000), [0], 1)])
+def test_reduce_mean_over_any_axes(ctx, shape, axes, keep):
+    """reduce.ts:40-131, 369-405: one pass per axis.  A pass over an inner axis adds in the
+    reference's order (bit-exact); a pass over the last axis adds across a wavefront, which may
+    cost the last bit of the double sum, at most 1 fp32 ulp per such pass."""
+    from util import ulp_diff
+
+    x = nrm(*shape)
+    got = H.reduce_mean(ctx, ctx.move_tensor(x), axes, keep)
+    want = ref.reduce_mean(x, axes, keep)
+    assert tuple(got.dims) == want.shape
+    ax = sorted(a % len(shape) for a in axes) if axes else list(range(len(shape)))
+    if ax[-1] != len(shape) - 1:
+        assert_bit_exact(got.get_data(), want, "ReduceMean %s over %s" % (shape, axes))
+    else:
+        assert ulp_diff(got.get_data(), want).max() <= 1
+    with pytest.raises(H.OperatorError):
+        H.reduce_mean(ctx, ctx.move_tensor(x), [len(shape)], keep)
+
+
 # ------------------------------------------------------------------ MaxPool
 def test_maxpool_resnet_stem_full(ctx):
     x = nrm(32, 64, 112, 112)

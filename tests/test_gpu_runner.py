@@ -91,17 +91,31 @@ def test_non_strict_falls_back_per_node(tmp_path):
         node_runner.run_model(str(tmp_path), [X], "hip", strict=True)
     with pytest.raises(RuntimeError, match="only reducing final axis"):
         node_runner.run_model(str(tmp_path), [X], "hip", strict=False, oracle_cpu=True)
+    # an operator whose hip implementation throws (tests/js/retry_entries.js) and whose cpu one works
     g = modelgen.GraphBuilder(0)
     g.op("Relu", ["X"], "r")
-    g.op("ReduceMean", ["r"], "m", axes=[0], keepdims=1)   # hip supports only the last axis -> cpu retry
+    g.op("TestFlaky", ["r"], "m")
     g.op("Relu", ["m"], "Y")
-    data = g.finish([("X", [4, 6])], [("Y", [1, 6])])
+    data = g.finish([("X", [4, 6])], [("Y", [4, 6])])
     (tmp_path / "model.onnx").write_bytes(data)
     X = np.random.default_rng(7).standard_normal((4, 6)).astype(np.float32)
-    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=False, oracle_cpu=True)
-    assert rep["stats"]["retriedOnCpu"] == ["ReduceMean_1"]
+    retry = ["--cpu-entries", node_runner.RETRY_ENTRIES]
+    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=False, extra=retry)
+    assert rep["stats"]["retriedOnCpu"] == ["TestFlaky_1"]
     assert rep["stats"]["nodesByBackend"] == {"hip": 2, "cpu": 1}
-    np.testing.assert_allclose(outs[0], np.maximum(np.maximum(X, 0).mean(0, keepdims=True), 0), rtol=1e-6)
+    assert_bit_exact(outs[0], 2 * np.maximum(X, 0), "retried node")
+    with pytest.raises(RuntimeError, match="the hip implementation refuses"):
+        node_runner.run_model(str(tmp_path), [X], "hip", strict=True, extra=retry)
+    # ReduceMean over a leading axis runs on the device
+    g = modelgen.GraphBuilder(0)
+    g.op("ReduceMean", ["X"], "Y", axes=[0, 2], keepdims=0)
+    data = g.finish([("X", [5, 6, 7])], [("Y", [6])])
+    (tmp_path / "model.onnx").write_bytes(data)
+    X3 = np.random.default_rng(8).standard_normal((5, 6, 7)).astype(np.float32)
+    outs, rep = node_runner.run_model(str(tmp_path), [X3], "hip", strict=True)
+    assert rep["stats"]["nodesByBackend"] == {"hip": 1}
+    from oracle import ref
+    assert np.abs(outs[0] - ref.reduce_mean(X3, [0, 2], 0)).max() <= 1e-7
 
 
 def test_detr_style_small(tmp_path):

@@ -280,6 +280,55 @@ def test_means():
         ref.global_average_pool(rnd(2, 3, 4))                            # globalaveragepool.ts:16-18
 
 
+def test_reduce_mean_over_any_axes():
+    """The general form (one pass per axis, fp32 between passes).  Pinned by: exact rational
+    arithmetic on integers small enough that every pass is exact; a brute-force pass-by-pass
+    evaluation in Python floats; numpy float64 means within the ulps the passes can cost; the
+    trailing-axis function it generalises; shapes with and without keepdims."""
+    from fractions import Fraction
+
+    rng = np.random.default_rng(21)
+    xi = rng.integers(-500, 500, (3, 4, 5, 6)).astype(np.float32)
+    for axes in ([0], [1, 3], [0, 1, 2, 3], [2], [-1, -3]):
+        ax = sorted(a % 4 for a in axes)
+        got = ref.reduce_mean(xi, axes, 1)
+        cnt = int(np.prod([xi.shape[a] for a in ax]))
+        exact = xi.astype(np.int64).sum(tuple(ax), keepdims=True)
+        want = np.vectorize(lambda v: np.float32(Fraction(int(v), cnt)))(exact).astype(np.float32)
+        assert_bit_exact(got, want, "integers: every pass exact, one rounding at the end %s" % (axes,))
+    x = rnd(3, 4, 5, 6)
+    # brute force, two axes: pass over axis 1 (fp32 store), then over axis 3 divided by 4*6
+    first = np.zeros((3, 5, 6), np.float32)
+    for o in range(3):
+        for i in range(5):
+            for j in range(6):
+                acc = 0.0
+                for r in range(4):
+                    acc += float(x[o, r, i, j])
+                first[o, i, j] = acc
+    second = np.zeros((3, 5), np.float32)
+    for o in range(3):
+        for i in range(5):
+            acc = 0.0
+            for r in range(6):
+                acc += float(first[o, i, r])
+            second[o, i] = acc / 24
+    assert_bit_exact(ref.reduce_mean(x, [1, 3], 0), second, "pass by pass")
+    assert ref.reduce_mean(x, [3, 1], 1).shape == (3, 1, 5, 1)                 # order of the list is irrelevant
+    assert_bit_exact(ref.reduce_mean(x, [3, 1], 0), second, "axes are sorted")
+    for axes in ([0], [2], [0, 2], [1, 2, 3], []):
+        ax = tuple(axes) if axes else (0, 1, 2, 3)
+        want = x.astype(np.float64).mean(ax, keepdims=True).astype(np.float32)
+        got = ref.reduce_mean(x, axes, 1)
+        assert got.shape == want.shape
+        # every pass rounds a partial sum once: half an ulp of a value no larger than the sum of
+        # the magnitudes, which the divisions turn into half an ulp of max|x| per pass at most
+        assert np.abs(got - want).max() <= len(ax) * 2.0 ** -24 * np.abs(x).max(), axes
+    assert_bit_exact(ref.reduce_mean(x, [3], 1), ref.reduce_mean_last(x), "trailing axis")
+    assert_bit_exact(ref.reduce_mean(x, [-1], 1), ref.reduce_mean_last(x), "negative axis")
+    assert ref.reduce_mean(x, [], 0).shape == () and ref.reduce_mean(x, [0, 3], 0).shape == (4, 5)
+
+
 def sum_seq(plane):
     s = 0.0
     for v in plane.reshape(-1):

@@ -56,6 +56,7 @@ SIGNATURES = {
     "wdh_softmax": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
     "wdh_layernorm": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_float]),
     "wdh_reduce_mean": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
+    "wdh_reduce_axis": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64]),
     "wdh_maxpool2d": (_c.c_int, [c_buf, c_buf] + [_c.c_int] * 14),
     "wdh_global_avgpool": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
     "wdh_transpose": (_c.c_int, [c_buf, c_buf, _c.c_int, _i32p, _i64p]),

@@ -240,6 +240,36 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void mean_rows_wave(
   if (lane == 0) Y[row] = (float)(s / (double)len);
 }
 
+// ---- sum over one inner axis -----------------------------------------------------
+// X viewed as [outer, red, inner] with inner > 1: thread (o, i) adds its `red` elements,
+// which lie `inner` apart, in index order in double; neighbouring threads read
+// neighbouring addresses.  Rows along a middle axis are short in the graphs this
+// serves (channel or head axes), so one thread per result is the whole schedule.
+__global__ __launch_bounds__(256) void sum_axis_kernel(const float *__restrict__ X,
+                                                       float *__restrict__ Y, long long outer,
+                                                       int red, long long inner, double divisor) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= outer * inner) return;
+  const long long o = idx / inner, i = idx - o * inner;
+  const float *x = X + o * red * inner + i;
+  double s = 0.0;
+  for (int r = 0; r < red; r++) s += (double)x[(long long)r * inner];
+  Y[idx] = (float)(s / divisor);
+}
+
+// the last axis with a divisor that is not its length (a pass of a multi-axis mean)
+__global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void sum_rows_wave(
+    const float *__restrict__ X, float *__restrict__ Y, long long outer, int len, double divisor) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= outer) return;
+  const float *x = X + row * len;
+  double s = 0.0;
+  for (int idx = lane; idx < len; idx += 64) s += (double)x[idx];
+  s = wave_sum_d(s);
+  if (lane == 0) Y[row] = (float)(s / divisor);
+}
+
 unsigned row_blocks(long long outer) {
   return (unsigned)((outer + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
 }
@@ -337,6 +367,31 @@ extern "C" int wdh_reduce_mean(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
     hipLaunchKernelGGL(mean_rows_wave, dim3(row_blocks(outer)),
                        dim3(64 * WAVES_PER_BLOCK), 0, st, (const float *)px,
                        (float *)py, (long long)outer, len);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+extern "C" int wdh_reduce_axis(wdh_buf hX, wdh_buf hY, int64_t outer, int red, int64_t inner,
+                               int64_t divisor) {
+  WDH_REQUIRE_INIT();
+  if (outer < 0 || red < 0 || inner < 0) return fail(WDH_EINVAL, "wdh_reduce_axis: negative extent");
+  if (divisor <= 0) return fail(WDH_EINVAL, "wdh_reduce_axis: divisor %lld", (long long)divisor);
+  const long long results = (long long)outer * inner;
+  if (results == 0) return WDH_OK;
+  if (red == 0) return fail(WDH_EINVAL, "wdh_reduce_axis: empty reduction");
+  if (inner == 1 && divisor == red) return wdh_reduce_mean(hX, hY, outer, red);
+  if ((results + 255) / 256 > 0x7fffffffLL || (outer + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK > 0x7fffffffLL)
+    return fail(WDH_EINVAL, "wdh_reduce_axis: too many results");
+  void *px, *py;
+  if (!wdh::operand(hX, (size_t)results * red * 4, "wdh_reduce_axis: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)results * 4, "wdh_reduce_axis: Y", &py)) return WDH_EINVAL;
+  if (inner == 1)
+    hipLaunchKernelGGL(sum_rows_wave, dim3(row_blocks(outer)), dim3(64 * WAVES_PER_BLOCK), 0, wdh::stream(),
+                       (const float *)px, (float *)py, (long long)outer, red, (double)divisor);
+  else
+    hipLaunchKernelGGL(sum_axis_kernel, dim3((unsigned)((results + 255) / 256)), dim3(256), 0, wdh::stream(),
+                       (const float *)px, (float *)py, (long long)outer, red, (long long)inner,
+                       (double)divisor);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
 }

@@ -417,6 +417,35 @@ def reduce_mean_last(ctx, x, keepdims=1):
     return y
 
 
+def reduce_mean(ctx, x, axes=(), keepdims=1):
+    """ReduceMean over any axes (all of them when `axes` is empty): cpu reduce.ts:40-131, 369-405 --
+    one pass per axis in ascending order, fp32 between the passes, the last pass divides by the
+    product of the reduced extents."""
+    _require_f32(x)
+    nd = x.ndim
+    ax = sorted(int(a) + nd if int(a) < 0 else int(a) for a in axes) if len(axes) else list(range(nd))
+    if any(not 0 <= a < nd for a in ax) or len(set(ax)) != len(ax):
+        raise OperatorError("ReduceMean: axes out of range or repeated")
+    shape, cur, total = list(x.dims), x, 1
+    for i, a in enumerate(ax):
+        red = shape[a]
+        total *= red
+        outer, inner = int(np.prod(shape[:a], dtype=np.int64)), int(np.prod(shape[a + 1:], dtype=np.int64))
+        shape[a] = 1
+        nxt = ctx.empty_tensor(shape)
+        call("wdh_reduce_axis", cur.handle, nxt.handle, outer, red, inner, total if i == len(ax) - 1 else 1)
+        if cur is not x:
+            cur.dispose()
+        cur = nxt
+    if cur is x:                                   # rank 0: nothing to reduce
+        return x.alias(list(x.dims))
+    if not keepdims:
+        out = cur.alias([d for i, d in enumerate(shape) if i not in ax])
+        cur.dispose()
+        return out
+    return cur
+
+
 def maxpool_shape(dims_x, kernel_shape, auto_pad="NOTSET", ceil_mode=0, dilations=None, pads=None,
                   strides=None):
     """operators/base/maxpool.ts:32-137"""

@@ -325,6 +325,13 @@ FN(js_reduce_mean) {
   return make_undefined(env);
 }
 
+FN(js_reduce_axis) {
+  ARGS("wdh_reduce_axis", 6);
+  I64(0, X); I64(1, Y); I64(2, outer); I64(3, red); I64(4, inner); I64(5, divisor);
+  CHECK(wdh_reduce_axis(X, Y, outer, (int)red, inner, divisor));
+  return make_undefined(env);
+}
+
 FN(js_maxpool2d) {
   ARGS("wdh_maxpool2d", 16);
   I64(0, X); I64(1, Y);
@@ -423,7 +430,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"read", js_read}, {"copy", js_copy}, {"sync", js_sync}, {"memStats", js_mem_stats},
       {"trim", js_trim}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
       {"gemm", js_gemm}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
-      {"softmax", js_softmax}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean},
+      {"softmax", js_softmax}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
       {"stridedCopy", js_strided_copy}, {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end},
