@@ -183,6 +183,17 @@ int wdh_gemm(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
              int64_t sB0, int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
              float beta, int epilogue, wdh_buf R);
 
+/* wdh_gemm with a spaced-out result: Y[b, i, j] = Y[b*sYb + i*sY0 + j] (R alike), rows
+ * contiguous.  It lets a MatMul write straight into the layout a following Transpose
+ * would have produced (attention heads merged back: [heads, tokens, d] stored as
+ * [tokens, heads, d], CPUTranspose.copyNd, transpose.ts:46-168, absorbed into the
+ * product).  wdh_gemm is this call with sYb = m*n, sY0 = n.  Batch entries must not
+ * overlap: sYb >= m*sY0, or sYb >= n and sY0 >= batch*sYb. */
+int wdh_gemm_ex(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
+                int n, int k, int64_t sAb, int64_t sA0, int64_t sA1, int64_t sBb,
+                int64_t sB0, int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
+                float beta, int epilogue, wdh_buf R, int64_t sYb, int64_t sY0);
+
 /* wdh_gemm for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments, same kernels and bit-identical

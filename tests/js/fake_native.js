@@ -86,17 +86,22 @@ const native = {
   },
 
   gemm(A, B, C, Y, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1, alpha, beta, epi, R) {
+    native.gemmEx(A, B, C, Y, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1, alpha, beta, epi, R, m * n, n);
+  },
+
+  gemmEx(A, B, C, Y, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1, alpha, beta, epi, R, sYb, sY0) {
     count("gemm");
-    need(Y, batch * m * n * 4, "wdh_gemm: Y");
+    need(Y, ((batch - 1) * sYb + (m - 1) * sY0 + n) * 4, "wdh_gemm: Y");
     const a = f32(A, "A"), b = f32(B, "B"), y = f32(Y, "Y");
     const c = C ? f32(C, "C") : null, r = R ? f32(R, "R") : null;
     const out = new Float32Array(1);
     for (let z = 0; z < batch; z++) for (let i = 0; i < m; i++) for (let j = 0; j < n; j++) {
       let sum = 0;
       for (let x = 0; x < k; x++) sum += a[z * sAb + i * sA0 + x * sA1] * b[z * sBb + x * sB0 + j * sB1];
-      out[0] = sum * alpha;
+      out[0] = sum; // the device accumulates in fp32: alpha scales an fp32 value
+      out[0] = out[0] * alpha;
       if (c) out[0] += c[i * sC0 + j * sC1] * beta;
-      const off = (z * m + i) * n + j;
+      const off = z * sYb + i * sY0 + j;
       if (r) out[0] += r[off];
       y[off] = epi === 1 ? reluJs(out[0]) : out[0];
     }

@@ -246,6 +246,55 @@ test("fusion: Conv+Add+Relu, Conv+Relu, MatMul+bias+Relu, MatMul+residual; share
 });
 
 // ---- hip tensors over the fake native -----------------------------------------------------------
+test("fusion: attention block -- Transposes, scale and head merge ride on the MatMuls; bias then residual", () => {
+  const f32init = (name, dims, values) => ({ name, dims, dataType: 1, floatData: values });
+  const nd = (opType, input, output, attrs) => ({
+    opType, input, output, name: output[0], attribute: (attrs || []),
+  });
+  const perm = (p) => [{ name: "perm", type: 7, ints: p, floats: [], strings: [] }];
+  const model = {
+    graph: {
+      node: [
+        nd("Transpose", ["q3"], ["qh"], perm([1, 0, 2])),
+        nd("Transpose", ["k3"], ["kt"], perm([1, 2, 0])),
+        nd("Transpose", ["v3"], ["vh"], perm([1, 0, 2])),
+        nd("MatMul", ["qh", "kt"], ["scores"]),
+        nd("Mul", ["scores", "scale"], ["scaled"]),
+        nd("Softmax", ["scaled"], ["attn"]),
+        nd("MatMul", ["attn", "vh"], ["ctx"]),
+        nd("Transpose", ["ctx"], ["ctx_t"], perm([1, 0, 2])),
+        nd("Reshape", ["ctx_t", "shape"], ["merged"]),
+        nd("MatMul", ["merged", "w"], ["o_mm"]),
+        nd("Add", ["o_mm", "b"], ["o_lin"]),
+        nd("Add", ["src", "o_lin"], ["res"]),
+        nd("Transpose", ["res"], ["res_t"], perm([1, 0])), // rank 2: stays a node
+        nd("MatMul", ["res_t", "w2"], ["out"]),
+      ],
+      initializer: [f32init("scale", [], [0.125]), f32init("b", [4], [0, 0, 0, 0]), f32init("w", [4, 4], new Array(16).fill(1)),
+        f32init("w2", [4, 4], new Array(16).fill(1))],
+      input: [], output: [{ name: "out" }],
+    },
+  };
+  assert.strictEqual(fuseForHip(model), 3);
+  const ops = model.graph.node.map((n) => n.opType);
+  assert.deepStrictEqual(ops, ["WebDNNHipFusedMatMul", "Softmax", "WebDNNHipFusedMatMul", "Reshape", "WebDNNHipFusedMatMul", "Transpose", "MatMul"]);
+  const attr = (node, name) => node.attribute.find((a) => a.name === name);
+  const [scores, , ctx, , proj] = model.graph.node;
+  assert.deepStrictEqual(scores.input, ["q3", "k3"]);
+  assert.deepStrictEqual(attr(scores, "perm_a").ints, [1, 0, 2]);
+  assert.deepStrictEqual(attr(scores, "perm_b").ints, [1, 2, 0]);
+  assert.strictEqual(attr(scores, "alpha").f, 0.125);
+  assert.deepStrictEqual(scores.output, ["scaled"]);
+  assert.deepStrictEqual(ctx.input, ["attn", "v3"]);
+  assert.deepStrictEqual(attr(ctx, "perm_b").ints, [1, 0, 2]);
+  assert.deepStrictEqual(attr(ctx, "perm_y").ints, [1, 0, 2]);
+  assert.deepStrictEqual(ctx.output, ["ctx_t"]);
+  assert.deepStrictEqual(proj.input, ["merged", "w", "b", "src"]);
+  assert.strictEqual(attr(proj, "has_bias").i, 1);
+  assert.strictEqual(attr(proj, "has_residual").i, 1);
+  assert.deepStrictEqual(proj.output, ["res"]);
+});
+
 test("HipTensor: alias shares one reference-counted buffer; data round trip; use after dispose throws", async () => {
   const cpu = new WebDNNCPUContextImpl();
   const ctx = new WebDNNHipContextImpl(cpu, { native: fakeNative, contractionTile: 3, splitK: 2 });

@@ -979,3 +979,45 @@ def test_conv3x3_lds_tile_kernel_every_tile_shape(ctx, tile):
             ctx.set_option("split_k", -1)
         assert_close_max(got, want, GEMM_TOL, "tile %d %s" % (tile, (n, cin, h, w, cout)))
         assert_close_max(cut, ref.unary("Relu", want), GEMM_TOL, "tile %d split 3" % tile)
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(8, 850, 32, 850), (8, 100, 32, 100), (3, 70, 50, 33), (2, 64, 64, 256)])
+def test_gemm_ex_writes_the_result_where_a_transpose_would_put_it(ctx, batch, m, n, k):
+    """wdh_gemm_ex with sYb = n, sY0 = batch*n stores [batch, m, n] as [m, batch, n] (attention heads
+    merged back); operands read through the strides an absorbed Transpose leaves behind."""
+    rng = np.random.default_rng(batch * 1000 + m)
+    # A as [m, batch, k] (tokens, heads, d) read as [batch, m, k]; B as [k_tokens.., ] read transposed
+    A_store = rng.uniform(-1, 1, (m, batch, k)).astype(np.float32)
+    B_store = rng.uniform(-1, 1, (n, batch, k)).astype(np.float32)      # B[b, x, j] = B_store[j, b, x]
+    A = np.ascontiguousarray(A_store.transpose(1, 0, 2))
+    B = np.ascontiguousarray(B_store.transpose(1, 2, 0))
+    ta, tb = ctx.move_tensor(A_store), ctx.move_tensor(B_store)
+    want = np.stack([ref.gemm(A[b], B[b], None, 0.25, 1.0) for b in range(batch)])
+    for split in (-1, 3):
+        y = ctx.empty_tensor([m, batch, n])
+        y.set_data(np.full((m, batch, n), np.nan, np.float32))
+        try:
+            ctx.set_option("split_k", split)
+            capi.call("wdh_gemm_ex", ta.handle, tb.handle, 0, y.handle, batch, m, n, k,
+                      k, batch * k, 1, k, 1, batch * k, 0, 0, 0.25, 1.0, 0, 0, n, batch * n)
+        finally:
+            ctx.set_option("split_k", -1)
+        got = y.get_data()
+        assert_close_max(got.transpose(1, 0, 2), want, GEMM_TOL, "interleaved result, split %d" % split)
+        # the same product stored batch-major must hold the same bits
+        d = ctx.empty_tensor([batch, m, n])
+        try:
+            ctx.set_option("split_k", split)
+            capi.call("wdh_gemm", ta.handle, tb.handle, 0, d.handle, batch, m, n, k,
+                      k, batch * k, 1, k, 1, batch * k, 0, 0, 0.25, 1.0, 0, 0)
+        finally:
+            ctx.set_option("split_k", -1)
+        assert_bit_exact(got.transpose(1, 0, 2), d.get_data(), "same sums, other addresses")
+        y.dispose(); d.dispose()
+    y = ctx.empty_tensor([m, batch, n])
+    with pytest.raises(capi.HipError):      # rows would overlap
+        capi.call("wdh_gemm_ex", ta.handle, tb.handle, 0, y.handle, batch, m, n, k,
+                  k, batch * k, 1, k, 1, batch * k, 0, 0, 1.0, 1.0, 0, 0, n, n)
+    with pytest.raises(capi.HipError):      # row stride below the row length
+        capi.call("wdh_gemm_ex", ta.handle, tb.handle, 0, y.handle, batch, m, n, k,
+                  k, batch * k, 1, k, 1, batch * k, 0, 0, 1.0, 1.0, 0, 0, m * n, n - 1)

@@ -46,6 +46,10 @@ SIGNATURES = {
                             _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
                             _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_float,
                             _c.c_int, c_buf]),
+    "wdh_gemm_ex": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
+                               _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+                               _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_float,
+                               _c.c_int, c_buf, _c.c_int64, _c.c_int64]),
     "wdh_gemm_static": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
                                    _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
                                    _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_float,

@@ -192,6 +192,7 @@ struct Params {
   long long sAb, sA0, sA1;   // A[b, i, x] = A[b*sAb + i*sA0 + x*sA1]
   long long sBb, sB0, sB1;   // B[b, x, j] = B[b*sBb + x*sB0 + j*sB1]
   long long sC0, sC1;
+  long long sYb, sY0;        // Gemm/MatMul: Y[b, i, j] = Y[b*sYb + i*sY0 + j] (and R alike)
   float alpha, beta;
   int epilogue;
   int tiles_m, tiles_n;
@@ -210,7 +211,7 @@ struct Params {
   int fast;         // every operand spans less than 2 GiB: descriptor loads allowed
   int a_bytes;      // fast: bytes of one z of A / of B (conv: of X from the first byte
   int b_bytes;      //       of a group to the end of the tensor, plus the padding shift)
-  int y_bytes;      // > 0: bytes of one z of Y (conv: of all of Y), below 2 GiB, and C spans
+  int y_bytes;      // > 0: bytes of the span of Y over all z, below 2 GiB, and C spans
   int c_bytes;      //      c_bytes (< 2 GiB): whole tiles may use the descriptor epilogue
   ConvGeom cv;
 };
@@ -478,7 +479,7 @@ __device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int
       off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
       if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
     } else {
-      off = ((long long)bz * p.m + row) * p.n + col;
+      off = (long long)bz * p.sYb + (long long)row * p.sY0 + col;
       if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
     }
     if (p.R) y = y + p.R[off];
@@ -524,9 +525,11 @@ __device__ __forceinline__ void finish_tile(const Params &p,
   // differ) and one scalar offset per accumulator row, so a stored element costs
   // no address arithmetic, no bounds test and no change of the execution mask.
   if (p.y_bytes > 0 && row0 + BM <= p.m && col0 + BN <= p.n) {
-    const long long zoff = CONV ? 0 : (long long)bz * p.m * p.n;
-    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, p.y_bytes);
-    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, p.y_bytes);
+    // (Gemm: the window runs from this z's first element to the end of the span all z cover)
+    const long long zoff = CONV ? 0 : (long long)bz * p.sYb;
+    const int y_window = p.y_bytes - (int)(zoff * 4);
+    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, y_window);
+    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, y_window);
     const rsrc_t rsrc_c = make_rsrc(p.C ? p.C : p.Y, p.C ? p.c_bytes : 0);
 #pragma unroll
     for (int nt = 0; nt < NT; nt++) {
@@ -542,7 +545,7 @@ __device__ __forceinline__ void finish_tile(const Params &p,
         cstride = 1;
       } else {
         ybase = col;
-        ystride = p.n;
+        ystride = (int)p.sY0;
         voff_c = (int)((4 * half * p.sC0 + col * p.sC1) * 4);
         cstride = (int)p.sC0;
       }
@@ -594,8 +597,8 @@ __device__ __forceinline__ void finish_tile(const Params &p,
       ybase = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g) * ohw + q;
       ystride = ohw;
     } else {
-      ybase = (long long)bz * p.m * p.n + colc;
-      ystride = p.n;
+      ybase = (long long)bz * p.sYb + colc;
+      ystride = p.sY0;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) {
@@ -1143,7 +1146,7 @@ __global__ void contraction_strided_kernel(Params p) {
     acc = __builtin_fmaf(A[(long long)x * p.sA1], B[(long long)x * p.sB0], acc);
   float y = p.alpha * acc;
   if (p.C) y = __builtin_fmaf(p.C[(long long)i * p.sC0 + (long long)j * p.sC1], p.beta, y);
-  long long off = (long long)bz * total + idx;
+  long long off = (long long)bz * p.sYb + (long long)i * p.sY0 + j;
   if (p.R) y = y + p.R[off];
   if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
   p.Y[off] = y;
@@ -1475,6 +1478,15 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
                         int64_t sA0, int64_t sA1, int64_t sBb, int64_t sB0,
                         int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
                         float beta, int epilogue, wdh_buf hR) {
+  return wdh_gemm_ex(hA, hB, hC, hY, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1, alpha, beta,
+                     epilogue, hR, (int64_t)m * n, n);
+}
+
+extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
+                           int batch, int m, int n, int k, int64_t sAb,
+                           int64_t sA0, int64_t sA1, int64_t sBb, int64_t sB0,
+                           int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
+                           float beta, int epilogue, wdh_buf hR, int64_t sYb, int64_t sY0) {
   WDH_REQUIRE_INIT();
   if (batch < 0 || m < 0 || n < 0 || k < 0)
     return fail(WDH_EINVAL, "wdh_gemm: negative extent (batch=%d m=%d n=%d k=%d)",
@@ -1488,6 +1500,13 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
     return fail(WDH_EINVAL, "wdh_gemm: unknown epilogue %d", epilogue);
   const long long out_elems = (long long)batch * m * n;
   if (out_elems == 0) return WDH_OK;
+  // Y (and R) rows are contiguous; rows and batch entries may be spaced out, either batch
+  // entries apart (sYb >= m*sY0) or interleaved row by row (sY0 >= batch*sYb)
+  if (sY0 < n || sYb < 0 ||
+      (batch > 1 && !(sYb >= (int64_t)m * sY0 || (sYb >= n && sY0 >= (int64_t)batch * sYb))))
+    return fail(WDH_EINVAL, "wdh_gemm: result strides (%lld, %lld) make rows overlap", (long long)sYb,
+                (long long)sY0);
+  const long long y_span = span(batch, sYb, m, sY0, n, 1);
 
   Params p = {};
   void *ptr;
@@ -1503,11 +1522,12 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
     p.C = (const float *)ptr;
   }
   if (hR) {
-    if (!wdh::operand(hR, (size_t)out_elems * 4, "wdh_gemm: R", &ptr)) return WDH_EINVAL;
+    if (!wdh::operand(hR, (size_t)y_span * 4, "wdh_gemm: R", &ptr)) return WDH_EINVAL;
     p.R = (const float *)ptr;
   }
-  if (!wdh::operand(hY, (size_t)out_elems * 4, "wdh_gemm: Y", &ptr)) return WDH_EINVAL;
+  if (!wdh::operand(hY, (size_t)y_span * 4, "wdh_gemm: Y", &ptr)) return WDH_EINVAL;
   p.Y = (float *)ptr;
+  p.sYb = sYb; p.sY0 = sY0;
   p.m = m; p.n = n; p.k = k;
   p.sAb = sAb; p.sA0 = sA0; p.sA1 = sA1;
   p.sBb = sBb; p.sB0 = sB0; p.sB1 = sB1;
@@ -1554,7 +1574,7 @@ extern "C" int wdh_gemm(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   p.a_bytes = p.fast ? (int)a_bytes : 0;
   p.b_bytes = p.fast ? (int)b_bytes : 0;
   {
-    const long long y_bytes = (long long)m * n * 4;
+    const long long y_bytes = y_span * 4;
     const long long c_bytes = p.C ? span(1, 0, m, p.sC0, n, p.sC1) * 4 : 0;
     const bool ok = g_descriptors && y_bytes < 0x7fffffffLL && c_bytes < 0x7fffffffLL;
     p.y_bytes = ok ? (int)y_bytes : 0;

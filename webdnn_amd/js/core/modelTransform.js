@@ -8,6 +8,7 @@
 // node of a backend-specific op type.
 const { getLogger } = require("../logging");
 const { AttributeType } = require("./onnxProto");
+const { tensorProtoToArray } = require("../operators/operatorUtil");
 
 const logger = getLogger("WebDNN.modelTransform");
 
@@ -41,15 +42,32 @@ function intAttr(name, value) {
   return { name, i: value, type: AttributeType.INT, floats: [], ints: [], strings: [] };
 }
 
+function intsAttr(name, values) {
+  return { name, type: AttributeType.INTS, floats: [], ints: values.slice(), strings: [] };
+}
+
+function floatAttr(name, value) {
+  return { name, f: value, type: AttributeType.FLOAT, floats: [], ints: [], strings: [] };
+}
+
 function stringAttr(name, value) {
   return { name, s: Buffer.from(value, "utf-8"), type: AttributeType.STRING, floats: [], ints: [], strings: [] };
 }
 
 // Conv [+ Add(residual)] [+ Relu]  ->  WebDNNHipFusedConv
-// MatMul [+ Add(bias | residual)] [+ Relu]  ->  WebDNNHipFusedMatMul
-// A link of the chain is absorbed only when its input has no other consumer, so no
-// intermediate tensor that something else reads disappears.  The fused node takes the
-// place of the chain's last node: everything it reads has been produced by then.
+// [Transpose ->] MatMul [* constant scalar] [+ Add(bias)] [+ Add(residual)] [+ Relu | -> Transpose]
+//                                                                        ->  WebDNNHipFusedMatMul
+// A link of the chain is absorbed only when the tensor between the two nodes has no other
+// reader, so no intermediate tensor that something else reads disappears.  The fused node
+// takes the place of the chain's last node: everything it reads has been produced by then.
+//
+// What the MatMul forms cost nothing to absorb (the kernel already has the means):
+//   a Transpose that feeds only this MatMul   -> the operand is read through permuted strides
+//   a Mul by a one-element constant           -> the product's alpha (the accumulator is fp32,
+//                                                so f32(alpha * acc) is what the Mul would store)
+//   a Transpose(1,0,2) of the rank-3 result   -> the rows are written where the Transpose
+//                                                would have put them
+// which is the whole head split / scale / head merge of an attention block.
 function fuseForHip(model) {
   const graph = model.graph;
   const nodes = graph.node;
@@ -61,9 +79,27 @@ function fuseForHip(model) {
   for (const init of graph.initializer) initializers.set(init.name, init);
 
   const readerOf = new Map(); // tensor name -> index of its only reader
+  const producerOf = new Map(); // tensor name -> index of the node that writes it
   nodes.forEach((node, idx) => {
     for (const name of node.input) if (consumers.get(name) === 1) readerOf.set(name, idx);
+    for (const name of node.output) producerOf.set(name, idx);
   });
+  const permOf = (node) => {
+    const attr = node.attribute.find((a) => a.name === "perm");
+    return attr && attr.ints ? attr.ints.map(Number) : [];
+  };
+  // value of a one-element float constant, or null
+  const scalarConstant = (name) => {
+    const init = initializers.get(name);
+    if (!init) return null;
+    let t;
+    try {
+      t = tensorProtoToArray(init);
+    } catch (e) {
+      return null;
+    }
+    return t.dataType === "float32" && t.data.length === 1 ? t.data[0] : null;
+  };
 
   const removed = new Set();
   let fusedCount = 0;
@@ -78,54 +114,94 @@ function fuseForHip(model) {
     let hasBias = isConv && inputs.length > 2;
     let hasResidual = false;
     let activation = "";
+    let alpha = null;
+    const perms = { a: [], b: [], y: [] };
     let tail = i; // index of the last absorbed node
     let cur = head.output[0];
     const absorbed = [];
+    const onlyReader = (name) => {
+      const idx = readerOf.get(name);
+      return idx !== undefined && !removed.has(idx) ? idx : undefined;
+    };
 
-    // + Add
-    let next = readerOf.get(cur);
-    if (next !== undefined && !removed.has(next) && nodes[next].opType === "Add" && nodes[next].input.length === 2) {
-      const add = nodes[next];
-      const other = add.input[0] === cur ? add.input[1] : add.input[0];
-      if (other !== cur) {
-        const init = initializers.get(other);
-        if (!isConv && !hasBias && init && init.dims.length <= 1) {
-          // MatMul + constant vector: a bias along the last axis
-          inputs.push(other);
-          hasBias = true;
+    if (!isConv) {
+      // Transpose -> operand
+      ["a", "b"].forEach((which, k) => {
+        const src = producerOf.get(inputs[k]);
+        if (src === undefined || removed.has(src) || consumers.get(inputs[k]) !== 1) return;
+        const t = nodes[src];
+        const perm = permOf(t);
+        if (t.opType !== "Transpose" || perm.length !== 3) return; // rank 3: [batch, rows, columns]
+        perms[which] = perm;
+        inputs[k] = t.input[0];
+        absorbed.push(src);
+      });
+      // * constant scalar
+      const next = onlyReader(cur);
+      if (next !== undefined && nodes[next].opType === "Mul" && nodes[next].input.length === 2) {
+        const mul = nodes[next];
+        const other = mul.input[0] === cur ? mul.input[1] : mul.input[0];
+        const value = other !== cur ? scalarConstant(other) : null;
+        if (value !== null) {
+          alpha = value;
           absorbed.push(next);
           tail = next;
-          cur = add.output[0];
-        } else if (!init) {
-          // an activation tensor: residual connection
-          inputs.push(other);
-          hasResidual = true;
-          absorbed.push(next);
-          tail = next;
-          cur = add.output[0];
+          cur = mul.output[0];
         }
       }
     }
+    // + Add (a constant vector after a MatMul: bias; an activation tensor: residual), twice at most:
+    // bias first, then the residual, the order in which the epilogue adds them
+    for (let round = 0; round < 2 && !hasResidual; round++) {
+      const next = onlyReader(cur);
+      if (next === undefined || nodes[next].opType !== "Add" || nodes[next].input.length !== 2) break;
+      const add = nodes[next];
+      const other = add.input[0] === cur ? add.input[1] : add.input[0];
+      if (other === cur) break;
+      const init = initializers.get(other);
+      if (!isConv && !hasBias && init && init.dims.length <= 1) {
+        inputs.push(other);
+        hasBias = true;
+      } else if (!init) {
+        inputs.push(other);
+        hasResidual = true;
+      } else {
+        break;
+      }
+      absorbed.push(next);
+      tail = next;
+      cur = add.output[0];
+    }
     // + Relu
-    next = readerOf.get(cur);
-    if (next !== undefined && !removed.has(next) && nodes[next].opType === "Relu") {
+    let next = onlyReader(cur);
+    if (next !== undefined && nodes[next].opType === "Relu") {
       activation = "Relu";
+      absorbed.push(next);
+      tail = next;
+      cur = nodes[next].output[0];
+    } else if (!isConv && next !== undefined && nodes[next].opType === "Transpose" && !hasBias && !hasResidual &&
+      permOf(nodes[next]).join() === "1,0,2") {
+      // -> Transpose(1,0,2): heads merged back
+      perms.y = [1, 0, 2];
       absorbed.push(next);
       tail = next;
       cur = nodes[next].output[0];
     }
     if (absorbed.length === 0) continue;
 
+    const extra = [
+      intAttr("has_bias", hasBias ? 1 : 0),
+      intAttr("has_residual", hasResidual ? 1 : 0),
+      stringAttr("activation", activation),
+    ];
+    if (alpha !== null) extra.push(floatAttr("alpha", alpha));
+    for (const which of ["a", "b", "y"]) if (perms[which].length) extra.push(intsAttr("perm_" + which, perms[which]));
     const fused = {
       input: inputs,
       output: [cur],
       name: nodes[tail].name,
       opType: isConv ? "WebDNNHipFusedConv" : "WebDNNHipFusedMatMul",
-      attribute: head.attribute.concat([
-        intAttr("has_bias", hasBias ? 1 : 0),
-        intAttr("has_residual", hasResidual ? 1 : 0),
-        stringAttr("activation", activation),
-      ]),
+      attribute: head.attribute.concat(extra),
       domain: "webdnn.hip",
     };
     removed.add(i);

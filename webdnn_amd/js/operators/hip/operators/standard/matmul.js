@@ -1,9 +1,26 @@
 "use strict";
 // MatMul (result rank 2 or 3, as the CPU operator) and its fused forms.
-// Semantics: src/descriptor_runner/operators/cpu/operators/standard/matmul.ts:11-111.
+// Semantics: src/descriptor_runner/operators/cpu/operators/standard/matmul.ts:11-111; the
+// absorbed Transposes follow CPUTranspose (transpose.ts:12-168).
 const { MatMul } = require("../../../base/matmul");
-const { broadcastUni, getAttrInt, getAttrString } = require("../../../operatorUtil");
+const { broadcastUni, getAttrFloat, getAttrInt, getAttrInts, getAttrString } = require("../../../operatorUtil");
+const { permutedView, denseStrides } = require("../../../shapes");
 const { addThenActivate } = require("./conv");
+
+// An operand as the product sees it: dims and element strides.  With a permutation absorbed
+// from a Transpose the strides are the tensor's own, permuted, and nothing is copied -- unless
+// neither of the last two axes ends up contiguous, which the kernel could only serve one
+// element at a time: then the Transpose is carried out after all (temp = its result).
+function operandView(context, tensor, perm) {
+  if (!perm.length) return { dims: tensor.dims, strides: tensor.strides, temp: null };
+  const { outShape, inStrides } = permutedView(tensor.dims, tensor.strides, perm);
+  const rank = outShape.length;
+  const contiguous = (axis) => outShape[axis] === 1 || inStrides[axis] === 1;
+  if (rank >= 2 && (contiguous(rank - 1) || contiguous(rank - 2))) return { dims: outShape, strides: inStrides, temp: null };
+  const temp = context.emptyTensor(outShape, tensor.dataType);
+  context.native.transpose(tensor.handle, temp.handle, outShape, inStrides);
+  return { dims: outShape, strides: temp.strides, temp };
+}
 
 class HipMatMul extends MatMul {
   // fused: inputs are (A, B[, bias][, residual]) as announced by the node's attributes
@@ -13,6 +30,10 @@ class HipMatMul extends MatMul {
     this.hasBias = false;
     this.hasResidual = false;
     this.activation = "";
+    this.alpha = 1.0;
+    this.permA = [];
+    this.permB = [];
+    this.permY = [];
   }
 
   initialize(attribute) {
@@ -24,41 +45,54 @@ class HipMatMul extends MatMul {
       if (this.activation !== "" && this.activation !== "Relu") {
         throw new Error(`FusedMatMul: activation ${this.activation} is not supported`);
       }
+      this.alpha = getAttrFloat(attribute, "alpha", 1.0);
+      this.permA = getAttrInts(attribute, "perm_a", []);
+      this.permB = getAttrInts(attribute, "perm_b", []);
+      this.permY = getAttrInts(attribute, "perm_y", []);
     }
   }
 
   async run(context, inputs) {
     context.assertsHipTensorArray(inputs);
-    const inputA = inputs[0],
-      inputB = inputs[1];
     let next = 2;
     const bias = this.hasBias ? inputs[next++] : null;
     const residual = this.hasResidual ? inputs[next++] : null;
     for (const t of inputs) if (t.dataType !== "float32") throw new Error("only float32 is supported");
-    const { resultDims, resultDimsAfterSqueeze, stridesA, stridesB, innerProductLength } = this.calcShape(
-      inputA.dims,
-      inputB.dims
-    );
-    let batch, m, n, sAb, sBb;
-    const nd = resultDims.length;
-    if (nd === 2) {
-      batch = 1;
-      sAb = sBb = 0;
-    } else if (nd === 3) {
-      batch = resultDims[0];
-      sAb = stridesA[0];
-      sBb = stridesB[0];
-    } else {
-      throw new Error("MatMul: result rank >= 4 is not supported");
+    const viewA = operandView(context, inputs[0], this.permA),
+      viewB = operandView(context, inputs[1], this.permB);
+    try {
+      return [this.product(context, inputs[0], inputs[1], viewA, viewB, bias, residual)];
+    } finally {
+      if (viewA.temp) viewA.temp.dispose();
+      if (viewB.temp) viewB.temp.dispose();
     }
-    m = resultDims[nd - 2];
-    n = resultDims[nd - 1];
+  }
+
+  product(context, tensorA, tensorB, viewA, viewB, bias, residual) {
+    const plan = this.calcShape(viewA.dims, viewB.dims);
+    const { resultDims, resultDimsAfterSqueeze, innerProductLength } = plan;
+    const nd = resultDims.length;
+    if (nd !== 2 && nd !== 3) throw new Error("MatMul: result rank >= 4 is not supported");
+    // strides of a permuted view replace the dense ones the plan assumes (same broadcasting rule:
+    // a batch axis of extent 1 is re-read)
+    const stridesOf = (view, planned) => {
+      if (view.dims.length !== nd) return planned; // rank-1 / lower-rank operands are never permuted views
+      return view.strides.map((s, axis) => (axis < nd - 2 && view.dims[axis] === 1 ? 0 : s));
+    };
+    const stridesA = stridesOf(viewA, plan.stridesA),
+      stridesB = stridesOf(viewB, plan.stridesB);
+    let batch = nd === 3 ? resultDims[0] : 1,
+      m = resultDims[nd - 2];
+    const n = resultDims[nd - 1];
+    let sAb = nd === 3 ? stridesA[0] : 0;
+    const sBb = nd === 3 ? stridesB[0] : 0;
     const sA0 = stridesA[nd - 2],
       sA1 = stridesA[nd - 1],
       sB0 = stridesB[nd - 2],
       sB1 = stridesB[nd - 1];
+    const mergeHeads = this.permY.length === 3 && nd === 3 && resultDimsAfterSqueeze.length === 3;
     // a batch that only broadcasts B over dense rows of A is one tall GEMM
-    if (batch > 1 && sBb === 0 && sAb === m * sA0 && !residual && (!bias || bias.ndim <= 1)) {
+    if (batch > 1 && sBb === 0 && sAb === m * sA0 && !residual && (!bias || bias.ndim <= 1) && !this.permY.length) {
       m *= batch;
       batch = 1;
       sAb = 0;
@@ -70,19 +104,40 @@ class HipMatMul extends MatMul {
     const sameShape = residual && residual.ndim === resultDimsAfterSqueeze.length &&
       residual.dims.every((d, i) => d === resultDimsAfterSqueeze[i]);
     const inEpilogue = !residual || sameShape;
-    const output = context.emptyTensor(resultDimsAfterSqueeze, "float32");
-    context.native.gemm(inputA.handle, inputB.handle, bias ? bias.handle : 0, output.handle, batch, m, n,
-      innerProductLength, sAb, sA0, sA1, sBb, sB0, sB1, strideC[0], strideC[1], 1.0, 1.0,
-      inEpilogue && this.activation === "Relu" ? 1 : 0, sameShape ? residual.handle : 0);
-    if (inEpilogue) return [output];
-    return [addThenActivate(context, output, residual, this.activation)];
+    const epilogue = inEpilogue && this.activation === "Relu" ? 1 : 0;
+    if (mergeHeads) {
+      // [batch, m, n] written as [m, batch, n]: what Transpose(1,0,2) would produce
+      const output = context.emptyTensor([m, batch, n], "float32");
+      context.native.gemmEx(operandHandle(viewA, tensorA), operandHandle(viewB, tensorB), 0, output.handle, batch, m, n,
+        innerProductLength, sAb, sA0, sA1, sBb, sB0, sB1, 0, 0, this.alpha, 1.0, 0, 0, n, batch * n);
+      return output;
+    }
+    let output = context.emptyTensor(resultDimsAfterSqueeze, "float32");
+    context.native.gemm(operandHandle(viewA, tensorA), operandHandle(viewB, tensorB), bias ? bias.handle : 0,
+      output.handle, batch, m, n, innerProductLength, sAb, sA0, sA1, sBb, sB0, sB1, strideC[0], strideC[1],
+      this.alpha, 1.0, epilogue, sameShape ? residual.handle : 0);
+    if (!inEpilogue) output = addThenActivate(context, output, residual, this.activation);
+    if (this.permY.length) {
+      // a result Transpose that could not be folded into the store (rank other than 3)
+      const { outShape, inStrides } = permutedView(output.dims, denseStrides(output.dims), this.permY);
+      const moved = context.emptyTensor(outShape, "float32");
+      context.native.transpose(output.handle, moved.handle, outShape, inStrides);
+      output.dispose();
+      output = moved;
+    }
+    return output;
   }
+}
+
+// the buffer an operand is read from: the materialised Transpose if there had to be one
+function operandHandle(view, tensor) {
+  return view.temp ? view.temp.handle : tensor.handle;
 }
 
 function getOpEntries() {
   return [
     { opType: "MatMul", backend: "hip", opsetMin: 1, factory: () => new HipMatMul(false) },
-    // produced by the hip fusion pass (MatMul + Add [+ Relu] / + residual Add)
+    // produced by the hip fusion pass ([Transpose ->] MatMul [* scalar] [+ bias] [+ residual] [+ Relu | -> Transpose])
     { opType: "WebDNNHipFusedMatMul", backend: "hip", opsetMin: 1, factory: () => new HipMatMul(true) },
   ];
 }

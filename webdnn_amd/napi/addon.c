@@ -269,6 +269,18 @@ FN(js_gemm) {
   return make_undefined(env);
 }
 
+FN(js_gemm_ex) {
+  ARGS("wdh_gemm_ex", 22);
+  I64(0, A); I64(1, B); I64(2, C); I64(3, Y); I64(4, batch); I64(5, m); I64(6, n); I64(7, k);
+  I64(8, sAb); I64(9, sA0); I64(10, sA1); I64(11, sBb); I64(12, sB0); I64(13, sB1);
+  I64(14, sC0); I64(15, sC1);
+  F64(16, alpha); F64(17, beta);
+  I64(18, epilogue); I64(19, R); I64(20, sYb); I64(21, sY0);
+  CHECK(wdh_gemm_ex(A, B, C, Y, (int)batch, (int)m, (int)n, (int)k, sAb, sA0, sA1, sBb, sB0, sB1, sC0,
+                    sC1, (float)alpha, (float)beta, (int)epilogue, R, sYb, sY0));
+  return make_undefined(env);
+}
+
 FN(js_conv2d) {
   ARGS("wdh_conv2d", 22);
   I64(0, X); I64(1, W); I64(2, Bias); I64(3, Y);
@@ -429,7 +441,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"setOption", js_set_option}, {"alloc", js_alloc}, {"free", js_free}, {"write", js_write},
       {"read", js_read}, {"copy", js_copy}, {"sync", js_sync}, {"memStats", js_mem_stats},
       {"trim", js_trim}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
-      {"gemm", js_gemm}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
+      {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
       {"softmax", js_softmax}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
