@@ -78,6 +78,10 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       input rows of a tile in LDS and read the taps from there;
  *                       0 = they gather taps from global memory like every other
  *                       geometry (both forms compute the same sums).
+ *   "gemm_wavesplit"    1 (default) = a Gemm / MatMul with few result tiles and K >= 128
+ *                       runs as one launch of 32x32 blocks whose 16 wavefronts share K
+ *                       among themselves; 0 = it takes the ordinary tiles (K cut across
+ *                       workgroups, partial sums added by a second kernel).
  *   "descriptor_loads"  1 (default) = operands below 2 GiB are read and written
  *                       through buffer descriptors with 32-bit offsets; 0 = every
  *                       operand is treated as if it spanned 2 GiB or more (64-bit

@@ -1021,3 +1021,52 @@ def test_gemm_ex_writes_the_result_where_a_transpose_would_put_it(ctx, batch, m,
     with pytest.raises(capi.HipError):      # row stride below the row length
         capi.call("wdh_gemm_ex", ta.handle, tb.handle, 0, y.handle, batch, m, n, k,
                   k, batch * k, 1, k, 1, batch * k, 0, 0, 1.0, 1.0, 0, 0, m * n, n - 1)
+
+
+@pytest.mark.parametrize("n,cin,h,w,cout,group", [(3, 32, 10, 10, 40, 1), (1, 64, 50, 68, 70, 1), (5, 32, 6, 6, 24, 2),
+                                                  (2, 16, 2, 2, 8, 1)])
+def test_conv_1x1_in_place_with_a_ragged_last_tile(ctx, n, cin, h, w, cout, group):
+    """1x1 stride-1 convs read X as the B matrix also when the pixel count is no multiple of the tile
+    (DETR's 13600-, 3400- and 850-pixel stages): the last tile hangs over the end of the pixels."""
+    X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin // group, 1), nrm(cout)
+    R = nrm(n, cout, h, w)
+    got = hip_conv(ctx, X, W, B, None, group)
+    assert ctx.last_plan()["form"] == "conv 1x1, X in place"
+    assert_close_max(got, ref.conv(X, W, B, None, group), GEMM_TOL, "ragged in-place 1x1")
+    fused = hip_conv(ctx, X, W, B, None, group, epilogue="relu", R=R)
+    assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "ragged in-place 1x1 + residual + relu")
+
+
+@pytest.mark.parametrize("batch,m,n,k,tb", [(1, 850, 256, 256, 0), (1, 100, 256, 2048, 0), (8, 850, 32, 850, 0),
+                                            (1, 32, 1000, 2048, 1), (3, 70, 45, 333, 1), (1, 100, 92, 256, 0),
+                                            (8, 100, 100, 128, 1), (2, 33, 31, 1000, 0)])
+def test_small_products_cut_k_across_the_wavefronts_of_a_workgroup(ctx, batch, m, n, k, tb):
+    """Few result tiles, K >= 128: one launch of 32x32 blocks (gemm_wavesplit_kernel).  Against the
+    oracle, and against the ordinary tiles with a reduce pass (same products, another order)."""
+    rng = np.random.default_rng(m * 7 + k)
+    A = rng.uniform(-1, 1, (batch, m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    R = rng.standard_normal((batch, m, n)).astype(np.float32)
+    ta, tb_, tc, tr = (ctx.move_tensor(v) for v in (A, B, C, R))
+    sb = (k * n, 1, k) if tb else (k * n, n, 1)
+    out = {}
+    for mode in (1, 0):
+        y = ctx.empty_tensor([batch, m, n])
+        try:
+            ctx.set_option("gemm_wavesplit", mode)
+            capi.call("wdh_gemm", ta.handle, tb_.handle, tc.handle, y.handle, batch, m, n, k,
+                      m * k, k, 1, sb[0], sb[1], sb[2], 0, 1, 0.5, 2.0, 1, tr.handle)
+        finally:
+            ctx.set_option("gemm_wavesplit", 1)
+        out[mode] = (y.get_data(), ctx.last_plan())
+        y.dispose()
+    assert out[1][1]["tile"] == "32x32" and out[0][1]["tile"] != "32x32", (out[1][1], out[0][1])
+    want = np.stack([ref.gemm(A[b], B[b], C, 0.5, 2.0, 0, tb) for b in range(batch)])
+    want = ref.unary("Relu", ref.binary("Add", want, R))
+    assert_close_max(out[1][0], want, GEMM_TOL, "wave-split product")
+    assert_close_max(out[1][0], out[0][0], 1e-5, "wave-split vs tiles + reduce pass")
+    again = ctx.empty_tensor([batch, m, n])
+    capi.call("wdh_gemm", ta.handle, tb_.handle, tc.handle, again.handle, batch, m, n, k,
+              m * k, k, 1, sb[0], sb[1], sb[2], 0, 1, 0.5, 2.0, 1, tr.handle)
+    assert_bit_exact(again.get_data(), out[1][0], "same order every time")

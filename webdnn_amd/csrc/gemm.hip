@@ -1131,6 +1131,116 @@ __global__ __launch_bounds__(NTHREADS, BM == 64 ? (BN == 64 ? 4 : (BN == 128 ? 3
   finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0);
 }
 
+// ---- small products: K cut across the wavefronts of one workgroup -------------------
+// A product with few result tiles (a transformer's 850x256 linear layers, attention x V,
+// a classifier head) cannot fill the chip with 64x64 tiles, and cutting K across
+// workgroups costs a second launch to add the pieces up.  Here a workgroup of 16
+// wavefronts owns one 32x32 block of the result and every wavefront multiplies a 1/16
+// share of K for the whole block: operand fragments go from global memory straight into
+// the lanes the matrix core reads them from (A rows and k-contiguous B columns as 16-byte
+// pieces, an n-contiguous B as one element per k), the 16 partial blocks meet in LDS and
+// thread t adds up element t in wavefront order -- a fixed order, so results do not
+// depend on scheduling -- before the usual epilogue.  One launch, no workspace.
+constexpr int WS_WAVES = 16;
+template <bool B_IS_KC, bool VEC>
+__global__ __launch_bounds__(64 * WS_WAVES, 1) void gemm_wavesplit_kernel(Params p) {
+  __shared__ float part[WS_WAVES][16][64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 31, half = lane >> 5;
+  const int tiles_per_z = p.tiles_m * p.tiles_n;
+  const int bz = fdiv((int)blockIdx.x, p.fd_tiles_per_z);
+  const int tile = (int)blockIdx.x - bz * tiles_per_z;
+  const int tm = fdiv(tile, p.fd_group), tn = tile - tm * p.tiles_n;  // fd_group: division by tiles_n
+  const int row0 = tm * 32, col0 = tn * 32;
+
+  const rsrc_t rsrc_a = make_rsrc(p.A + (long long)bz * p.sAb, p.a_bytes);
+  const rsrc_t rsrc_b = make_rsrc(p.B + (long long)bz * p.sBb, p.b_bytes);
+  int ra = row0 + li;
+  ra = ra < p.m ? ra : p.m - 1;  // rows and columns past the edge are never stored
+  int cb = col0 + li;
+  cb = cb < p.n ? cb : p.n - 1;
+  const int lda = (int)p.sA0, ldb = B_IS_KC ? (int)p.sB1 : (int)p.sB0;
+  const int voff_a = (ra * lda + 4 * half) * 4;
+  const int voff_b = B_IS_KC ? (cb * ldb + 4 * half) * 4 : (4 * half * ldb + cb) * 4;
+
+  // this wavefront's share of K, in slabs of 16
+  const int kbeg = wave * p.kchunk;
+  const int kend = kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k;
+
+  f32x16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+  struct Frag {
+    f32x4 a[2], b[2];
+  };
+  // the 16 k of a slab are consumed in the order k = 8*(s/4) + 4*half + s%4, s = 0..7
+  auto fetch = [&](int k0, Frag &f) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      // (rows whose length is no multiple of four floats are not 16-byte aligned)
+      if (VEC) {
+        f.a[j] = buf_load4(rsrc_a, voff_a, (k0 + 8 * j) * 4);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) f.a[j][e] = buf_load(rsrc_a, voff_a + 4 * e, (k0 + 8 * j) * 4);
+      }
+      if (B_IS_KC && VEC) {
+        f.b[j] = buf_load4(rsrc_b, voff_b, (k0 + 8 * j) * 4);
+      } else if (B_IS_KC) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) f.b[j][e] = buf_load(rsrc_b, voff_b + 4 * e, (k0 + 8 * j) * 4);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) f.b[j][e] = buf_load(rsrc_b, voff_b, (k0 + 8 * j + e) * ldb * 4);
+      }
+    }
+    if (k0 + BK > p.k) {
+      // ragged end of K: what lies past it belongs to the next row (or to nobody)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (k0 + 8 * j + 4 * half + e >= p.k) {
+            f.a[j][e] = 0.0f;
+            f.b[j][e] = 0.0f;
+          }
+    }
+  };
+  auto multiply = [&](const Frag &f) {
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[s >> 2][s & 3], f.b[s >> 2][s & 3], acc, 0, 0, 0);
+  };
+  if (kbeg < kend) {
+    Frag cur, nxt;
+    fetch(kbeg, cur);
+    for (int k0 = kbeg; k0 < kend; k0 += BK) {
+      if (k0 + BK < kend) fetch(k0 + BK, nxt);
+      multiply(cur);
+      cur = nxt;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; r++) part[wave][r][lane] = acc[r];
+  __syncthreads();
+
+  // thread t owns element t of the block: accumulator register r = t / 64 of lane t % 64
+  const int r = tid >> 6;
+  float sum = 0.0f;
+#pragma unroll
+  for (int w = 0; w < WS_WAVES; w++) sum += part[w][r][lane];
+  const int row = row0 + 8 * (r >> 2) + 4 * half + (r & 3), col = col0 + li;
+  if (row >= p.m || col >= p.n) return;
+  float y = p.alpha * sum;
+  if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
+  const long long off = (long long)bz * p.sYb + (long long)row * p.sY0 + col;
+  if (p.R) y = y + p.R[off];
+  if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
+  p.Y[off] = y;
+}
+
 // Reference-order scalar kernel for operands that are dense in neither index
 // (never produced by the runner's dense tensors, kept so the entry point is total).
 __global__ void contraction_strided_kernel(Params p) {
@@ -1191,6 +1301,7 @@ int g_descriptors = 1;    // 0: every operand is treated as if it spanned 2 GiB 
 struct LastPlan { int bm, bn, split, form; long long full, tail; } g_last_plan = {};
 int g_last_form = 0;
 bool g_static_scratch = false;  // set for the duration of a wdh_gemm_static call
+int g_wavesplit = 1;      // 0: small products take the ordinary tiles too
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
 
 // How the tiles of one launch are spread over the chip.
@@ -1440,6 +1551,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     g_descriptors = value;
     return WDH_OK;
   }
+  if (strcmp(name, "gemm_wavesplit") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: gemm_wavesplit %d (use 0 or 1)", value);
+    g_wavesplit = value;
+    return WDH_OK;
+  }
   if (strcmp(name, "conv3x3_halo") == 0) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: conv3x3_halo %d (use 0 or 1)", value);
@@ -1580,6 +1697,33 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
     p.y_bytes = ok ? (int)y_bytes : 0;
     p.c_bytes = ok ? (int)c_bytes : 0;
   }
+  // Few result tiles and a K worth cutting: one launch with K cut across the wavefronts of a
+  // workgroup (gemm_wavesplit_kernel) instead of chunks in a workspace and a reduce pass
+  if (g_wavesplit && g_forced_tile < 0 && g_forced_split < 0 && useA_kc && p.fast && k >= 128) {
+    const long long blocks32 = (long long)((m + 31) / 32) * ((n + 31) / 32) * batch;
+    const long long tiles64 = (long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
+    if (blocks32 <= 4LL * wdh::compute_units() && tiles64 < 2LL * wdh::compute_units() &&
+        (useB_kc || (long long)(k - 1) * p.sB0 * 4 < 0x7fffffffLL)) {
+      p.tiles_m = (m + 31) / 32;
+      p.tiles_n = (n + 31) / 32;
+      p.nz = batch;
+      p.fd_tiles_per_z = make_fastdiv((long long)p.tiles_m * p.tiles_n);
+      p.fd_group = make_fastdiv(p.tiles_n);
+      p.kchunk = ((k + BK - 1) / BK + WS_WAVES - 1) / WS_WAVES * BK;  // slabs per wavefront, in elements
+      g_last_plan = {32, 32, WS_WAVES, useB_kc ? WDH_FORM_GEMM_KC : WDH_FORM_GEMM_MC, blocks32, 0};
+      const dim3 grid((unsigned)blocks32), block(64 * WS_WAVES);
+      if (useB_kc && vec)
+        hipLaunchKernelGGL((gemm_wavesplit_kernel<true, true>), grid, block, 0, wdh::stream(), p);
+      else if (useB_kc)
+        hipLaunchKernelGGL((gemm_wavesplit_kernel<true, false>), grid, block, 0, wdh::stream(), p);
+      else if (vec)
+        hipLaunchKernelGGL((gemm_wavesplit_kernel<false, true>), grid, block, 0, wdh::stream(), p);
+      else
+        hipLaunchKernelGGL((gemm_wavesplit_kernel<false, false>), grid, block, 0, wdh::stream(), p);
+      WDH_LAUNCH_CHECK();
+      return WDH_OK;
+    }
+  }
   if (useA_kc && useB_kc) return launch<true, B_KC>(p, batch, vec);
   if (useA_kc && !useB_kc) return launch<true, B_MC>(p, batch, vec);
   if (!useA_kc && useB_kc) return launch<false, B_KC>(p, batch, vec);
@@ -1679,12 +1823,13 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   const long long w_bytes = (long long)cout_g * kdim * 4;
   const bool small = g_descriptors && x_bytes < 0x7fffffffLL && w_bytes < 0x7fffffffLL;
   const bool vec = aligned16(p.A) && kdim % 4 == 0 && ((long long)cout_g * kdim) % 4 == 0;
-  // 1x1, stride 1, no padding: X is the B matrix as it lies (B_PIXELS), provided every tile
-  // and K slab is whole; a forced tile may be up to 256 columns wide
+  // 1x1, stride 1, no padding: X is the B matrix as it lies (B_PIXELS), provided every K slab
+  // is whole and four consecutive pixels never straddle two images.  The last tile may hang
+  // over the end of the pixels: its surplus columns read the next k row or, past the last
+  // image, the zeros the descriptor returns, and are never stored.
   const long long plane = (long long)h * w;
   if (small && vec && ntaps == 1 && sh == 1 && sw == 1 && pt == 0 && pl == 0 && pb == 0 && pr == 0 &&
-      plane % 4 == 0 && kdim % BK == 0 && aligned16(p.B) &&
-      npix % (g_forced_tile >= 0 ? 256 : 64) == 0) {
+      plane % 4 == 0 && kdim % BK == 0 && aligned16(p.B)) {
     p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
     p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
     p.sBb = (long long)c_in_g * plane; p.sB0 = plane; p.sB1 = 1;
