@@ -89,6 +89,8 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       convolution).  A test hook: it runs the large-operand code
  *                       on ordinary sizes. */
 int wdh_set_option(const char *name, int value);
+/* wdh_init also applies the options named in the environment variable WDH_OPTIONS
+ * ("name=value,name=value"), for hosts that cannot call wdh_set_option themselves. */
 
 /* How the most recent wdh_gemm / wdh_conv2d launch was laid out (for per-layer
  * reports; cf. the per-node records of measurePerformance,

@@ -1037,9 +1037,9 @@ def test_conv_1x1_in_place_with_a_ragged_last_tile(ctx, n, cin, h, w, cout, grou
     assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "ragged in-place 1x1 + residual + relu")
 
 
-@pytest.mark.parametrize("batch,m,n,k,tb", [(1, 850, 256, 256, 0), (1, 100, 256, 2048, 0), (8, 850, 32, 850, 0),
-                                            (1, 32, 1000, 2048, 1), (3, 70, 45, 333, 1), (1, 100, 92, 256, 0),
-                                            (8, 100, 100, 128, 1), (2, 33, 31, 1000, 0)])
+@pytest.mark.parametrize("batch,m,n,k,tb", [(1, 850, 256, 256, 0), (1, 850, 256, 2048, 0), (8, 850, 32, 850, 0),
+                                            (1, 200, 1000, 256, 1), (3, 70, 45, 333, 1), (1, 100, 92, 256, 0),
+                                            (8, 100, 100, 128, 1), (2, 33, 31, 500, 0)])
 def test_small_products_cut_k_across_the_wavefronts_of_a_workgroup(ctx, batch, m, n, k, tb):
     """Few result tiles, K >= 128: one launch of 32x32 blocks (gemm_wavesplit_kernel).  Against the
     oracle, and against the ordinary tiles with a reduce pass (same products, another order)."""
@@ -1070,3 +1070,12 @@ def test_small_products_cut_k_across_the_wavefronts_of_a_workgroup(ctx, batch, m
     capi.call("wdh_gemm", ta.handle, tb_.handle, tc.handle, again.handle, batch, m, n, k,
               m * k, k, 1, sb[0], sb[1], sb[2], 0, 1, 0.5, 2.0, 1, tr.handle)
     assert_bit_exact(again.get_data(), out[1][0], "same order every time")
+
+
+def test_few_blocks_with_a_long_k_keep_the_ordinary_tiles(ctx):
+    """The ResNet classifier head, [32,2048] x [1000,2048]^T: 32 blocks of 32x32 would leave the 8 MB of
+    weights to 32 workgroups; it stays with 64x64 tiles cut along K."""
+    A, B, C = uni(32, 2048), uni(1000, 2048), uni(1000)
+    got = hip_gemm(ctx, A, B, C, 1.0, 1.0, 0, 1)
+    assert ctx.last_plan()["tile"] == "64x64" and ctx.last_plan()["split"] > 1
+    assert_close_max(got, ref.gemm(A, B, C, 1.0, 1.0, 0, 1), GEMM_TOL, "classifier head")

@@ -1702,7 +1702,9 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   if (g_wavesplit && g_forced_tile < 0 && g_forced_split < 0 && useA_kc && p.fast && k >= 128) {
     const long long blocks32 = (long long)((m + 31) / 32) * ((n + 31) / 32) * batch;
     const long long tiles64 = (long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
+    // (few blocks each streaming a long K would leave the weights to a handful of CUs)
     if (blocks32 <= 4LL * wdh::compute_units() && tiles64 < 2LL * wdh::compute_units() &&
+        (blocks32 * 2 >= wdh::compute_units() || k <= 512) &&
         (useB_kc || (long long)(k - 1) * p.sB0 * 4 < 0x7fffffffLL)) {
       p.tiles_m = (m + 31) / 32;
       p.tiles_n = (n + 31) / 32;

@@ -7,6 +7,7 @@
 //  src/shader/wasm/pre.js:4-91, src/shader/wasm/src/core/allocation.cpp:4-15).
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <map>
@@ -195,6 +196,19 @@ int wdh_init(int device) {
   }
   g.device = device;
   g.ready = true;
+  // WDH_OPTIONS="name=value,name=value": wdh_set_option calls made on behalf of a caller that
+  // cannot make them itself (a model run through an unmodified host); unknown names are errors
+  if (const char *env = getenv("WDH_OPTIONS")) {
+    char buf[512];
+    snprintf(buf, sizeof(buf), "%s", env);
+    for (char *item = strtok(buf, ","); item; item = strtok(nullptr, ",")) {
+      char *eq = strchr(item, '=');
+      if (!eq) return fail(WDH_EINVAL, "WDH_OPTIONS: \"%s\" is not name=value", item);
+      *eq = '\0';
+      const int rc = wdh_set_option(item, atoi(eq + 1));
+      if (rc != WDH_OK) return rc;
+    }
+  }
   wdh::clear_error();
   return WDH_OK;
 }
