@@ -82,6 +82,11 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       runs as one launch of 32x32 blocks whose 16 wavefronts share K
  *                       among themselves; 0 = it takes the ordinary tiles (K cut across
  *                       workgroups, partial sums added by a second kernel).
+ *   "wide_stores"       1 (default) = whole result tiles whose rows are 16-byte aligned
+ *                       (Conv: output planes of a multiple of four pixels; Gemm: row and
+ *                       batch strides of Y that are multiples of four) are turned through
+ *                       LDS and stored 16 bytes per lane; 0 = every lane stores single
+ *                       elements (same arithmetic, same bits).
  *   "descriptor_loads"  1 (default) = operands below 2 GiB are read and written
  *                       through buffer descriptors with 32-bit offsets; 0 = every
  *                       operand is treated as if it spanned 2 GiB or more (64-bit

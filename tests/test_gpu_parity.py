@@ -1079,3 +1079,44 @@ def test_few_blocks_with_a_long_k_keep_the_ordinary_tiles(ctx):
     got = hip_gemm(ctx, A, B, C, 1.0, 1.0, 0, 1)
     assert ctx.last_plan()["tile"] == "64x64" and ctx.last_plan()["split"] > 1
     assert_close_max(got, ref.gemm(A, B, C, 1.0, 1.0, 0, 1), GEMM_TOL, "classifier head")
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
+def test_sixteen_byte_stores_hold_the_bits_of_four_byte_stores(ctx, tile):
+    """Whole tiles leave through LDS in 16-byte stores when the result's rows allow it
+    (wide_stores, on by default).  Same arithmetic, so the same bits as the per-element
+    stores: Gemm with a bias along n, along m, a full C, MatMul-style residual + Relu, and
+    Conv in all three forms with bias + residual + Relu.  Repeated, since a store that races
+    with the registers it reads shows only now and then."""
+    def both(run):
+        out = []
+        for wide in (0, 1):
+            try:
+                ctx.set_option("wide_stores", wide)
+                ctx.set_option("contraction_tile", tile)
+                out.append(run())
+            finally:
+                ctx.set_option("wide_stores", 1)
+                ctx.set_option("contraction_tile", -1)
+        return out
+
+    m, n, k = 1024, 1536, 96
+    A, B = uni(m, k), uni(k, n)
+    tA, tB = ctx.move_tensor(A), ctx.move_tensor(B)
+    for what, C in (("bias along n", uni(n)), ("bias along m", uni(m, 1)), ("full C", uni(m, n)), ("no C", None)):
+        tC = ctx.move_tensor(C) if C is not None else None
+        for rep in range(3):
+            narrow, wide = both(lambda: H.gemm(ctx, tA, tB, tC, 0.5, 2.0, epilogue="relu").get_data())
+            assert_bit_exact(wide, narrow, "gemm, %s, tile %d" % (what, tile))
+        assert_close_max(wide, ref.unary("Relu", ref.gemm(A, B, C, 0.5, 2.0)), GEMM_TOL, "gemm, " + what)
+    convs = [(4, 64, 56, 56, 64, 3, [1, 1, 1, 1], [1, 1]),    # LDS-tile form
+             (4, 64, 28, 28, 256, 1, [0, 0, 0, 0], [1, 1]),   # X in place
+             (4, 24, 30, 30, 80, 3, [1, 1, 1, 1], [2, 2]),    # gathered: 15x15 outputs, rows not 16-byte multiples
+             (4, 24, 32, 32, 80, 5, [2, 2, 2, 2], [2, 2])]    # gathered: 16x16 outputs
+    for n_, cin, h, w, cout, kk, pads, strides in convs:
+        X, W, Bv = uni(n_, cin, h, w, lo=0), he(cout, cin, kk), nrm(cout)
+        want = ref.conv(X, W, Bv, None, 1, None, pads, strides)
+        R = nrm(*want.shape)
+        narrow, wide = both(lambda: hip_conv(ctx, X, W, Bv, None, 1, pads, strides, "relu", R))
+        assert_bit_exact(wide, narrow, "conv %s tile %d" % ((cin, h, cout, kk), tile))
+        assert_close_max(wide, np.maximum(want + R, 0), GEMM_TOL, "conv %s" % ((cin, h, cout, kk),))

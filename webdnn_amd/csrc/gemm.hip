@@ -116,6 +116,10 @@ __device__ __forceinline__ f32x4 buf_load4(rsrc_t r, int voff, int soff) {
 __device__ __forceinline__ void buf_store(rsrc_t r, float v, int voff, int soff) {
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void buf_store4(rsrc_t r, f32x4 v, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
+}
 
 // Division of a non-negative 32-bit integer by a divisor fixed for the launch: the
 // host turns the divisor into a multiplier and a shift, the kernel pays one
@@ -213,6 +217,7 @@ struct Params {
   int b_bytes;      //       of a group to the end of the tensor, plus the padding shift)
   int y_bytes;      // > 0: bytes of the span of Y over all z, below 2 GiB, and C spans
   int c_bytes;      //      c_bytes (< 2 GiB): whole tiles may use the descriptor epilogue
+  int wide;         // whole tiles may store four columns per lane (see finish_tile)
   ConvGeom cv;
 };
 
@@ -489,6 +494,11 @@ __device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int
 }
 
 // ---- epilogue shared by the contraction kernels ----------------------------------
+// LDS a wavefront turns one 32x32 block through: rows of 36 floats (16-byte aligned, and
+// the two halves of a wavefront land on different banks)
+constexpr int STAGE_LD = 36;
+constexpr int STAGE_FLOATS = 32 * STAGE_LD;
+
 // A lane holds column (li) of each 32x32 block of its wavefront's part of the tile,
 // rows 8*(r/4) + 4*half + r%4 for accumulator register r.  Chunk workgroups store raw
 // sums for splitk_reduce_kernel; whole tiles apply alpha, the C/bias term, the
@@ -497,7 +507,7 @@ template <int BM, int BN, int WM, int WN, bool CONV>
 __device__ __forceinline__ void finish_tile(const Params &p,
                                             f32x16 (&acc)[BM / (WM * 32)][BN / (WN * 32)],
                                             bool whole, int lin, int chunk, int bz, int row0,
-                                            int col0) {
+                                            int col0, float *stage) {
   constexpr int MT = BM / (WM * 32), NT = BN / (WN * 32);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -519,6 +529,87 @@ __device__ __forceinline__ void finish_tile(const Params &p,
           part[lr * BN + wcol + nt * 32 + li] = acc[mt][nt][r];
         }
     return;  // splitk_reduce_kernel adds the chunks up
+  }
+  // Whole tiles whose rows can be written 16 bytes at a time: each 32x32 block is
+  // turned through the wavefront's own corner of the LDS the main loop has finished
+  // with, so that a lane holds four neighbouring columns of a row and the block
+  // leaves in four 16-byte stores (and its residual arrives in four loads) where
+  // the accumulator layout would need sixteen of four bytes.  The epilogue is
+  // bound by the number of memory instructions, not by the bytes.
+  if (p.wide && row0 + BM <= p.m && col0 + BN <= p.n) {
+    __syncthreads();  // no wavefront still reads the main loop's tiles
+    float *st = stage;  // this wavefront's 32 rows of STAGE_LD
+    const long long zoff = CONV ? 0 : (long long)bz * p.sYb;
+    const int y_window = p.y_bytes - (int)(zoff * 4);
+    const rsrc_t rsrc_y = make_rsrc(p.Y + zoff, y_window);
+    const rsrc_t rsrc_r = make_rsrc(p.R ? p.R + zoff : p.Y + zoff, y_window);
+    const rsrc_t rsrc_c = make_rsrc(p.C ? p.C : p.Y, p.C ? p.c_bytes : 0);
+    const int lr = lane >> 3, lc = (lane & 7) * 4;  // row (of every eight) and first column
+    const bool c_per_row = CONV || p.sC1 == 0;
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      const int col = col0 + wcol + nt * 32 + lc;
+      int ybase, ystride, voff_c, cstride;  // in elements; byte offsets stay below 2^31
+      if (CONV) {
+        const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+        const unsigned img = (unsigned)fdiv(col, p.cv.fd_ohw);
+        ybase = (int)((img * (unsigned)p.cv.cout_total + (unsigned)(bz * p.cv.cout_g)) * ohw +
+                      ((unsigned)col - img * ohw));
+        ystride = (int)ohw;
+        voff_c = (bz * p.cv.cout_g + lr) * 4;
+        cstride = 1;
+      } else {
+        ybase = col;
+        ystride = (int)p.sY0;
+        voff_c = (int)((lr * p.sC0 + col * p.sC1) * 4);
+        cstride = (int)p.sC0;
+      }
+      const int voff_y = (ybase + lr * ystride) * 4;
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int rbase = __builtin_amdgcn_readfirstlane(row0 + wrow + mt * 32);
+        f32x4 cv[4], rv[4];
+        if (p.C) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int soff = (rbase + 8 * i) * cstride * 4;
+            if (c_per_row) {
+              const float c = buf_load(rsrc_c, voff_c, soff);
+              cv[i] = f32x4{c, c, c, c};
+            } else {
+              cv[i] = buf_load4(rsrc_c, voff_c, soff);
+            }
+          }
+        }
+        if (p.R) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) rv[i] = buf_load4(rsrc_r, voff_y, (rbase + 8 * i) * ystride * 4);
+        }
+        __builtin_amdgcn_wave_barrier();  // the previous block's reads come first
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          st[(8 * (r >> 2) + 4 * half + (r & 3)) * STAGE_LD + li] = acc[mt][nt][r];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const f32x4 v = *reinterpret_cast<const f32x4 *>(&st[(lr + 8 * i) * STAGE_LD + lc]);
+          f32x4 y;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            float t = p.alpha * v[e];
+            if (p.C) t = __builtin_fmaf(cv[i][e], p.beta, t);
+            if (p.R) t = t + rv[i][e];
+            if (p.epilogue == WDH_EPI_RELU) t = relu_js(t);
+            y[e] = t;
+          }
+          // (row offset in the vector register: a 16-byte store whose scalar offset is a
+          // register gets no wait states from the compiler before its data registers are
+          // written again, and this chip then now and then stores the new value)
+          buf_store4(rsrc_y, y, voff_y + (rbase + 8 * i) * ystride * 4, 0);
+        }
+      }
+    }
+    return;
   }
   // Whole tiles of results below 2 GiB: every address is one per-lane byte
   // offset (column, plus the four rows by which the two halves of a wavefront
@@ -913,7 +1004,9 @@ __global__ __launch_bounds__(NTHREADS, min_blocks(BM, BN)) void contraction_kern
     __syncthreads();
   }
 
-  finish_tile<BM, BN, WM, WN, CONV>(p, acc, whole, lin, chunk, bz, row0, col0);
+  static_assert(2 * A_FLOATS >= 2 * STAGE_FLOATS && 2 * B_FLOATS >= 2 * STAGE_FLOATS, "epilogue staging");
+  finish_tile<BM, BN, WM, WN, CONV>(p, acc, whole, lin, chunk, bz, row0, col0,
+                                    (wave < 2 ? &lds_a[0][0] : &lds_b[0][0]) + (wave & 1) * STAGE_FLOATS);
 }
 
 // ---- 3x3, stride 1, dilation 1: taps read from an input tile staged in LDS -------
@@ -1128,7 +1221,9 @@ __global__ __launch_bounds__(NTHREADS, BM == 64 ? (BN == 64 ? 4 : (BN == 128 ? 3
     __builtin_amdgcn_sched_barrier(0);
     compute();
   }
-  finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0);
+  static_assert(AU * HALO_AROWS * HALO_ROWA >= 4 * STAGE_FLOATS, "epilogue staging");
+  finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0,
+                                    as + (threadIdx.x >> 6) * STAGE_FLOATS);
 }
 
 // ---- small products: K cut across the wavefronts of one workgroup -------------------
@@ -1303,6 +1398,22 @@ int g_last_form = 0;
 bool g_static_scratch = false;  // set for the duration of a wdh_gemm_static call
 int g_wavesplit = 1;      // 0: small products take the ordinary tiles too
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
+int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
+
+// Whether whole tiles may leave in 16-byte stores: Y (and the residual, which has Y's
+// layout) must be 16-byte aligned with rows and z steps that keep the alignment, and the
+// C term must be a value per row or contiguous along the columns.
+static void set_wide(Params &p, bool conv) {
+  auto aligned = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  bool ok = g_wide_stores && p.y_bytes > 0 && aligned(p.Y) && (!p.R || aligned(p.R));
+  if (conv) {
+    ok = ok && (p.cv.oh * p.cv.ow) % 4 == 0;
+  } else {
+    ok = ok && p.sY0 % 4 == 0 && p.sYb % 4 == 0;
+    if (p.C) ok = ok && (p.sC1 == 0 || (p.sC1 == 1 && p.sC0 % 4 == 0 && aligned(p.C)));
+  }
+  p.wide = ok ? 1 : 0;
+}
 
 // How the tiles of one launch are spread over the chip.
 struct WorkPlan {
@@ -1557,6 +1668,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     g_wavesplit = value;
     return WDH_OK;
   }
+  if (strcmp(name, "wide_stores") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: wide_stores %d (use 0 or 1)", value);
+    g_wide_stores = value;
+    return WDH_OK;
+  }
   if (strcmp(name, "conv3x3_halo") == 0) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: conv3x3_halo %d (use 0 or 1)", value);
@@ -1696,6 +1813,7 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
     const bool ok = g_descriptors && y_bytes < 0x7fffffffLL && c_bytes < 0x7fffffffLL;
     p.y_bytes = ok ? (int)y_bytes : 0;
     p.c_bytes = ok ? (int)c_bytes : 0;
+    set_wide(p, false);
   }
   // Few result tiles and a K worth cutting: one launch with K cut across the wavefronts of a
   // workgroup (gemm_wavesplit_kernel) instead of chunks in a workspace and a reduce pass
@@ -1845,6 +1963,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.b_bytes = (int)x_bytes;  // window of group 0; the kernel shortens it per group
     p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
     p.c_bytes = cout * 4;
+    set_wide(p, true);
     return launch<true, B_PIXELS>(p, group, true);
   }
   // 3x3, stride 1, no dilation, input channels in blocks of 8: taps read from an input
@@ -1871,6 +1990,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       p.b_bytes = (int)((long long)n * c * h * w * 4);
       p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
       p.c_bytes = cout * 4;
+      set_wide(p, true);
       switch (tile) {
         case T128x128: return launch_halo_tile<128, 128, 2, 2>(p, group, vecw);
         case T64x256: return launch_halo_tile<64, 256, 1, 4>(p, group, vecw);
@@ -1937,6 +2057,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.b_bytes = small ? (int)x_bytes : 0;  // window of group 0; the kernel shortens it per group
   p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
   p.c_bytes = cout * 4;
+  set_wide(p, true);
   if (mode == B_IM2COL32) return launch<true, B_IM2COL32>(p, group, vec);
   if (mode == B_IM2COL64) return launch<true, B_IM2COL64>(p, group, vec);
   return launch<true, B_IM2COL_BIG>(p, group, vec);
