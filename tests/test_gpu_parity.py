@@ -309,7 +309,7 @@ def test_softmax_edges(ctx):
 
 
 @pytest.mark.parametrize("shape", [(850, 1, 256), (100, 1, 256), (6, 2048), (3, 5000), (4, 7), (2, 3, 1), (9, 1000),
-                                   (5, 250), (7, 1024), (3, 132),
+                                   (5, 250), (7, 1024), (3, 132), (17, 64), (1, 4), (13, 200), (8191, 256), (66, 8),
                                    (27200, 256), (8195, 250), (8193, 1000), (8194, 1028)])       # more rows than resident wavefronts
 def test_layernorm(ctx, shape):
     x, g, b = nrm(*shape, std=2.0), nrm(shape[-1]), nrm(shape[-1])
@@ -389,6 +389,24 @@ def test_maxpool_attributes(ctx, attrs):
         want = ref.maxpool(x, **attrs)
         assert tuple(got.dims) == want.shape
         assert_bit_exact(got.get_data(), want, "maxpool %s on %s" % (attrs, shape))
+
+
+@pytest.mark.parametrize("pads", [[1, 1, 1, 1], [1, 1, 0, 0], [1, 1, 0, 1], [1, 1, 1, 0]])
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8), (1, 2, 7, 12), (3, 1, 33, 64), (1, 1, 400, 544), (2, 2, 5, 4)])
+def test_maxpool_3x3_stride2_pairs(ctx, shape, pads):
+    """The stem's pooling geometry on rows that are a multiple of four wide takes a kernel of its own
+    (two cells per thread); other pads of the same window fall back to the general kernels.  Even and
+    odd heights, NaN and -inf cells, a plane of NaN only."""
+    x = nrm(*shape)
+    x[0, 0, 0, 0] = np.nan
+    x[0, 0, 3, 2] = np.nan
+    x[0, 0, -1, -1] = -np.inf
+    x[-1, -1, :2, :4] = np.nan
+    for ceil_mode in (0, 1):
+        got = H.maxpool(ctx, ctx.move_tensor(x), [3, 3], pads=pads, strides=[2, 2], ceil_mode=ceil_mode)
+        want = ref.maxpool(x, [3, 3], pads=pads, strides=[2, 2], ceil_mode=ceil_mode)
+        assert tuple(got.dims) == want.shape
+        assert_bit_exact(got.get_data(), want, "maxpool 3x3/2 pads %s ceil %d on %s" % (pads, ceil_mode, shape))
 
 
 def test_maxpool_errors(ctx):

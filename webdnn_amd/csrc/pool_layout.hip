@@ -128,6 +128,52 @@ __global__ __launch_bounds__(256) void maxpool2d_band_kernel(PoolParams p, PoolB
   }
 }
 
+// 3x3 window, stride 2, one cell of padding on top and left, rows a multiple of four
+// wide (the pool after a ResNet stem).  A thread owns two neighbouring output cells:
+// their five input columns are one aligned 16-byte piece plus the column before it, so
+// a thread issues three 16-byte and three 4-byte loads (all before the first compare)
+// and one 8-byte store.  Neighbouring output rows share an input row; the vector L1
+// serves the second reader.  No LDS and no barrier.
+__global__ __launch_bounds__(256) void maxpool3x3s2_pairs(PoolParams p, unsigned pairs_per_row,
+                                                           unsigned total_pairs) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const unsigned id = blockIdx.x * 256u + threadIdx.x;
+  if (id >= total_pairs) return;
+  const unsigned rowid = id / pairs_per_row;          // plane * oh + oy
+  const unsigned pair = id - rowid * pairs_per_row;
+  const unsigned plane = rowid / (unsigned)p.oh;
+  const int oy = (int)(rowid - plane * (unsigned)p.oh);
+  const float *x = p.X + (long long)plane * p.h * p.w;
+  const int c0 = 4 * (int)pair;                       // first column of the 16-byte piece
+  f32x4 mid[3];
+  float left[3];
+#pragma unroll
+  for (int ky = 0; ky < 3; ky++) {
+    const int iy = 2 * oy - 1 + ky;
+    const bool rok = (unsigned)iy < (unsigned)p.h;
+    const float *row = x + (long long)(rok ? iy : 0) * p.w;
+    const f32x4 m = *reinterpret_cast<const f32x4 *>(row + c0);
+    const float l = row[c0 > 0 ? c0 - 1 : 0];
+    const float ninf = -INFINITY;
+    mid[ky] = rok ? m : f32x4{ninf, ninf, ninf, ninf};
+    left[ky] = rok && c0 > 0 ? l : ninf;
+  }
+  float a = -INFINITY, b = -INFINITY;   // cells 2*pair and 2*pair + 1
+#pragma unroll
+  for (int ky = 0; ky < 3; ky++) {
+    // strict comparisons, NaN never selected: maxpool.ts:98-101
+    if (left[ky] > a) a = left[ky];
+    if (mid[ky][0] > a) a = mid[ky][0];
+    if (mid[ky][1] > a) a = mid[ky][1];
+    if (mid[ky][1] > b) b = mid[ky][1];
+    if (mid[ky][2] > b) b = mid[ky][2];
+    if (mid[ky][3] > b) b = mid[ky][3];
+  }
+  float *y = p.Y + (long long)rowid * p.ow + 2 * pair;
+  *reinterpret_cast<f32x2 *>(y) = f32x2{a, b};
+}
+
 // ---- transpose -----------------------------------------------------------------
 // Strided copy (Slice, Concat, Split): both sides addressed through strides.
 struct StridedCopyParams {
@@ -340,6 +386,16 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
   p.h = h; p.w = w; p.oh = oh; p.ow = ow; p.kh = kh; p.kw = kw;
   p.pt = pt; p.pl = pl; p.sh = sh; p.sw = sw; p.dh = dh; p.dw = dw;
   hipStream_t st = wdh::stream();
+  // the stem's pool: two cells per thread straight from global memory
+  if (kh == 3 && kw == 3 && sh == 2 && sw == 2 && dh == 1 && dw == 1 && pt == 1 && pl == 1 &&
+      w % 4 == 0 && 2 * ow == w && 2 * (oh - 1) - 1 < h && ((uintptr_t)px & 15) == 0 &&
+      ((uintptr_t)py & 7) == 0 && planes * oh * (ow / 2) < 0xffffffffLL) {
+    const unsigned pairs_per_row = (unsigned)(ow / 2);
+    const unsigned total = (unsigned)(planes * oh * pairs_per_row);
+    hipLaunchKernelGGL(maxpool3x3s2_pairs, dim3((total + 255) / 256), dim3(256), 0, st, p, pairs_per_row, total);
+    WDH_LAUNCH_CHECK();
+    return WDH_OK;
+  }
   // band variant: enough rows for two cells per thread, the span within 32 KB of LDS
   {
     PoolBand b;
