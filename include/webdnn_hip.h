@@ -273,6 +273,20 @@ int wdh_cast(int from_dtype, int to_dtype, wdh_buf X, wdh_buf Y, size_t length);
  * Softmax over the last axis: X viewed as [outer, len]; replaces
  * Softmax.run (operators/cpu/operators/standard/softmax.ts:34-57). */
 int wdh_softmax(wdh_buf X, wdh_buf Y, int64_t outer, int len);
+/* softmax(alpha * Q K^T) V for `batch` heads in one launch: what the chain MatMul -> Mul
+ * by a constant -> Softmax -> MatMul computes (operators/cpu/operators/standard/
+ * matmul.ts:11-111, softmax.ts:34-57; the reference runs the four nodes one after the
+ * other), with the rounding points of that chain.  Element (b, i, x) of Q is at
+ * b*sQb + i*sQi + x, key j of K at b*sKb + j*sKj + x, of V at b*sVb + j*sVj + x and
+ * result (b, i, x) at b*sYb + i*sYi + x: the head dimension d (32, 64 or 128) is the
+ * contiguous one everywhere, which is how the heads lie in a [tokens, heads, d]
+ * projection, so no Transpose of Q, K, V or of the result is needed.  At most 1024
+ * keys (a 32 x keys block of scores is kept in LDS); Q and K 16-byte aligned with
+ * strides that are multiples of 4; Y must not alias an input.  Anything else is
+ * WDH_EINVAL: the caller runs the separate operators instead. */
+int wdh_attention(wdh_buf Q, wdh_buf K, wdh_buf V, wdh_buf Y, int batch, int tq, int tk, int d,
+                  int64_t sQb, int64_t sQi, int64_t sKb, int64_t sKj, int64_t sVb,
+                  int64_t sVj, int64_t sYb, int64_t sYi, float alpha);
 /* LayerNormalization over the last axis (ONNX opset 17, biased variance).
  * The reference has no such operator on any backend; this is what the
  * decomposed ReduceMean/Sub/Pow/Sqrt/Div/Mul/Add subgraph

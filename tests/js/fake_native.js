@@ -174,6 +174,38 @@ const native = {
     }
   },
 
+  // same limits as the library, so that the operator's choice between the one-launch form and
+  // the separate steps is exercised on the CPU tier too
+  attention(Q, K, V, Y, batch, tq, tk, d, sQb, sQi, sKb, sKj, sVb, sVj, sYb, sYi, alpha) {
+    count("attention");
+    if (d !== 32 && d !== 64 && d !== 128) throw new Error(`wdh_attention failed (-2): head dimension ${d}`);
+    if (tk > 1024) throw new Error(`wdh_attention failed (-2): ${tk} keys`);
+    if ([sQb, sQi, sKb, sKj].some((v) => v % 4 !== 0)) throw new Error("wdh_attention failed (-2): strides of Q and K must be multiples of 4 elements");
+    if (batch === 0 || tq === 0) return;
+    if (tk === 0) throw new Error("wdh_attention failed (-2): no keys");
+    need(Y, ((batch - 1) * sYb + (tq - 1) * sYi + d) * 4, "wdh_attention: Y");
+    const q = f32(Q), k = f32(K), v = f32(V), y = f32(Y);
+    const s = new Float32Array(tk), out = new Float32Array(1);
+    for (let b = 0; b < batch; b++) for (let i = 0; i < tq; i++) {
+      let max = -Infinity;
+      for (let j = 0; j < tk; j++) {
+        let dot = 0;
+        for (let x = 0; x < d; x++) dot += q[b * sQb + i * sQi + x] * k[b * sKb + j * sKj + x];
+        out[0] = dot;
+        s[j] = out[0] * alpha;
+        if (s[j] > max) max = s[j];
+      }
+      let sum = 0;
+      for (let j = 0; j < tk; j++) { s[j] = Math.exp(s[j] - max); sum += s[j]; }
+      for (let j = 0; j < tk; j++) s[j] /= sum;
+      for (let x = 0; x < d; x++) {
+        let acc = 0;
+        for (let j = 0; j < tk; j++) acc += s[j] * v[b * sVb + j * sVj + x];
+        y[b * sYb + i * sYi + x] = acc;
+      }
+    }
+  },
+
   layernorm(X, G, B, Y, outer, len, eps) {
     count("layernorm");
     const x = f32(X), y = f32(Y), g = G ? f32(G) : null, b = B ? f32(B) : null, t = new Float32Array(4);
@@ -301,7 +333,7 @@ const native = {
 // Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
 // alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
 // calls that need device data on the host throw and spoil the capture.
-const RECORDED = ["copy", "gemm", "conv2d", "binary", "unary", "softmax", "layernorm", "reduceMean", "reduceAxis", "maxpool2d",
+const RECORDED = ["copy", "gemm", "gemmEx", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "reduceMean", "reduceAxis", "maxpool2d",
   "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
 const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
 const graphs = new Map();

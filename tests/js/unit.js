@@ -275,24 +275,41 @@ test("fusion: attention block -- Transposes, scale and head merge ride on the Ma
       input: [], output: [{ name: "out" }],
     },
   };
-  assert.strictEqual(fuseForHip(model), 3);
+  const unfused = JSON.parse(JSON.stringify(model));
+  assert.strictEqual(fuseForHip(model), 4);
   const ops = model.graph.node.map((n) => n.opType);
-  assert.deepStrictEqual(ops, ["WebDNNHipFusedMatMul", "Softmax", "WebDNNHipFusedMatMul", "Reshape", "WebDNNHipFusedMatMul", "Transpose", "MatMul"]);
+  assert.deepStrictEqual(ops, ["WebDNNHipAttention", "Reshape", "WebDNNHipFusedMatMul", "Transpose", "MatMul"]);
   const attr = (node, name) => node.attribute.find((a) => a.name === name);
-  const [scores, , ctx, , proj] = model.graph.node;
-  assert.deepStrictEqual(scores.input, ["q3", "k3"]);
-  assert.deepStrictEqual(attr(scores, "perm_a").ints, [1, 0, 2]);
-  assert.deepStrictEqual(attr(scores, "perm_b").ints, [1, 2, 0]);
-  assert.strictEqual(attr(scores, "alpha").f, 0.125);
-  assert.deepStrictEqual(scores.output, ["scaled"]);
-  assert.deepStrictEqual(ctx.input, ["attn", "v3"]);
-  assert.deepStrictEqual(attr(ctx, "perm_b").ints, [1, 0, 2]);
-  assert.deepStrictEqual(attr(ctx, "perm_y").ints, [1, 0, 2]);
-  assert.deepStrictEqual(ctx.output, ["ctx_t"]);
+  const [att, , proj] = model.graph.node;
+  assert.deepStrictEqual(att.input, ["q3", "k3", "v3"]);
+  assert.deepStrictEqual(attr(att, "perm_q").ints, [1, 0, 2]);
+  assert.deepStrictEqual(attr(att, "perm_k").ints, [1, 2, 0]);
+  assert.deepStrictEqual(attr(att, "perm_v").ints, [1, 0, 2]);
+  assert.deepStrictEqual(attr(att, "perm_y").ints, [1, 0, 2]);
+  assert.strictEqual(attr(att, "alpha").f, 0.125);
+  assert.strictEqual(attr(att, "softmax_axis").i, -1);
+  assert.deepStrictEqual(att.output, ["ctx_t"]);
   assert.deepStrictEqual(proj.input, ["merged", "w", "b", "src"]);
   assert.strictEqual(attr(proj, "has_bias").i, 1);
   assert.strictEqual(attr(proj, "has_residual").i, 1);
   assert.deepStrictEqual(proj.output, ["res"]);
+  // probabilities that something else reads too (or that leave the graph) keep the three nodes
+  const watched = JSON.parse(JSON.stringify(unfused));
+  watched.graph.output.push({ name: "attn" });
+  assert.strictEqual(fuseForHip(watched), 3);
+  assert.deepStrictEqual(watched.graph.node.slice(0, 3).map((n) => n.opType), ["WebDNNHipFusedMatMul", "Softmax", "WebDNNHipFusedMatMul"]);
+  const [scores, , ctx] = watched.graph.node;
+  assert.deepStrictEqual(scores.input, ["q3", "k3"]);
+  assert.deepStrictEqual(attr(scores, "perm_a").ints, [1, 0, 2]);
+  assert.deepStrictEqual(attr(scores, "perm_b").ints, [1, 2, 0]);
+  assert.strictEqual(attr(scores, "alpha").f, 0.125);
+  assert.deepStrictEqual(ctx.input, ["attn", "v3"]);
+  assert.deepStrictEqual(attr(ctx, "perm_y").ints, [1, 0, 2]);
+  // a Softmax over another axis is no attention
+  const other = JSON.parse(JSON.stringify(unfused));
+  other.graph.node[5].attribute = [{ name: "axis", type: 2, i: 1, floats: [], ints: [], strings: [] }];
+  assert.strictEqual(fuseForHip(other), 3);
+  assert.ok(other.graph.node.some((n) => n.opType === "Softmax"));
 });
 
 test("HipTensor: alias shares one reference-counted buffer; data round trip; use after dispose throws", async () => {

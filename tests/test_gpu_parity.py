@@ -1138,3 +1138,66 @@ def test_sixteen_byte_stores_hold_the_bits_of_four_byte_stores(ctx, tile):
         narrow, wide = both(lambda: hip_conv(ctx, X, W, Bv, None, 1, pads, strides, "relu", R))
         assert_bit_exact(wide, narrow, "conv %s tile %d" % ((cin, h, cout, kk), tile))
         assert_close_max(wide, np.maximum(want + R, 0), GEMM_TOL, "conv %s" % ((cin, h, cout, kk),))
+
+
+def attention_chain_ref(q, k, v, heads, alpha):
+    """The oracle's MatMul -> Mul -> Softmax -> MatMul per head."""
+    tq, width = q.shape
+    d = width // heads
+    out = np.empty((tq, width), np.float32)
+    for h in range(heads):
+        sl = slice(h * d, (h + 1) * d)
+        s = ref.matmul(np.ascontiguousarray(q[:, sl]), np.ascontiguousarray(k[:, sl].T))
+        s = ref.binary("Mul", s, np.float32(alpha).reshape(()))
+        out[:, sl] = ref.matmul(ref.softmax(s), np.ascontiguousarray(v[:, sl]))
+    return out
+
+
+@pytest.mark.parametrize("tq,tk,heads,d", [(850, 850, 8, 32), (100, 850, 8, 32), (100, 100, 8, 32), (1, 1, 1, 32),
+                                           (33, 1024, 2, 64), (70, 257, 3, 128), (32, 31, 4, 32), (5, 1000, 1, 64)])
+def test_attention_one_launch_equals_the_four_node_chain(ctx, tq, tk, heads, d):
+    """wdh_attention against the oracle's chain, and against the library's own unfused chain
+    (MatMul with strided heads, scale as alpha, Softmax, MatMul) within 1e-5."""
+    rng = np.random.default_rng(tq * 7 + tk)
+    q = rng.standard_normal((tq, heads * d)).astype(np.float32)
+    k = rng.standard_normal((tk, heads * d)).astype(np.float32)
+    v = rng.standard_normal((tk, heads * d)).astype(np.float32)
+    alpha = 1.0 / np.sqrt(d)
+    tq_, tk_, tv_ = ctx.move_tensor(q), ctx.move_tensor(k), ctx.move_tensor(v)
+    got = H.attention(ctx, tq_, tk_, tv_, heads, alpha).get_data()
+    want = attention_chain_ref(q, k, v, heads, alpha)
+    assert_close_max(got, want, GEMM_TOL, "attention vs oracle chain")
+    # the unfused chain on the device, heads addressed through strides
+    w = heads * d
+    scores = ctx.empty_tensor([heads, tq, tk])
+    capi.call("wdh_gemm_ex", tq_.handle, tk_.handle, 0, scores.handle, heads, tq, tk, d,
+              d, w, 1, d, 1, w, 0, 0, float(alpha), 1.0, 0, 0, tq * tk, tk)
+    probs = H.softmax(ctx, scores)
+    chain = ctx.empty_tensor([tq, w])
+    capi.call("wdh_gemm_ex", probs.handle, tv_.handle, 0, chain.handle, heads, tq, d, tk,
+              tq * tk, tk, 1, d, w, 1, 0, 0, 1.0, 1.0, 0, 0, d, w)
+    assert_close_max(got, chain.get_data(), 1e-5, "attention vs unfused chain")
+
+
+def test_attention_special_values_and_limits(ctx):
+    """A +inf in V beside masked keys, a NaN score, and the shapes the entry point turns down."""
+    rng = np.random.default_rng(5)
+    q = rng.standard_normal((40, 32)).astype(np.float32)
+    k = rng.standard_normal((50, 32)).astype(np.float32)
+    v = rng.standard_normal((50, 32)).astype(np.float32)
+    v[49, 3] = np.inf
+    q[7, 0] = np.nan
+    got = H.attention(ctx, ctx.move_tensor(q), ctx.move_tensor(k), ctx.move_tensor(v), 1, 0.25).get_data()
+    want = attention_chain_ref(q, k, v, 1, 0.25)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    fin = np.isfinite(want)
+    assert_close_max(got[fin], want[fin], GEMM_TOL, "finite cells")
+    t = lambda *s: ctx.move_tensor(rng.standard_normal(s).astype(np.float32))
+    with pytest.raises(capi.HipError):
+        H.attention(ctx, t(4, 48), t(4, 48), t(4, 48), 1, 1.0)            # head dimension 48
+    with pytest.raises(capi.HipError):
+        H.attention(ctx, t(4, 32), t(1025, 32), t(1025, 32), 1, 1.0)      # more keys than LDS holds
+    with pytest.raises(H.OperatorError):
+        H.attention(ctx, t(4, 64), t(6, 64), t(5, 64), 2, 1.0)            # k and v disagree
+    assert H.attention(ctx, t(0, 64), t(6, 64), t(6, 64), 2, 1.0).dims == [0, 64]

@@ -192,6 +192,43 @@ def test_unit_level_js(tmp_path):
     assert summary["failed"] == 0 and summary["passed"] >= 14, summary
 
 
+@pytest.mark.parametrize("hd,one_launch", [(32, True), (8, False)])
+def test_attention_chain_becomes_one_node(tmp_path, hd, one_launch):
+    """MatMul -> Mul -> Softmax -> MatMul with the head Transposes around it becomes one
+    WebDNNHipAttention node.  Head dimensions the kernel is built for take one native call; others
+    run the steps one by one inside the node.  Either way the output is the unfused graph's."""
+    g = modelgen.GraphBuilder(1)
+    tq, tk, h = 7, 9, 2
+    d = h * hd
+    g.const("sq", np.array([tq, h, hd], np.int64))
+    g.const("sk", np.array([tk, h, hd], np.int64))
+    g.const("so", np.array([tq, d], np.int64))
+    g.const("scale", np.array(1.0 / np.sqrt(hd), np.float32))
+    g.op("Transpose", [g.op("Reshape", ["Q", "sq"], "q3")], "qh", perm=[1, 0, 2])
+    g.op("Transpose", [g.op("Reshape", ["K", "sk"], "k3")], "kt", perm=[1, 2, 0])
+    g.op("Transpose", [g.op("Reshape", ["V", "sk"], "v3")], "vh", perm=[1, 0, 2])
+    g.op("Softmax", [g.op("Mul", [g.op("MatMul", ["qh", "kt"], "scores"), "scale"], "scaled")], "attn", axis=-1)
+    g.op("Reshape", [g.op("Transpose", [g.op("MatMul", ["attn", "vh"], "ctx")], "ctx_t", perm=[1, 0, 2]), "so"], "Y")
+    data = g.finish([("Q", [tq, d]), ("K", [tk, d]), ("V", [tk, d])], [("Y", [tq, d])], opset=13)
+    (tmp_path / "model.onnx").write_bytes(data)
+    rng = np.random.default_rng(3)
+    feeds = {n: rng.standard_normal(s).astype(np.float32) for n, s in (("Q", (tq, d)), ("K", (tk, d)), ("V", (tk, d)))}
+    ins = [feeds["Q"], feeds["K"], feeds["V"]]
+    outs, rep = node_runner.run_model(str(tmp_path), ins, "hip", strict=True, fake_native=True)
+    assert rep["nodes"] == 5                       # 4 Reshapes + the attention node
+    calls = rep["nativeCalls"]
+    if one_launch:
+        assert calls.get("attention") == 1 and "gemm" not in calls and "softmax" not in calls
+    else:
+        assert calls.get("attention") is None and calls["gemm"] == 2 and calls["softmax"] == 1
+    assert rep["liveBuffers"] == rep["initializerCopies"]
+    want = graph_ref.run_graph(modelgen.parse_model(data), feeds)["Y"]
+    np.testing.assert_allclose(outs[0], want, rtol=0, atol=1e-6)
+    plain, rep_p = node_runner.run_model(str(tmp_path), ins, "hip", strict=True, fuse=False, fake_native=True)
+    assert rep_p["nodes"] == 12
+    np.testing.assert_allclose(outs[0], plain[0], rtol=0, atol=1e-6)
+
+
 def test_detr_style_graph_on_the_hip_host_path(tmp_path):
     """The config-5 graph at toy size: every operator and shape trick it uses (head split by
     Reshape+Transpose, K^T by Transpose, scalar Mul, Softmax, LayerNormalization, fused MatMul+bias,

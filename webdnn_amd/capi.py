@@ -58,6 +58,8 @@ SIGNATURES = {
     "wdh_binary": (_c.c_int, [_c.c_int, _c.c_int, c_buf, c_buf, c_buf, _c.c_int, _i32p, _i64p, _i64p]),
     "wdh_unary": (_c.c_int, [_c.c_int, _c.c_int, c_buf, c_buf, _c.c_size_t]),
     "wdh_softmax": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
+    "wdh_attention": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int, _c.c_int, _c.c_int, _c.c_int] +
+                      [_c.c_int64] * 8 + [_c.c_float]),
     "wdh_layernorm": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_float]),
     "wdh_reduce_mean": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
     "wdh_reduce_axis": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64]),

@@ -18,21 +18,14 @@
 #include <math.h>
 
 #include "common.h"
+#include "rowmath.h"
 
 namespace {
 
+using namespace wdh::rowmath;
+
 constexpr int WAVES_PER_BLOCK = 4;
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
 __device__ __forceinline__ double wave_sum_d(double v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -87,17 +80,6 @@ __device__ __forceinline__ void store_row(float *y, int len, int lane, const flo
 }
 
 // ---- softmax ---------------------------------------------------------------
-// e^x through the hardware's 2^r: x*log2(e) is split into the nearest integer n and a
-// remainder r (|r| <= 1/2) that keeps the bits the single-precision product would drop,
-// so the result is within two ulp for every x, large negative ones included.
-__device__ __forceinline__ float exp_f32(float x) {
-  x = x < -150.0f ? -150.0f : x;  // e^-150 is already 0 in single precision; NaN stays NaN
-  const float log2e_hi = 1.44269502162933349609375f, log2e_lo = 1.925963033500011e-8f;
-  const float n = __builtin_rintf(x * log2e_hi);
-  float r = __builtin_fmaf(x, log2e_hi, -n);
-  r = __builtin_fmaf(x, log2e_lo, r);
-  return __builtin_ldexpf(__builtin_amdgcn_exp2f(r), (int)n);
-}
 template <int NV, bool VEC>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_reg(
     const float *__restrict__ X, float *__restrict__ Y, long long outer, int len) {
@@ -420,7 +402,7 @@ extern "C" int wdh_layernorm(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY,
   hipStream_t st = wdh::stream();
   const bool vec = len % 4 == 0 &&
                    (((uintptr_t)px | (uintptr_t)py | (uintptr_t)pg | (uintptr_t)pb) & 15) == 0;
-  if (len <= 256 && vec) {
+  if (len <= 256 && vec && outer >= 4096) {  // (fewer rows: a wavefront per row, for four times the wavefronts)
     // (eight lanes per row measured slower: 12.4 us against 10.0 us on 27200 rows of 256)
     const long long per_block = WAVES_PER_BLOCK * 4;
     const dim3 g((unsigned)((outer + per_block - 1) / per_block));

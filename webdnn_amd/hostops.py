@@ -389,6 +389,23 @@ def softmax(ctx, x, axis=-1):
     return y
 
 
+def attention(ctx, q, k, v, heads, alpha):
+    """softmax(alpha * Q_h K_h^T) V_h for every head h, heads side by side as in a
+    [tokens, heads * d] projection: q [tq, heads*d], k and v [tk, heads*d] -> [tq, heads*d].
+    The chain the reference runs node by node (cpu matmul.ts:11-111, softmax.ts:34-57)."""
+    _require_f32(q, k, v)
+    if q.ndim != 2 or k.ndim != 2 or v.ndim != 2:
+        raise OperatorError("attention: q, k, v must be [tokens, heads*d]")
+    width = q.dims[1]
+    if heads <= 0 or width % heads or k.dims[1] != width or v.dims[1] != width or k.dims[0] != v.dims[0]:
+        raise OperatorError("attention: shapes %s %s %s do not hold %d heads" % (q.dims, k.dims, v.dims, heads))
+    d = width // heads
+    y = ctx.empty_tensor(q.dims)
+    call("wdh_attention", q.handle, k.handle, v.handle, y.handle, heads, q.dims[0], k.dims[0], d,
+         d, width, d, width, d, width, d, width, float(alpha))
+    return y
+
+
 def layer_normalization(ctx, x, scale=None, bias=None, axis=-1, epsilon=1e-5):
     """ONNX LayerNormalization (opset 17) over the last axis."""
     _require_f32(x, scale, bias)

@@ -214,7 +214,80 @@ function fuseForHip(model) {
     graph.node = nodes.filter((n, idx) => !removed.has(idx));
     logger.info(`hip fusion: ${fusedCount} chains fused, ${removed.size} nodes removed`);
   }
-  return fusedCount;
+  return fusedCount + fuseAttention(graph);
+}
+
+// (Fused)MatMul -> Softmax -> (Fused)MatMul  ->  WebDNNHipAttention
+// where the first product carries nothing but operand permutations and a scale, the Softmax
+// normalises the last axis of its rank-3 result, and the second product takes the
+// probabilities as they are (no permutation of its first operand), adds nothing and may
+// write the merged-heads layout.  Both intermediate tensors must have no other reader.
+// Runs after the MatMul chains have been fused, so the Transposes and the scale are
+// already attributes of the two products.
+function fuseAttention(graph) {
+  const nodes = graph.node;
+  const readers = new Map();
+  const bump = (name) => readers.set(name, (readers.get(name) || 0) + 1);
+  for (const node of nodes) for (const name of node.input) bump(name);
+  for (const out of graph.output) bump(out.name);
+  const producerOf = new Map();
+  nodes.forEach((node, idx) => node.output.forEach((name) => producerOf.set(name, idx)));
+  const attr = (node, name) => node.attribute.find((a) => a.name === name);
+  const intOf = (node, name, dflt) => {
+    const a = attr(node, name);
+    return a && a.i !== undefined && a.i !== null ? Number(a.i) : dflt;
+  };
+  const intsOf = (node, name) => {
+    const a = attr(node, name);
+    return a && a.ints ? a.ints.map(Number) : [];
+  };
+  const stringOf = (node, name) => {
+    const a = attr(node, name);
+    return a && a.s ? Buffer.from(a.s).toString("utf-8") : "";
+  };
+  const isProduct = (node) => node.opType === "MatMul" || node.opType === "WebDNNHipFusedMatMul";
+  const plain = (node) => node.input.length === 2 && intOf(node, "has_bias", 0) === 0 &&
+    intOf(node, "has_residual", 0) === 0 && stringOf(node, "activation") === "";
+
+  const removed = new Set();
+  let count = 0;
+  nodes.forEach((soft, si) => {
+    if (soft.opType !== "Softmax" || soft.input.length !== 1 || soft.output.length !== 1) return;
+    const axis = intOf(soft, "axis", -1);
+    if (axis !== -1 && axis !== 2) return;
+    const pi = producerOf.get(soft.input[0]);
+    if (pi === undefined || removed.has(pi) || readers.get(soft.input[0]) !== 1) return;
+    const scores = nodes[pi];
+    if (!isProduct(scores) || !plain(scores) || intsOf(scores, "perm_y").length) return;
+    if (readers.get(soft.output[0]) !== 1) return;
+    const ci = nodes.findIndex((n, idx) => idx > si && !removed.has(idx) && n.input.includes(soft.output[0]));
+    if (ci < 0) return;
+    const ctx = nodes[ci];
+    if (!isProduct(ctx) || !plain(ctx) || ctx.input[0] !== soft.output[0] || ctx.input[1] === soft.output[0]) return;
+    if (intsOf(ctx, "perm_a").length || attr(ctx, "alpha")) return;
+    const alphaAttr = attr(scores, "alpha");
+    const extra = [intAttr("softmax_axis", axis)];
+    if (alphaAttr) extra.push(floatAttr("alpha", alphaAttr.f));
+    const perms = { perm_q: intsOf(scores, "perm_a"), perm_k: intsOf(scores, "perm_b"), perm_v: intsOf(ctx, "perm_b"),
+      perm_y: intsOf(ctx, "perm_y") };
+    for (const name of Object.keys(perms)) if (perms[name].length) extra.push(intsAttr(name, perms[name]));
+    nodes[ci] = {
+      input: [scores.input[0], scores.input[1], ctx.input[1]],
+      output: ctx.output.slice(),
+      name: ctx.name,
+      opType: "WebDNNHipAttention",
+      attribute: extra,
+      domain: "webdnn.hip",
+    };
+    removed.add(pi);
+    removed.add(si);
+    count++;
+  });
+  if (count > 0) {
+    graph.node = nodes.filter((n, idx) => !removed.has(idx));
+    logger.info(`hip fusion: ${count} attention chains fused`);
+  }
+  return count;
 }
 
 // For every node name, the tensors that can be disposed right after it has run.
@@ -237,4 +310,4 @@ function findTensorReleaseTiming(model, initializerTensorNames) {
   return timing;
 }
 
-module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip };
+module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention };

@@ -141,4 +141,4 @@ function getOpEntries() {
     { opType: "WebDNNHipFusedMatMul", backend: "hip", opsetMin: 1, factory: () => new HipMatMul(true) },
   ];
 }
-module.exports = { getOpEntries };
+module.exports = { getOpEntries, HipMatMul, operandView };
