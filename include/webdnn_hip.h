@@ -294,6 +294,13 @@ int wdh_attention(wdh_buf Q, wdh_buf K, wdh_buf V, wdh_buf Y, int batch, int tq,
  * computes.  Gamma/Beta are [len] or 0 (1 / 0 respectively). */
 int wdh_layernorm(wdh_buf X, wdh_buf Gamma, wdh_buf Beta, wdh_buf Y,
                   int64_t outer, int len, float eps);
+/* LayerNormalization followed by the Add that reads its result: Y as wdh_layernorm, and
+ * Y2 = Y + P with P of X's shape (both results are kept: the graph reads the normalised rows
+ * again later).  Replaces the node pair LayerNormalization -> Add (binary7.ts:24-75 for the
+ * Add; the reference has no LayerNormalization); Y2 holds exactly what the separate Add
+ * would store.  Y2 must not alias X, Y or P. */
+int wdh_layernorm_add(wdh_buf X, wdh_buf Gamma, wdh_buf Beta, wdh_buf Y, wdh_buf P, wdh_buf Y2,
+                      int64_t outer, int len, float eps);
 /* ReduceMean over the trailing `len` elements of each of `outer` rows;
  * replaces ReduceMean (reduce.ts:369-405) for trailing-axes reductions. */
 int wdh_reduce_mean(wdh_buf X, wdh_buf Y, int64_t outer, int len);

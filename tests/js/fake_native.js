@@ -34,6 +34,24 @@ function toInt32(d) {
   return d | 0; // ToInt32, like a store into an Int32Array
 }
 
+function layernormRows(X, G, B, Y, outer, len, eps) {
+  const x = f32(X), y = f32(Y), g = G ? f32(G) : null, b = B ? f32(B) : null, t = new Float32Array(4);
+  for (let o = 0; o < outer; o++) {
+    let s = 0;
+    for (let r = 0; r < len; r++) s += x[o * len + r];
+    t[0] = s / len; // mean
+    let q = 0;
+    for (let r = 0; r < len; r++) { t[1] = x[o * len + r] - t[0]; t[2] = t[1] * t[1]; q += t[2]; }
+    t[2] = q / len; t[2] = t[2] + Math.fround(eps); t[3] = Math.sqrt(t[2]);
+    for (let r = 0; r < len; r++) {
+      t[1] = x[o * len + r] - t[0]; t[1] = t[1] / t[3];
+      if (g) t[1] = t[1] * g[r];
+      if (b) t[1] = t[1] + b[r];
+      y[o * len + r] = t[1];
+    }
+  }
+}
+
 const native = {
   init(device) {
     count("init");
@@ -208,21 +226,15 @@ const native = {
 
   layernorm(X, G, B, Y, outer, len, eps) {
     count("layernorm");
-    const x = f32(X), y = f32(Y), g = G ? f32(G) : null, b = B ? f32(B) : null, t = new Float32Array(4);
-    for (let o = 0; o < outer; o++) {
-      let s = 0;
-      for (let r = 0; r < len; r++) s += x[o * len + r];
-      t[0] = s / len; // mean
-      let q = 0;
-      for (let r = 0; r < len; r++) { t[1] = x[o * len + r] - t[0]; t[2] = t[1] * t[1]; q += t[2]; }
-      t[2] = q / len; t[2] = t[2] + Math.fround(eps); t[3] = Math.sqrt(t[2]);
-      for (let r = 0; r < len; r++) {
-        t[1] = x[o * len + r] - t[0]; t[1] = t[1] / t[3];
-        if (g) t[1] = t[1] * g[r];
-        if (b) t[1] = t[1] + b[r];
-        y[o * len + r] = t[1];
-      }
-    }
+    layernormRows(X, G, B, Y, outer, len, eps);
+  },
+
+  layernormAdd(X, G, B, Y, P, Y2, outer, len, eps) {
+    count("layernormAdd");
+    layernormRows(X, G, B, Y, outer, len, eps);
+    need(Y2, outer * len * 4, "wdh_layernorm_add: Y2");
+    const y = f32(Y), p = f32(P), y2 = f32(Y2);
+    for (let i = 0; i < outer * len; i++) y2[i] = y[i] + p[i];
   },
 
   reduceAxis(X, Y, outer, red, inner, divisor) {
@@ -333,7 +345,7 @@ const native = {
 // Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
 // alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
 // calls that need device data on the host throw and spoil the capture.
-const RECORDED = ["copy", "gemm", "gemmEx", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "reduceMean", "reduceAxis", "maxpool2d",
+const RECORDED = ["copy", "gemm", "gemmEx", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "layernormAdd", "reduceMean", "reduceAxis", "maxpool2d",
   "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
 const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
 const graphs = new Map();

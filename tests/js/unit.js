@@ -312,6 +312,36 @@ test("fusion: attention block -- Transposes, scale and head merge ride on the Ma
   assert.ok(other.graph.node.some((n) => n.opType === "Softmax"));
 });
 
+test("fusion: LayerNormalization followed by an Add of an already known tensor becomes one two-output node", () => {
+  const { fuseLayerNormAdd } = require("../../webdnn_amd/js/core/modelTransform");
+  const nd = (opType, input, output) => ({ opType, input, output, name: output[0], attribute: [] });
+  const init = (name) => ({ name, dims: [4], dataType: 1, floatData: [0, 0, 0, 0] });
+  const graph = {
+    node: [
+      nd("LayerNormalization", ["x", "g", "b"], ["n1"]),
+      nd("Relu", ["n1"], ["r"]),
+      nd("Add", ["n1", "pos"], ["n1p"]),          // pos: initializer -> fused
+      nd("Add", ["n1", "pos"], ["again"]),        // a second Add of the same result stays
+      nd("LayerNormalization", ["n1p", "g", "b"], ["n2"]),
+      nd("Add", ["late", "n2"], ["n2l"]),         // `late` is produced after n2 -> stays
+      nd("Relu", ["r"], ["late"]),
+      nd("LayerNormalization", ["again", "g", "b"], ["n3"]),
+      nd("Add", ["r", "n3"], ["out"]),            // r: an earlier node's output -> fused
+    ],
+    initializer: [init("g"), init("b"), init("pos")], input: [{ name: "x" }], output: [{ name: "out" }, { name: "n2l" }],
+  };
+  assert.strictEqual(fuseLayerNormAdd(graph), 2);
+  assert.deepStrictEqual(graph.node.map((n) => [n.opType, n.input.join(), n.output.join()]), [
+    ["WebDNNHipLayerNormAdd", "x,g,b,pos", "n1,n1p"],
+    ["Relu", "n1", "r"],
+    ["Add", "n1,pos", "again"],
+    ["LayerNormalization", "n1p,g,b", "n2"],
+    ["Add", "late,n2", "n2l"],
+    ["Relu", "r", "late"],
+    ["WebDNNHipLayerNormAdd", "again,g,b,r", "n3,out"],
+  ]);
+});
+
 test("HipTensor: alias shares one reference-counted buffer; data round trip; use after dispose throws", async () => {
   const cpu = new WebDNNCPUContextImpl();
   const ctx = new WebDNNHipContextImpl(cpu, { native: fakeNative, contractionTile: 3, splitK: 2 });

@@ -1201,3 +1201,18 @@ def test_attention_special_values_and_limits(ctx):
     with pytest.raises(H.OperatorError):
         H.attention(ctx, t(4, 64), t(6, 64), t(5, 64), 2, 1.0)            # k and v disagree
     assert H.attention(ctx, t(0, 64), t(6, 64), t(6, 64), 2, 1.0).dims == [0, 64]
+
+
+@pytest.mark.parametrize("shape", [(850, 256), (100, 1, 256), (27200, 256), (9, 1000), (5, 250), (3, 5000), (4100, 64)])
+def test_layernorm_add_holds_what_the_two_nodes_store(ctx, shape):
+    """wdh_layernorm_add: first result = wdh_layernorm's bits, second = the Add kernel's bits on it."""
+    x, p = nrm(*shape), nrm(*shape)
+    g, b = nrm(shape[-1]), nrm(shape[-1])
+    tx, tg, tb, tp = (ctx.move_tensor(t) for t in (x, g, b, p))
+    y, y2 = H.layer_normalization_add(ctx, tx, tg, tb, tp)
+    alone = H.layer_normalization(ctx, tx, tg, tb)
+    assert_bit_exact(y.get_data(), alone.get_data(), "normalised rows %s" % (shape,))
+    assert_bit_exact(y2.get_data(), H.binary(ctx, "Add", alone, tp).get_data(), "rows + addend %s" % (shape,))
+    assert_close_max(y.get_data(), ref.layernorm_decomposed(x, g, b, 1e-5), 1e-5, "against the oracle")
+    with pytest.raises(H.OperatorError):
+        H.layer_normalization_add(ctx, tx, tg, tb, ctx.move_tensor(nrm(shape[-1])))

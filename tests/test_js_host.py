@@ -229,6 +229,38 @@ def test_attention_chain_becomes_one_node(tmp_path, hd, one_launch):
     np.testing.assert_allclose(outs[0], plain[0], rtol=0, atol=1e-6)
 
 
+def test_layernorm_with_the_add_that_follows(tmp_path):
+    """LayerNormalization -> Add(constant) becomes one two-output node: same-shape addends ride in the
+    launch (layernormAdd), broadcasting ones are added by the Add kernel inside the node.  The
+    normalised tensor keeps its other readers.  Bit-identical to the unfused graph."""
+    g = modelgen.GraphBuilder(2)
+    t, d = 6, 16
+    rng = g.rng()
+    g.const("gamma", rng.standard_normal(d).astype(np.float32))
+    g.const("beta", rng.standard_normal(d).astype(np.float32))
+    g.const("pos", rng.standard_normal((t, d)).astype(np.float32))
+    g.const("row", rng.standard_normal((d,)).astype(np.float32))
+    g.op("LayerNormalization", ["X", "gamma", "beta"], "n1", axis=-1, epsilon=1e-5)
+    g.op("Add", ["n1", "pos"], "n1p")
+    g.op("Mul", ["n1", "n1p"], "m")
+    g.op("LayerNormalization", ["m", "gamma", "beta"], "n2", axis=-1, epsilon=1e-5)
+    g.op("Add", ["row", "n2"], "n2r")
+    g.op("Sub", ["n2r", "n2"], "Y")
+    data = g.finish([("X", [t, d])], [("Y", [t, d])], opset=17)
+    (tmp_path / "model.onnx").write_bytes(data)
+    feeds = {"X": np.random.default_rng(9).standard_normal((t, d)).astype(np.float32)}
+    outs, rep = node_runner.run_model(str(tmp_path), [feeds["X"]], "hip", strict=True, fake_native=True)
+    assert rep["nodes"] == 4
+    calls = rep["nativeCalls"]
+    assert calls["layernormAdd"] == 1 and calls["layernorm"] == 1 and calls["binary"] == 3
+    assert rep["liveBuffers"] == rep["initializerCopies"]
+    plain, rep_p = node_runner.run_model(str(tmp_path), [feeds["X"]], "hip", strict=True, fuse=False, fake_native=True)
+    assert rep_p["nodes"] == 6
+    assert_bit_exact(outs[0], plain[0], "LayerNormalization+Add fused")
+    want = graph_ref.run_graph(modelgen.parse_model(data), feeds)["Y"]
+    np.testing.assert_allclose(outs[0], want, rtol=0, atol=5e-6)
+
+
 def test_detr_style_graph_on_the_hip_host_path(tmp_path):
     """The config-5 graph at toy size: every operator and shape trick it uses (head split by
     Reshape+Transpose, K^T by Transpose, scalar Mul, Softmax, LayerNormalization, fused MatMul+bias,

@@ -61,6 +61,7 @@ SIGNATURES = {
     "wdh_attention": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int, _c.c_int, _c.c_int, _c.c_int] +
                       [_c.c_int64] * 8 + [_c.c_float]),
     "wdh_layernorm": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_float]),
+    "wdh_layernorm_add": (_c.c_int, [c_buf, c_buf, c_buf, c_buf, c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_float]),
     "wdh_reduce_mean": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),
     "wdh_reduce_axis": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64]),
     "wdh_maxpool2d": (_c.c_int, [c_buf, c_buf] + [_c.c_int] * 14),

@@ -132,7 +132,7 @@ template <int NV, bool VEC>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
     const float *__restrict__ X, const float *__restrict__ G,
     const float *__restrict__ Bt, float *__restrict__ Y, long long outer, int len,
-    float eps) {
+    float eps, const float *__restrict__ P, float *__restrict__ Y2) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
@@ -162,6 +162,13 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
     v[i] = t;
   }
   store_row<NV, VEC>(Y + row * len, len, lane, v);
+  if (P) {  // second output: the normalised row plus a row of P (the Add that follows in the graph)
+    float pv[NV];
+    load_row<NV, VEC>(P + row * len, len, lane, 0.0f, pv);
+#pragma unroll
+    for (int i = 0; i < NV; i++) v[i] = v[i] + pv[i];
+    store_row<NV, VEC>(Y2 + row * len, len, lane, v);
+  }
 }
 
 // Short rows (len <= 256, 16-byte aligned): a wavefront owns 64/SUB rows, SUB lanes each.
@@ -178,7 +185,7 @@ template <int SUB>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
     const float *__restrict__ X, const float *__restrict__ G,
     const float *__restrict__ Bt, float *__restrict__ Y, long long outer, int len,
-    float eps) {
+    float eps, const float *__restrict__ P, float *__restrict__ Y2) {
   constexpr int NJ = 256 / (4 * SUB);  // 16-byte pieces per lane
   constexpr int SEG = 4 * SUB;
   const int lane = threadIdx.x & 63, sub = lane & (SUB - 1);
@@ -232,13 +239,19 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
       for (int e = 0; e < 4; e++) t[e] = t[e] + bt[e];
     }
     *reinterpret_cast<f32x4 *>(y + idx) = t;
+    if (P) {
+      const f32x4 pv = *reinterpret_cast<const f32x4 *>(P + row * len + idx);
+#pragma unroll
+      for (int e = 0; e < 4; e++) t[e] = t[e] + pv[e];
+      *reinterpret_cast<f32x4 *>(Y2 + row * len + idx) = t;
+    }
   }
 }
 
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_stream(
     const float *__restrict__ X, const float *__restrict__ G,
     const float *__restrict__ Bt, float *__restrict__ Y, long long outer, int len,
-    float eps) {
+    float eps, const float *__restrict__ P, float *__restrict__ Y2) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
@@ -259,6 +272,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_stream(
     if (G) t = t * G[idx];
     if (Bt) t = t + Bt[idx];
     y[idx] = t;
+    if (P) Y2[row * len + idx] = t + P[row * len + idx];
   }
 }
 
@@ -385,40 +399,60 @@ extern "C" int wdh_softmax(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   return WDH_OK;
 }
 
-extern "C" int wdh_layernorm(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY,
-                             int64_t outer, int len, float eps) {
-  WDH_REQUIRE_INIT();
-  if (int rc = check_rows("wdh_layernorm", outer, len)) return rc;
+namespace {
+int layernorm_launch(const char *who, wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY, wdh_buf hP, wdh_buf hY2,
+                     int64_t outer, int len, float eps) {
+  if (int rc = check_rows(who, outer, len)) return rc;
   if (outer == 0 || len == 0) return WDH_OK;
-  void *px, *py, *pg = nullptr, *pb = nullptr;
+  void *px, *py, *pg = nullptr, *pb = nullptr, *pp = nullptr, *py2 = nullptr;
   const size_t bytes = (size_t)outer * len * 4;
-  if (!wdh::operand(hX, bytes, "wdh_layernorm: X", &px)) return WDH_EINVAL;
-  if (!wdh::operand(hY, bytes, "wdh_layernorm: Y", &py)) return WDH_EINVAL;
-  if (hG && !wdh::operand(hG, (size_t)len * 4, "wdh_layernorm: Gamma", &pg)) return WDH_EINVAL;
-  if (hB && !wdh::operand(hB, (size_t)len * 4, "wdh_layernorm: Beta", &pb)) return WDH_EINVAL;
-  const float *X = (const float *)px, *G = (const float *)pg, *B = (const float *)pb;
-  float *Y = (float *)py;
+  if (!wdh::operand(hX, bytes, "layernorm: X", &px)) return WDH_EINVAL;
+  if (!wdh::operand(hY, bytes, "layernorm: Y", &py)) return WDH_EINVAL;
+  if (hG && !wdh::operand(hG, (size_t)len * 4, "layernorm: Gamma", &pg)) return WDH_EINVAL;
+  if (hB && !wdh::operand(hB, (size_t)len * 4, "layernorm: Beta", &pb)) return WDH_EINVAL;
+  if (hP) {
+    if (!wdh::operand(hP, bytes, "layernorm: P", &pp)) return WDH_EINVAL;
+    if (!wdh::operand(hY2, bytes, "layernorm: Y2", &py2)) return WDH_EINVAL;
+    if (py2 == py || py2 == px || py2 == pp) return fail(WDH_EINVAL, "%s: Y2 aliases another operand", who);
+  }
+  const float *X = (const float *)px, *G = (const float *)pg, *B = (const float *)pb, *P = (const float *)pp;
+  float *Y = (float *)py, *Y2 = (float *)py2;
   dim3 grid(row_blocks(outer)), block(64 * WAVES_PER_BLOCK);
   hipStream_t st = wdh::stream();
   const bool vec = len % 4 == 0 &&
-                   (((uintptr_t)px | (uintptr_t)py | (uintptr_t)pg | (uintptr_t)pb) & 15) == 0;
+                   (((uintptr_t)px | (uintptr_t)py | (uintptr_t)pg | (uintptr_t)pb | (uintptr_t)pp |
+                     (uintptr_t)py2) & 15) == 0;
   if (len <= 256 && vec && outer >= 4096) {  // (fewer rows: a wavefront per row, for four times the wavefronts)
     // (eight lanes per row measured slower: 12.4 us against 10.0 us on 27200 rows of 256)
     const long long per_block = WAVES_PER_BLOCK * 4;
     const dim3 g((unsigned)((outer + per_block - 1) / per_block));
-    hipLaunchKernelGGL(layernorm_rows_part<16>, g, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL(layernorm_rows_part<16>, g, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   } else if (len <= 64 * 4 && vec)
-    hipLaunchKernelGGL((layernorm_rows_reg<4, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL((layernorm_rows_reg<4, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   else if (len <= 64 * 4)
-    hipLaunchKernelGGL((layernorm_rows_reg<4, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL((layernorm_rows_reg<4, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   else if (len <= 64 * 16 && vec)
-    hipLaunchKernelGGL((layernorm_rows_reg<16, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL((layernorm_rows_reg<16, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   else if (len <= 64 * 16)
-    hipLaunchKernelGGL((layernorm_rows_reg<16, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL((layernorm_rows_reg<16, false>), grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   else
-    hipLaunchKernelGGL(layernorm_rows_stream, grid, block, 0, st, X, G, B, Y, outer, len, eps);
+    hipLaunchKernelGGL(layernorm_rows_stream, grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
+}
+}  // namespace
+
+extern "C" int wdh_layernorm(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY,
+                             int64_t outer, int len, float eps) {
+  WDH_REQUIRE_INIT();
+  return layernorm_launch("wdh_layernorm", hX, hG, hB, hY, 0, 0, outer, len, eps);
+}
+
+extern "C" int wdh_layernorm_add(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY, wdh_buf hP, wdh_buf hY2,
+                                 int64_t outer, int len, float eps) {
+  WDH_REQUIRE_INIT();
+  if (!hP || !hY2) return fail(WDH_EINVAL, "wdh_layernorm_add: P and Y2 are required");
+  return layernorm_launch("wdh_layernorm_add", hX, hG, hB, hY, hP, hY2, outer, len, eps);
 }
 
 extern "C" int wdh_reduce_mean(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {

@@ -424,6 +424,27 @@ def layer_normalization(ctx, x, scale=None, bias=None, axis=-1, epsilon=1e-5):
     return y
 
 
+def layer_normalization_add(ctx, x, scale, bias, addend, axis=-1, epsilon=1e-5):
+    """LayerNormalization and the Add that follows it: returns (normalised, normalised + addend),
+    addend of x's shape.  One launch for the node pair."""
+    _require_f32(x, scale, bias, addend)
+    if axis < 0:
+        axis += x.ndim
+    if axis != x.ndim - 1:
+        raise OperatorError("LayerNormalization: only the last axis is supported")
+    if list(addend.dims) != list(x.dims):
+        raise OperatorError("LayerNormalization+Add: the addend must have the input's shape")
+    length = x.dims[-1]
+    for t in (scale, bias):
+        if t is not None and t.length != length:
+            raise OperatorError("LayerNormalization: scale/bias must have the normalised length")
+    y, y2 = ctx.empty_tensor(x.dims), ctx.empty_tensor(x.dims)
+    call("wdh_layernorm_add", x.handle, scale.handle if scale is not None else 0,
+         bias.handle if bias is not None else 0, y.handle, addend.handle, y2.handle,
+         x.length // length if length else 0, length, epsilon)
+    return y, y2
+
+
 def reduce_mean_last(ctx, x, keepdims=1):
     """ReduceMean over the last axis: cpu reduce.ts:369-405."""
     _require_f32(x)

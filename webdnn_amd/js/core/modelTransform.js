@@ -214,7 +214,48 @@ function fuseForHip(model) {
     graph.node = nodes.filter((n, idx) => !removed.has(idx));
     logger.info(`hip fusion: ${fusedCount} chains fused, ${removed.size} nodes removed`);
   }
-  return fusedCount + fuseAttention(graph);
+  return fusedCount + fuseAttention(graph) + fuseLayerNormAdd(graph);
+}
+
+// LayerNormalization -> Add(other)  ->  WebDNNHipLayerNormAdd with two outputs
+// (the normalised tensor, which the graph usually reads again, and the sum).  `other` must exist
+// before the LayerNormalization runs: an initializer, a graph input or an earlier node's output.
+// Of several Adds reading the result the first qualifies.  Float32 Adds only compute fl(y + p),
+// which is what the kernel stores, so nothing about the numbers changes.
+function fuseLayerNormAdd(graph) {
+  const nodes = graph.node;
+  const known = new Set(graph.initializer.map((t) => t.name));
+  for (const input of graph.input) known.add(input.name);
+  const removed = new Set();
+  let count = 0;
+  nodes.forEach((ln, li) => {
+    if (ln.opType === "LayerNormalization" && ln.output.length === 1 && ln.input.length === 3 &&
+      ln.input.every((n) => n !== "")) {
+      const y = ln.output[0];
+      const ai = nodes.findIndex((n, idx) => idx > li && !removed.has(idx) && n.opType === "Add" && n.input.length === 2 &&
+        n.input.includes(y) && n.input[0] !== n.input[1] && known.has(n.input[0] === y ? n.input[1] : n.input[0]));
+      if (ai >= 0) {
+        const add = nodes[ai];
+        const other = add.input[0] === y ? add.input[1] : add.input[0];
+        nodes[li] = {
+          input: ln.input.concat([other]),
+          output: [y, add.output[0]],
+          name: ln.name,
+          opType: "WebDNNHipLayerNormAdd",
+          attribute: ln.attribute,
+          domain: "webdnn.hip",
+        };
+        removed.add(ai);
+        count++;
+      }
+    }
+    for (const name of nodes[li].output) known.add(name);
+  });
+  if (count > 0) {
+    graph.node = nodes.filter((n, idx) => !removed.has(idx));
+    logger.info(`hip fusion: ${count} LayerNormalization + Add pairs fused`);
+  }
+  return count;
 }
 
 // (Fused)MatMul -> Softmax -> (Fused)MatMul  ->  WebDNNHipAttention
@@ -310,4 +351,4 @@ function findTensorReleaseTiming(model, initializerTensorNames) {
   return timing;
 }
 
-module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention };
+module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention, fuseLayerNormAdd };

@@ -322,6 +322,14 @@ FN(js_softmax) {
   return make_undefined(env);
 }
 
+FN(js_layernorm_add) {
+  ARGS("wdh_layernorm_add", 9);
+  I64(0, X); I64(1, G); I64(2, B); I64(3, Y); I64(4, P); I64(5, Y2); I64(6, outer); I64(7, len);
+  F64(8, eps);
+  CHECK(wdh_layernorm_add(X, G, B, Y, P, Y2, outer, (int)len, (float)eps));
+  return make_undefined(env);
+}
+
 FN(js_attention) { /* (Q, K, V, Y, batch, tq, tk, d, sQb, sQi, sKb, sKj, sVb, sVj, sYb, sYi, alpha) */
   ARGS("wdh_attention", 17);
   I64(0, Q); I64(1, K); I64(2, V); I64(3, Y); I64(4, batch); I64(5, tq); I64(6, tk); I64(7, d);
@@ -452,7 +460,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"read", js_read}, {"copy", js_copy}, {"sync", js_sync}, {"memStats", js_mem_stats},
       {"trim", js_trim}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
       {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
-      {"softmax", js_softmax}, {"attention", js_attention}, {"layernorm", js_layernorm}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
+      {"softmax", js_softmax}, {"attention", js_attention}, {"layernorm", js_layernorm}, {"layernormAdd", js_layernorm_add}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
       {"stridedCopy", js_strided_copy}, {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end},
