@@ -205,6 +205,19 @@ int wdh_gemm_ex(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
                 int64_t sB0, int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
                 float beta, int epilogue, wdh_buf R, int64_t sYb, int64_t sY0);
 
+/* `count` (at most 16) independent linear layers Y_i[m_i, n_i] = A_i[m_i, k_i] W_i[k_i, n_i]
+ * (+ bias_i[n_i]) (then Relu if `epilogue` is WDH_EPI_RELU), all operands dense and
+ * row-major: each is exactly the wdh_gemm call of a MatMul node followed by its bias Add
+ * (operators/cpu/operators/standard/matmul.ts:11-111, binary7.ts:24-75).  Products small
+ * enough for the one-launch form of wdh_gemm (few 32x32 result blocks, K cut across the
+ * wavefronts of a workgroup) leave together in one launch, which is what this entry point
+ * is for: the query, key and value projections of an attention block are three such
+ * products; the others are launched one by one as wdh_gemm would.  Results are the bits
+ * wdh_gemm stores.  `bias` may be NULL, or hold 0 for a layer without bias; every Y_i
+ * must be a buffer of its own that no problem of the group reads. */
+int wdh_linear_group(int count, const wdh_buf *A, const wdh_buf *W, const wdh_buf *bias,
+                     const wdh_buf *Y, const int *m, const int *n, const int *k, int epilogue);
+
 /* wdh_gemm for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments, same kernels and bit-identical

@@ -125,6 +125,17 @@ const native = {
     }
   },
 
+  linearGroup(A, W, Bias, Y, m, n, k, epi) {
+    count("linearGroup");
+    for (let i = 0; i < A.length; i++) {
+      for (let j = 0; j < A.length; j++) {
+        if ((j !== i && Y[i] === Y[j]) || Y[i] === A[j] || Y[i] === W[j]) throw new Error("wdh_linear_group failed (-2): result is also an operand");
+      }
+      native.gemmEx(A[i], W[i], Bias[i], Y[i], 1, m[i], n[i], k[i], 0, k[i], 1, 0, n[i], 1, 0, 1, 1.0, 1.0, epi, 0, m[i] * n[i], n[i]);
+      if (--calls.gemm === 0) delete calls.gemm; // counted as one linearGroup call
+    }
+  },
+
   conv2d(X, W, Bias, Y, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epi, R) {
     count("conv2d");
     if (c % group || cout % group) throw new Error("wdh_conv2d failed (-2): channels not divisible by group");
@@ -345,7 +356,7 @@ const native = {
 // Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
 // alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
 // calls that need device data on the host throw and spoil the capture.
-const RECORDED = ["copy", "gemm", "gemmEx", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "layernormAdd", "reduceMean", "reduceAxis", "maxpool2d",
+const RECORDED = ["copy", "gemm", "gemmEx", "linearGroup", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "layernormAdd", "reduceMean", "reduceAxis", "maxpool2d",
   "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
 const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
 const graphs = new Map();

@@ -342,6 +342,41 @@ test("fusion: LayerNormalization followed by an Add of an already known tensor b
   ]);
 });
 
+test("fusion: neighbouring linear layers that do not read each other become one group node", () => {
+  const { groupLinears } = require("../../webdnn_amd/js/core/modelTransform");
+  const nd = (opType, input, output, attribute) => ({ opType, input, output, name: output[0], attribute: attribute || [] });
+  const fusedAttrs = (bias, act, extra) => [
+    { name: "has_bias", i: bias, type: 2, floats: [], ints: [], strings: [] },
+    { name: "has_residual", i: 0, type: 2, floats: [], ints: [], strings: [] },
+    { name: "activation", s: Buffer.from(act), type: 3, floats: [], ints: [], strings: [] },
+  ].concat(extra || []);
+  const graph = {
+    node: [
+      nd("WebDNNHipFusedMatMul", ["x", "wq", "bq"], ["q"], fusedAttrs(1, "")),
+      nd("WebDNNHipFusedMatMul", ["x", "wk", "bk"], ["k"], fusedAttrs(1, "")),
+      nd("MatMul", ["y", "wv"], ["v"]),
+      nd("MatMul", ["q", "wo"], ["o"]),                                               // reads q: starts a new run
+      nd("WebDNNHipFusedMatMul", ["y", "w1", "b1"], ["h"], fusedAttrs(1, "Relu")),    // another activation: alone
+      nd("Relu", ["o"], ["r"]),
+      nd("MatMul", ["r", "w2"], ["a"]),
+      nd("WebDNNHipFusedMatMul", ["r", "w3"], ["b"], fusedAttrs(0, "", [{ name: "alpha", f: 0.5, type: 1, floats: [], ints: [], strings: [] }])),
+      nd("MatMul", ["r", "w4"], ["c"]),
+    ],
+    initializer: [], input: [], output: [],
+  };
+  assert.strictEqual(groupLinears(graph), 1);
+  assert.deepStrictEqual(graph.node.map((n) => [n.opType, n.input.join(), n.output.join()]), [
+    ["WebDNNHipLinearGroup", "x,wq,bq,x,wk,bk,y,wv", "q,k,v"],
+    ["MatMul", "q,wo", "o"],
+    ["WebDNNHipFusedMatMul", "y,w1,b1", "h"],
+    ["Relu", "o", "r"],
+    ["MatMul", "r,w2", "a"],
+    ["WebDNNHipFusedMatMul", "r,w3", "b"],
+    ["MatMul", "r,w4", "c"],
+  ]);
+  assert.deepStrictEqual(graph.node[0].attribute.find((a) => a.name === "arity").ints, [3, 3, 2]);
+});
+
 test("HipTensor: alias shares one reference-counted buffer; data round trip; use after dispose throws", async () => {
   const cpu = new WebDNNCPUContextImpl();
   const ctx = new WebDNNHipContextImpl(cpu, { native: fakeNative, contractionTile: 3, splitK: 2 });

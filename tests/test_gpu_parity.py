@@ -1216,3 +1216,34 @@ def test_layernorm_add_holds_what_the_two_nodes_store(ctx, shape):
     assert_close_max(y.get_data(), ref.layernorm_decomposed(x, g, b, 1e-5), 1e-5, "against the oracle")
     with pytest.raises(H.OperatorError):
         H.layer_normalization_add(ctx, tx, tg, tb, ctx.move_tensor(nrm(shape[-1])))
+
+
+def test_linear_group_holds_the_bits_of_separate_gemms(ctx):
+    """wdh_linear_group: the projections of an attention block (and a mix of shapes, one of them too
+    large for the one-launch form, one without bias, one with a ragged K) against wdh_gemm one by one."""
+    rng = np.random.default_rng(11)
+    t = lambda *s: ctx.move_tensor(rng.standard_normal(s).astype(np.float32))
+    groups = [
+        [(850, 256, 256, True)] * 3,
+        [(100, 256, 256, True), (850, 256, 256, True), (850, 256, 256, True)],
+        [(100, 256, 256, True), (850, 2048, 256, True), (37, 130, 200, False), (64, 64, 1000, True),
+         (5, 7, 3, True), (100, 92, 256, True), (100, 256, 256, False), (33, 257, 129, True)],
+    ]
+    for shapes in groups:
+        for epi in (None, "relu"):
+            problems = [(t(m, k), t(k, n), t(n) if bias else None) for m, n, k, bias in shapes]
+            got = H.linear_group(ctx, problems, epi)
+            for (a, w, b), y in zip(problems, got):
+                want = H.gemm(ctx, a, w, b, epilogue=epi).get_data()
+                assert_bit_exact(y.get_data(), want, "group member %s" % (a.dims,))
+                assert_close_max(want, ref.unary("Relu", ref.gemm(a.get_data(), w.get_data(), None if b is None else b.get_data()))
+                                 if epi else ref.gemm(a.get_data(), w.get_data(), None if b is None else b.get_data()),
+                                 GEMM_TOL, "against the oracle")
+    assert H.linear_group(ctx, []) == []
+    a, w = t(4, 8), t(8, 4)
+    y = ctx.empty_tensor([4, 4])
+    arr = lambda *v: (ctypes.c_int64 * len(v))(*v)
+    i32 = lambda *v: (ctypes.c_int32 * len(v))(*v)
+    with pytest.raises(capi.HipError):   # one buffer as two results
+        capi.call("wdh_linear_group", 2, arr(a.handle, a.handle), arr(w.handle, w.handle), arr(0, 0),
+                  arr(y.handle, y.handle), i32(4, 4), i32(4, 4), i32(8, 8), 0)

@@ -229,6 +229,40 @@ def test_attention_chain_becomes_one_node(tmp_path, hd, one_launch):
     np.testing.assert_allclose(outs[0], plain[0], rtol=0, atol=1e-6)
 
 
+def test_neighbouring_linear_layers_run_as_one_group(tmp_path):
+    """Projections of one input and rank-3 MatMuls next to rank-2 ones:
+    grouped into one node; the rank-2 ones take one native call, a group with the rank-3 product in it
+    runs product by product.  Bit-identical to the ungrouped graph."""
+    g = modelgen.GraphBuilder(5)
+    t, d = 5, 12
+    rng = g.rng()
+    for name, shape in (("Wq", (d, d)), ("Wk", (d, 8)), ("Wv", (d, d)), ("bq", (d,)), ("bk", (8,)), ("W3", (d, 4))):
+        g.const(name, (rng.standard_normal(shape) * 0.3).astype(np.float32))
+    g.const("s3", np.array([1, t, d], np.int64))
+    g.op("Add", [g.op("MatMul", ["X", "Wq"], "q_mm"), "bq"], "q")
+    g.op("Add", [g.op("MatMul", ["X", "Wk"], "k_mm"), "bk"], "k")
+    g.op("MatMul", ["X", "Wv"], "v")
+    g.op("Reshape", ["X", "s3"], "x3")
+    g.op("MatMul", ["x3", "W3"], "p3")          # rank 3, alone in its run (the Reshape separates it)
+    g.op("MatMul", ["q", "Wq"], "qq")
+    g.op("MatMul", ["x3", "Wv"], "pv")          # rank 3 next to a rank-2 product: grouped, run one by one
+    g.op("MatMul", [g.op("Add", ["qq", "v"], "qv"), "Wk"], "Y")
+    data = g.finish([("X", [t, d])], [("Y", [t, 8]), ("k", [t, 8]), ("p3", [1, t, 4]), ("pv", [1, t, d])], opset=13)
+    (tmp_path / "model.onnx").write_bytes(data)
+    feeds = {"X": np.random.default_rng(6).standard_normal((t, d)).astype(np.float32)}
+    outs, rep = node_runner.run_model(str(tmp_path), [feeds["X"]], "hip", strict=True, fake_native=True)
+    calls = rep["nativeCalls"]
+    # (q, k) as a group; (p3, qq, pv) grouped but rank 3 among them: one by one; X Wv + qq as a fused node; Y
+    assert calls["linearGroup"] == 1 and calls["gemm"] == 5 and rep["nodes"] == 5
+    plain, rep_p = node_runner.run_model(str(tmp_path), [feeds["X"]], "hip", strict=True, fuse=False, fake_native=True)
+    assert rep_p["nodes"] > rep["nodes"]
+    for a, b in zip(outs, plain):
+        assert_bit_exact(a, b, "grouped linear layers")
+    want = graph_ref.run_graph(modelgen.parse_model(data), feeds)
+    for got, name in zip(outs, ("Y", "k", "p3", "pv")):
+        np.testing.assert_allclose(got, want[name], rtol=0, atol=2e-5)
+
+
 def test_layernorm_with_the_add_that_follows(tmp_path):
     """LayerNormalization -> Add(constant) becomes one two-output node: same-shape addends ride in the
     launch (layernormAdd), broadcasting ones are added by the Add kernel inside the node.  The

@@ -1238,14 +1238,14 @@ __global__ __launch_bounds__(NTHREADS, BM == 64 ? (BN == 64 ? 4 : (BN == 128 ? 3
 // depend on scheduling -- before the usual epilogue.  One launch, no workspace.
 constexpr int WS_WAVES = 16;
 template <bool B_IS_KC, bool VEC>
-__global__ __launch_bounds__(64 * WS_WAVES, 1) void gemm_wavesplit_kernel(Params p) {
+__device__ __forceinline__ void wavesplit_block(const Params &p, int block) {
   __shared__ float part[WS_WAVES][16][64];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 31, half = lane >> 5;
   const int tiles_per_z = p.tiles_m * p.tiles_n;
-  const int bz = fdiv((int)blockIdx.x, p.fd_tiles_per_z);
-  const int tile = (int)blockIdx.x - bz * tiles_per_z;
+  const int bz = fdiv(block, p.fd_tiles_per_z);
+  const int tile = block - bz * tiles_per_z;
   const int tm = fdiv(tile, p.fd_group), tn = tile - tm * p.tiles_n;  // fd_group: division by tiles_n
   const int row0 = tm * 32, col0 = tn * 32;
 
@@ -1336,6 +1336,28 @@ __global__ __launch_bounds__(64 * WS_WAVES, 1) void gemm_wavesplit_kernel(Params
   p.Y[off] = y;
 }
 
+template <bool B_IS_KC, bool VEC>
+__global__ __launch_bounds__(64 * WS_WAVES, 1) void gemm_wavesplit_kernel(Params p) {
+  wavesplit_block<B_IS_KC, VEC>(p, (int)blockIdx.x);
+}
+
+// Several independent small products in one launch (the query, key and value projections
+// of an attention block): the blocks of problem i follow those of problem i - 1 in the grid.
+constexpr int GROUP_MAX = 6;
+struct GroupParams {
+  int count;
+  int first[GROUP_MAX + 1];  // first block of each problem; first[count] = grid size
+  Params p[GROUP_MAX];
+};
+template <bool B_IS_KC, bool VEC>
+__global__ __launch_bounds__(64 * WS_WAVES, 1) void gemm_wavesplit_group_kernel(GroupParams g) {
+  int i = 0;
+#pragma unroll
+  for (int j = 1; j < GROUP_MAX; j++)
+    if (j < g.count && (int)blockIdx.x >= g.first[j]) i = j;
+  wavesplit_block<B_IS_KC, VEC>(g.p[i], (int)blockIdx.x - g.first[i]);
+}
+
 // Reference-order scalar kernel for operands that are dense in neither index
 // (never produced by the runner's dense tensors, kept so the entry point is total).
 __global__ void contraction_strided_kernel(Params p) {
@@ -1398,6 +1420,15 @@ int g_last_form = 0;
 bool g_static_scratch = false;  // set for the duration of a wdh_gemm_static call
 int g_wavesplit = 1;      // 0: small products take the ordinary tiles too
 int g_halo = 1;           // 0: 3x3 stride-1 convs use the gathered form too
+// wdh_linear_group: while set, products that qualify for gemm_wavesplit_kernel are queued here
+// instead of being launched, and leave together in one launch per kernel variant
+struct GroupQueue {
+  bool collecting = false;
+  int count = 0;
+  Params p[16];
+  long long blocks[16];
+  int variant[16];  // 2 * B_IS_KC + VEC
+} g_group;
 int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
 
 // Whether whole tiles may leave in 16-byte stores: Y (and the residual, which has Y's
@@ -1831,6 +1862,13 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
       p.fd_group = make_fastdiv(p.tiles_n);
       p.kchunk = ((k + BK - 1) / BK + WS_WAVES - 1) / WS_WAVES * BK;  // slabs per wavefront, in elements
       g_last_plan = {32, 32, WS_WAVES, useB_kc ? WDH_FORM_GEMM_KC : WDH_FORM_GEMM_MC, blocks32, 0};
+      if (g_group.collecting && g_group.count < 16) {
+        g_group.p[g_group.count] = p;
+        g_group.blocks[g_group.count] = blocks32;
+        g_group.variant[g_group.count] = 2 * (useB_kc ? 1 : 0) + (vec ? 1 : 0);
+        g_group.count++;
+        return WDH_OK;
+      }
       const dim3 grid((unsigned)blocks32), block(64 * WS_WAVES);
       if (useB_kc && vec)
         hipLaunchKernelGGL((gemm_wavesplit_kernel<true, true>), grid, block, 0, wdh::stream(), p);
@@ -1848,6 +1886,66 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   if (useA_kc && !useB_kc) return launch<true, B_MC>(p, batch, vec);
   if (!useA_kc && useB_kc) return launch<false, B_KC>(p, batch, vec);
   return launch<false, B_MC>(p, batch, vec);
+}
+
+namespace {
+// Launches what wdh_linear_group queued: one launch per kernel variant and GROUP_MAX problems.
+int flush_group() {
+  for (int variant = 0; variant < 4; variant++) {
+    GroupParams g;
+    g.count = 0;
+    long long blocks = 0;
+    auto launch_now = [&]() -> int {
+      if (g.count == 0) return WDH_OK;
+      g.first[g.count] = (int)blocks;
+      const dim3 grid((unsigned)blocks), block(64 * WS_WAVES);
+      switch (variant) {
+        case 3: hipLaunchKernelGGL((gemm_wavesplit_group_kernel<true, true>), grid, block, 0, wdh::stream(), g); break;
+        case 2: hipLaunchKernelGGL((gemm_wavesplit_group_kernel<true, false>), grid, block, 0, wdh::stream(), g); break;
+        case 1: hipLaunchKernelGGL((gemm_wavesplit_group_kernel<false, true>), grid, block, 0, wdh::stream(), g); break;
+        default: hipLaunchKernelGGL((gemm_wavesplit_group_kernel<false, false>), grid, block, 0, wdh::stream(), g); break;
+      }
+      WDH_LAUNCH_CHECK();
+      g.count = 0;
+      blocks = 0;
+      return WDH_OK;
+    };
+    for (int i = 0; i < g_group.count; i++) {
+      if (g_group.variant[i] != variant) continue;
+      if (g.count == GROUP_MAX || blocks + g_group.blocks[i] > 0x3fffffffLL)
+        if (int rc = launch_now()) return rc;
+      g.first[g.count] = (int)blocks;
+      g.p[g.count] = g_group.p[i];
+      blocks += g_group.blocks[i];
+      g.count++;
+    }
+    if (int rc = launch_now()) return rc;
+  }
+  return WDH_OK;
+}
+}  // namespace
+
+extern "C" int wdh_linear_group(int count, const wdh_buf *hA, const wdh_buf *hW, const wdh_buf *hBias,
+                                const wdh_buf *hY, const int *m, const int *n, const int *k, int epilogue) {
+  WDH_REQUIRE_INIT();
+  if (count < 0 || count > 16) return fail(WDH_EINVAL, "wdh_linear_group: %d problems (0..16)", count);
+  if (count > 0 && (!hA || !hW || !hY || !m || !n || !k)) return fail(WDH_EINVAL, "wdh_linear_group: NULL array");
+  // the results must be distinct buffers, none of them an input: the products run in no particular order
+  for (int i = 0; i < count; i++)
+    for (int j = 0; j < count; j++)
+      if ((j != i && hY[i] == hY[j]) || hY[i] == hA[j] || hY[i] == hW[j] || (hBias && hBias[j] && hY[i] == hBias[j]))
+        return fail(WDH_EINVAL, "wdh_linear_group: result %d is also an operand or another result", i);
+  g_group.collecting = true;
+  g_group.count = 0;
+  int rc = WDH_OK;
+  for (int i = 0; i < count && rc == WDH_OK; i++)
+    rc = wdh_gemm_ex(hA[i], hW[i], hBias ? hBias[i] : 0, hY[i], 1, m[i], n[i], k[i], 0, k[i], 1, 0, n[i], 1, 0, 1,
+                     1.0f, 1.0f, epilogue, 0, (int64_t)m[i] * n[i], n[i]);
+  g_group.collecting = false;
+  // (what was queued before a failure still runs: every queued problem passed its checks)
+  const int rc2 = flush_group();
+  g_group.count = 0;
+  return rc != WDH_OK ? rc : rc2;
 }
 
 // ---- conv ----------------------------------------------------------------

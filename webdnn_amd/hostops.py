@@ -389,6 +389,28 @@ def softmax(ctx, x, axis=-1):
     return y
 
 
+def linear_group(ctx, problems, epilogue=None):
+    """Independent linear layers in as few launches as possible: problems = [(a [m,k], w [k,n], bias [n] or None)],
+    returns the list of results.  Each is what gemm(a, w, bias) returns."""
+    count = len(problems)
+    ys, hs = [], {"a": [], "w": [], "b": [], "y": []}
+    ms, ns, ks = [], [], []
+    for a, w, b in problems:
+        _require_f32(a, w, b)
+        if a.ndim != 2 or w.ndim != 2 or a.dims[1] != w.dims[0] or (b is not None and list(b.dims) != [w.dims[1]]):
+            raise OperatorError("linear_group: shapes %s %s %s" % (a.dims, w.dims, None if b is None else b.dims))
+        y = ctx.empty_tensor([a.dims[0], w.dims[1]])
+        ys.append(y)
+        hs["a"].append(a.handle); hs["w"].append(w.handle); hs["b"].append(b.handle if b is not None else 0)
+        hs["y"].append(y.handle)
+        ms.append(a.dims[0]); ns.append(w.dims[1]); ks.append(a.dims[1])
+    arr64 = lambda v: (ctypes.c_int64 * count)(*v)
+    arr32 = lambda v: (ctypes.c_int32 * count)(*v)
+    call("wdh_linear_group", count, arr64(hs["a"]), arr64(hs["w"]), arr64(hs["b"]), arr64(hs["y"]),
+         arr32(ms), arr32(ns), arr32(ks), EPI[epilogue])
+    return ys
+
+
 def attention(ctx, q, k, v, heads, alpha):
     """softmax(alpha * Q_h K_h^T) V_h for every head h, heads side by side as in a
     [tokens, heads * d] projection: q [tq, heads*d], k and v [tk, heads*d] -> [tq, heads*d].

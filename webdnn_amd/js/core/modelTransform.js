@@ -214,7 +214,71 @@ function fuseForHip(model) {
     graph.node = nodes.filter((n, idx) => !removed.has(idx));
     logger.info(`hip fusion: ${fusedCount} chains fused, ${removed.size} nodes removed`);
   }
-  return fusedCount + fuseAttention(graph) + fuseLayerNormAdd(graph);
+  return fusedCount + fuseAttention(graph) + fuseLayerNormAdd(graph) + groupLinears(graph);
+}
+
+// Neighbouring linear layers that do not read each other  ->  one WebDNNHipLinearGroup node.
+// A linear layer here is a MatMul, or a fused MatMul that carries at most a bias and an
+// activation (no operand permutation, scale or residual).  Only nodes that follow each
+// other directly are grouped, so the order of everything else stays what it was; the group
+// takes the place of its last member.
+function groupLinears(graph) {
+  const nodes = graph.node;
+  const attr = (node, name) => node.attribute.find((a) => a.name === name);
+  const flag = (node, name) => {
+    const a = attr(node, name);
+    return a && a.i !== undefined && a.i !== null ? Number(a.i) : 0;
+  };
+  const activationOf = (node) => {
+    const a = attr(node, "activation");
+    return a && a.s ? Buffer.from(a.s).toString("utf-8") : "";
+  };
+  const isLinear = (node) => {
+    if (node.output.length !== 1) return false;
+    if (node.opType === "MatMul") return node.input.length === 2 && node.input.every((n) => n !== "");
+    if (node.opType !== "WebDNNHipFusedMatMul") return false;
+    if (flag(node, "has_residual") || attr(node, "alpha")) return false;
+    if (["perm_a", "perm_b", "perm_y"].some((name) => attr(node, name))) return false;
+    return node.input.length === 2 + flag(node, "has_bias");
+  };
+  const result = [];
+  let groups = 0;
+  let i = 0;
+  while (i < nodes.length) {
+    if (!isLinear(nodes[i])) {
+      result.push(nodes[i++]);
+      continue;
+    }
+    const run = [nodes[i]];
+    const produced = new Set(nodes[i].output);
+    const activation = activationOf(nodes[i]);
+    let j = i + 1;
+    while (j < nodes.length && run.length < 16 && isLinear(nodes[j]) && activationOf(nodes[j]) === activation &&
+      !nodes[j].input.some((name) => produced.has(name))) {
+      run.push(nodes[j]);
+      produced.add(nodes[j].output[0]);
+      j++;
+    }
+    if (run.length === 1) {
+      result.push(nodes[i++]);
+      continue;
+    }
+    result.push({
+      input: [].concat(...run.map((n) => n.input)),
+      output: run.map((n) => n.output[0]),
+      name: run[run.length - 1].name,
+      opType: "WebDNNHipLinearGroup",
+      attribute: [intsAttr("arity", run.map((n) => n.input.length)), stringAttr("activation", activation)],
+      domain: "webdnn.hip",
+    });
+    groups++;
+    i = j;
+  }
+  if (groups > 0) {
+    graph.node = result;
+    logger.info(`hip fusion: ${groups} groups of neighbouring linear layers`);
+  }
+  return groups;
 }
 
 // LayerNormalization -> Add(other)  ->  WebDNNHipLayerNormAdd with two outputs
@@ -351,4 +415,4 @@ function findTensorReleaseTiming(model, initializerTensorNames) {
   return timing;
 }
 
-module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention, fuseLayerNormAdd };
+module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention, fuseLayerNormAdd, groupLinears };

@@ -129,6 +129,60 @@ class HipMatMul extends MatMul {
   }
 }
 
+// Several independent linear layers (A [m, k] times a [k, n] weight, plus a bias row, then
+// Relu or nothing) as one node: what the hip fusion pass makes of neighbouring MatMul(+Add)
+// chains that do not read each other, such as the query, key and value projections of an
+// attention block.  Rank-2 operands go to the native grouped call, which puts the small
+// products into one launch; anything else runs product by product as the separate nodes would.
+class HipLinearGroup extends MatMul {
+  constructor() {
+    super("hip");
+  }
+
+  initialize(attribute) {
+    super.initialize(attribute);
+    this.arity = getAttrInts(attribute, "arity", []);
+    this.activation = getAttrString(attribute, "activation", "");
+    if (this.activation !== "" && this.activation !== "Relu") {
+      throw new Error(`LinearGroup: activation ${this.activation} is not supported`);
+    }
+    this.single = new HipMatMul(true);
+    this.single.initialize([]);
+    this.single.activation = this.activation;
+  }
+
+  async run(context, inputs, nOutputs) {
+    context.assertsHipTensorArray(inputs);
+    const problems = [];
+    let next = 0;
+    for (const count of this.arity) {
+      problems.push({ a: inputs[next], w: inputs[next + 1], bias: count === 3 ? inputs[next + 2] : null });
+      next += count;
+    }
+    if (next !== inputs.length || problems.length !== nOutputs) throw new Error("LinearGroup: malformed node");
+    for (const t of inputs) if (t.dataType !== "float32") throw new Error("only float32 is supported");
+    const plain = problems.length <= 16 && problems.every(({ a, w, bias }) => a.ndim === 2 && w.ndim === 2 &&
+      a.dims[1] === w.dims[0] && (!bias || (bias.ndim === 1 && bias.dims[0] === w.dims[1])));
+    if (plain) {
+      const outputs = problems.map(({ a, w }) => context.emptyTensor([a.dims[0], w.dims[1]], "float32"));
+      context.native.linearGroup(problems.map((p) => p.a.handle), problems.map((p) => p.w.handle),
+        problems.map((p) => (p.bias ? p.bias.handle : 0)), outputs.map((o) => o.handle), problems.map((p) => p.a.dims[0]),
+        problems.map((p) => p.w.dims[1]), problems.map((p) => p.a.dims[1]), this.activation === "Relu" ? 1 : 0);
+      return outputs;
+    }
+    const outputs = [];
+    try {
+      for (const { a, w, bias } of problems) {
+        outputs.push(this.single.product(context, a, w, operandView(context, a, []), operandView(context, w, []), bias, null));
+      }
+    } catch (e) {
+      for (const o of outputs) o.dispose();
+      throw e;
+    }
+    return outputs;
+  }
+}
+
 // the buffer an operand is read from: the materialised Transpose if there had to be one
 function operandHandle(view, tensor) {
   return view.temp ? view.temp.handle : tensor.handle;
@@ -139,6 +193,7 @@ function getOpEntries() {
     { opType: "MatMul", backend: "hip", opsetMin: 1, factory: () => new HipMatMul(false) },
     // produced by the hip fusion pass ([Transpose ->] MatMul [* scalar] [+ bias] [+ residual] [+ Relu | -> Transpose])
     { opType: "WebDNNHipFusedMatMul", backend: "hip", opsetMin: 1, factory: () => new HipMatMul(true) },
+    { opType: "WebDNNHipLinearGroup", backend: "hip", opsetMin: 1, factory: () => new HipLinearGroup() },
   ];
 }
 module.exports = { getOpEntries, HipMatMul, operandView };

@@ -281,6 +281,23 @@ FN(js_gemm_ex) {
   return make_undefined(env);
 }
 
+FN(js_linear_group) { /* (A[], W[], Bias[] (0 = none), Y[], m[], n[], k[], epilogue) */
+  ARGS("wdh_linear_group", 8);
+  int64_t a[16], w[16], b[16], y[16], m64[16], n64[16], k64[16];
+  int count = 0, c2 = 0, c3 = 0, c4 = 0, c5 = 0, c6 = 0, c7 = 0;
+  if (!to_i64_list(env, argv[0], a, 16, &count) || !to_i64_list(env, argv[1], w, 16, &c2) ||
+      !to_i64_list(env, argv[2], b, 16, &c3) || !to_i64_list(env, argv[3], y, 16, &c4) ||
+      !to_i64_list(env, argv[4], m64, 16, &c5) || !to_i64_list(env, argv[5], n64, 16, &c6) ||
+      !to_i64_list(env, argv[6], k64, 16, &c7) || c2 != count || c3 != count || c4 != count || c5 != count ||
+      c6 != count || c7 != count)
+    return throw_arg(env, FNAME, "seven integer arrays of one length (<= 16) expected");
+  I64(7, epilogue);
+  int m[16], n[16], k[16];
+  for (int i = 0; i < count; i++) { m[i] = (int)m64[i]; n[i] = (int)n64[i]; k[i] = (int)k64[i]; }
+  CHECK(wdh_linear_group(count, a, w, b, y, m, n, k, (int)epilogue));
+  return make_undefined(env);
+}
+
 FN(js_conv2d) {
   ARGS("wdh_conv2d", 22);
   I64(0, X); I64(1, W); I64(2, Bias); I64(3, Y);
@@ -459,7 +476,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"setOption", js_set_option}, {"alloc", js_alloc}, {"free", js_free}, {"write", js_write},
       {"read", js_read}, {"copy", js_copy}, {"sync", js_sync}, {"memStats", js_mem_stats},
       {"trim", js_trim}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
-      {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
+      {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"linearGroup", js_linear_group}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
       {"softmax", js_softmax}, {"attention", js_attention}, {"layernorm", js_layernorm}, {"layernormAdd", js_layernorm_add}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
