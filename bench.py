@@ -13,14 +13,19 @@ run is eager, the second records the run's kernels into a HIP graph, every timed
 graph (same kernels, same order, one launch) and reads the logits; `extra.resnet50_ms_per_step_eager`
 is the same step through the node-by-node loop.  `value` = 32 * steps / total time.
 
-`roofline` is for the dominant kernel of that workload, the implicit-GEMM contraction kernel: its
-algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over the device time of
+`roofline` is for the dominant kernels of that workload, the implicit-GEMM contraction kernels (the
+1x1 convs read X in place, the 3x3 stride-1 convs stage input rows in LDS, the rest gather taps; all
+share one tile schedule and epilogue): their algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over the device time of
 the timed steps, measured with one HIP event pair on the library's stream around each graph replay
 (the step's three other kernels are inside that bracket, which makes the figure a lower bound).
 `roofline.eager_per_node_events` is the same sum from an eager run with an event at every node
 boundary (a run whose launches were all queued before the device reached them, so the events see
 no host gaps; the events themselves cost the stream a few microseconds each).
-`extra` carries the two single-kernel figures the metric names: Gemm 4096^3 and the config-3 Conv.
+`extra` carries the two single-kernel figures the metric names (Gemm 4096^3 and the config-3 Conv, each
+timed as replays of a HIP graph that holds the launches back to back, with the one-by-one launch time
+beside it), the same ResNet-50 step with the batch handed over as a host tensor on every run
+(`resnet50_host_input_graph`: H2D inside the timed region), configs 2 and 5 with their device time,
+the bandwidth-bound kernels and a per-layer table of the step's 54 contraction launches.
 `cpu_baseline` times the JavaScript restatement of the reference's CPU operators (oracle/js) through
 the same runner with backendOrder ["cpu"] in Node.js on one host core, on three images of the batch (one per run, about 20 s).
 """
@@ -40,10 +45,11 @@ import numpy as np  # noqa: E402
 
 METRIC = "fp32 Gemm/Conv GFLOP/s (% MFMA peak) + ResNet-50 b32 images/sec, 1 MI355X"
 PEAK_FP32_MFMA_TFLOPS = 157.3
-# HBM-side bytes per contraction-kernel launch of the ResNet-50 step, averaged over its 54 launches:
-# rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB device copy;
-# recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read counters itself).
-TRAFFIC_BYTES_PER_LAUNCH = 78.6e6
+# HBM-side bytes per contraction launch of the ResNet-50 step, averaged over its 54 launches (reduce
+# passes included): rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB
+# device copy; recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read
+# counters itself).  The partial sums of tiles cut along K are in it (written once, read once).
+TRAFFIC_BYTES_PER_LAUNCH = 86.1e6
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 
@@ -431,9 +437,10 @@ def main():
                                "(BASELINE config 4)" % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
-            "kernel": "contraction_kernel (implicit-GEMM Conv + Gemm head), %d launches per step; device "
-                      "time = HIP events around each timed graph replay (whole step: includes MaxPool, "
-                      "GlobalAveragePool and the K-split reduce passes)" % resnet["contraction_launches"],
+            "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3 and gathered forms; Gemm "
+                      "head), %d launches per step; device time = HIP events around each timed graph replay "
+                      "(whole step: includes MaxPool, GlobalAveragePool and the K-split reduce passes)"
+                      % resnet["contraction_launches"],
             "achieved": round(achieved, 2),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
