@@ -437,7 +437,11 @@ def test_transpose_all_permutations(ctx, ndim):
                                          ((8, 850, 32), (1, 0, 2)), ((2, 3, 2, 2, 3), (4, 0, 3, 1, 2)),
                                          ((2, 3, 2, 2, 3, 2), (5, 3, 0, 4, 1, 2)), ((64, 64, 3, 3), (2, 3, 1, 0)),
                                          ((1000, 2048), (1, 0)), ((3, 1, 5), (2, 1, 0)), ((4, 300, 16), (0, 2, 1)),
-                                         ((2, 40, 3000), (1, 0, 2)), ((5, 6, 7, 4100), (2, 0, 1, 3))])
+                                         ((2, 40, 3000), (1, 0, 2)), ((5, 6, 7, 4100), (2, 0, 1, 3)),
+                                         # the tiled exchange with 16-byte reads / 8-byte writes: odd and even row
+                                         # lengths of the result, every tile width, rows that start off 8-byte boundaries
+                                         ((2, 850, 8, 32), (0, 2, 3, 1)), ((3, 851, 16), (0, 2, 1)), ((2, 77, 32), (2, 0, 1)),
+                                         ((1, 333, 260), (0, 2, 1)), ((3, 1001, 20), (0, 2, 1)), ((3, 64, 64), (0, 2, 1))])
 def test_transpose_model_shapes(ctx, shape, perm):
     x = nrm(*shape)
     got = H.transpose(ctx, ctx.move_tensor(x), list(perm)).get_data()

@@ -258,12 +258,6 @@ int launch_attention(const AttParams &p, int batch) {
   size_t bytes = (size_t)ATT_ROWS * p.pitch * 4;
   const size_t partials = (size_t)ATT_WAVES * ATT_ROWS * (HD + 1) * 4;
   if (partials > bytes) bytes = partials;
-  static bool raised = false;  // more than 64 KB of dynamic LDS has to be asked for once
-  if (!raised) {
-    WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<HD>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    raised = true;
-  }
   hipLaunchKernelGGL(attention_rows_kernel<HD>, dim3((unsigned)((long long)batch * p.row_blocks)),
                      dim3(64 * ATT_WAVES), bytes, wdh::stream(), p);
   WDH_LAUNCH_CHECK();
@@ -271,6 +265,21 @@ int launch_attention(const AttParams &p, int batch) {
 }
 
 }  // namespace
+
+namespace wdh {
+// More than 64 KB of dynamic LDS has to be asked for once per kernel and device (called by
+// wdh_init with the device current, so that no launch -- captured ones included -- has to).
+int init_attention() {
+  const int limit = 160 * 1024;
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<32>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, limit));
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<64>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, limit));
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<128>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, limit));
+  return WDH_OK;
+}
+}  // namespace wdh
 
 using wdh::fail;
 

@@ -22,6 +22,8 @@ int device();           // the device wdh_init selected
 // Looks up the device address of the static workspace of wdh_gemm_static for `device`,
 // which must be the current device (called by wdh_init).
 int init_static_scratch(int device);
+// Raises the dynamic LDS limit of the attention kernels on the current device (called by wdh_init).
+int init_attention();
 
 // Handle -> device pointer.  Returns nullptr (and records WDH_EINVAL) for an
 // unknown handle.  A zero-byte buffer resolves to a non-null dummy pointer.

@@ -307,6 +307,64 @@ __global__ __launch_bounds__(256) void transpose_tiled_kernel(TileParams p) {
   }
 }
 
+// The same exchange with wider accesses, for inputs whose rows along axis a are 16-byte
+// aligned multiples of four: a thread reads four neighbouring elements of axis a at once
+// and writes two neighbouring elements of the last axis at once (rows of the result start
+// on 8-byte boundaries far more often than on 16-byte ones: 850-float rows do).  12 memory
+// instructions per thread instead of 32; the LDS tile and its odd pitch are unchanged.
+template <int TA>
+__global__ __launch_bounds__(256) void transpose_tiled_wide(TileParams p) {
+  constexpr int TL = 4096 / TA;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  __shared__ uint32_t tile[TL][TA + 1];
+  long long rem = blockIdx.z, in_off = 0, out_off = 0;
+#pragma unroll
+  for (int d = MAXD - 1; d >= 0; d--) {
+    if (d < p.ndim) {
+      long long q = rem / p.oshape[d];
+      long long c = rem - q * p.oshape[d];
+      rem = q;
+      in_off += c * p.osin[d];
+      out_off += c * p.osout[d];
+    }
+  }
+  const unsigned a0 = blockIdx.x * TA, l0 = blockIdx.y * TL;
+  {  // read: TA/4 threads cover a row of the tile along axis a
+    constexpr unsigned TPR = TA / 4;
+    const unsigned ta = (threadIdx.x % TPR) * 4, a = a0 + ta;
+    for (unsigned r = threadIdx.x / TPR; r < TL; r += 256 / TPR) {
+      const unsigned l = l0 + r;
+      if (a < p.na && l < p.nl) {  // na is a multiple of 4: a + 3 < na
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(p.X + in_off + (long long)l * p.l_in + a);
+        tile[r][ta] = v.x; tile[r][ta + 1] = v.y; tile[r][ta + 2] = v.z; tile[r][ta + 3] = v.w;
+      }
+    }
+  }
+  __syncthreads();
+  {  // write: TL/2 threads cover a row of the result, two elements each
+    constexpr unsigned PPR = TL / 2;
+    const unsigned c = (threadIdx.x % PPR) * 2, l = l0 + c;
+    for (unsigned r = threadIdx.x / PPR; r < TA; r += 256 / PPR) {
+      const unsigned a = a0 + r;
+      if (a >= p.na || l >= p.nl) continue;
+      uint32_t *dst = p.Y + out_off + (long long)a * p.a_out + l;
+      const uint32_t v0 = tile[c][r];
+      if (l + 1 < p.nl) {
+        const uint32_t v1 = tile[c + 1][r];
+        if ((reinterpret_cast<uintptr_t>(dst) & 7) == 0) {
+          *reinterpret_cast<u32x2 *>(dst) = u32x2{v0, v1};
+        } else {
+          dst[0] = v0;
+          dst[1] = v1;
+        }
+      } else {
+        dst[0] = v0;
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void gather_axis_kernel(
     const uint32_t *__restrict__ D, const int *__restrict__ Idx,
     uint32_t *__restrict__ Y, long long outer, int axis_len, long long inner,
@@ -498,7 +556,13 @@ extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
     const unsigned gx = (t.na + ta - 1) / ta, gy = (t.nl + tl - 1) / tl;
     if (nouter <= 65535 && gy <= 65535) {
       const dim3 grid(gx, gy, (unsigned)nouter);
-      if (ta == 16) hipLaunchKernelGGL(transpose_tiled_kernel<16>, grid, dim3(256), 0, st, t);
+      bool wide = t.na % 4 == 0 && t.l_in % 4 == 0 && ((uintptr_t)px & 15) == 0;
+      for (int d = 0; d < t.ndim; d++) wide = wide && t.osin[d] % 4 == 0;
+      if (wide) {
+        if (ta == 16) hipLaunchKernelGGL(transpose_tiled_wide<16>, grid, dim3(256), 0, st, t);
+        else if (ta == 32) hipLaunchKernelGGL(transpose_tiled_wide<32>, grid, dim3(256), 0, st, t);
+        else hipLaunchKernelGGL(transpose_tiled_wide<64>, grid, dim3(256), 0, st, t);
+      } else if (ta == 16) hipLaunchKernelGGL(transpose_tiled_kernel<16>, grid, dim3(256), 0, st, t);
       else if (ta == 32) hipLaunchKernelGGL(transpose_tiled_kernel<32>, grid, dim3(256), 0, st, t);
       else hipLaunchKernelGGL(transpose_tiled_kernel<64>, grid, dim3(256), 0, st, t);
       WDH_LAUNCH_CHECK();

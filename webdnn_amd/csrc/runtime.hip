@@ -191,7 +191,8 @@ int wdh_init(int device) {
   }
   WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
   {
-    const int rc = wdh::init_static_scratch(device);
+    int rc = wdh::init_static_scratch(device);
+    if (rc == WDH_OK) rc = wdh::init_attention();
     if (rc != WDH_OK) return rc;
   }
   g.device = device;
