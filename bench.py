@@ -108,6 +108,29 @@ def bench_resnet(steps, warmup, workdir):
     }
 
 
+def bench_resnet_large_batch(steps, warmup, workdir, batch=128):
+    """The same network at four times the batch (not the configured workload, reported in `extra` only):
+    per-launch start-up and drain weigh a quarter as much, which separates what the kernels reach in steady
+    state from what a batch of 32 lets them show."""
+    from webdnn_amd import modelgen
+
+    d = os.path.join(workdir, "resnet50_b%d" % batch)
+    os.makedirs(d, exist_ok=True)
+    data, g = modelgen.resnet50_model(batch=batch)
+    with open(os.path.join(d, "model.onnx"), "wb") as f:
+        f.write(data)
+    inp = os.path.join(d, "input.bin")
+    np.random.default_rng(6).standard_normal((batch, 3, 224, 224)).astype(np.float32).tofile(inp)
+    rep = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--graph", "--measure-all"])
+    assert list(rep["stats"]["nodesByBackend"]) == ["hip"] and rep["graph"]["captured"], rep["stats"]
+    ms = sum(rep["msPerRun"]) / len(rep["msPerRun"])
+    dev_ms = sum(rep["deviceMsPerRun"]) / len(rep["deviceMsPerRun"])
+    return {"workload": "ResNet-50 v1 batch %d, same runner, graph replay, input resident" % batch,
+            "ms_per_step": round(ms, 4), "images_per_s": round(batch / ms * 1e3, 1),
+            "device_ms": round(dev_ms, 4), "device_tflops": round(g.flops / dev_ms / 1e9, 2),
+            "device_frac_mfma_peak": round(g.flops / dev_ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)}
+
+
 def bench_report_only(workdir, steps, warmup):
     """Configs 2 and 5, reported but not part of `value`: the FFN MatMul chain and the DETR-R50-style graph."""
     from webdnn_amd import modelgen
@@ -300,6 +323,8 @@ def bench_resnet_layers(steps, warmup, batch=32):
             ms = timed_steps(ctx, lambda: H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu",
                                                  residual=R).dispose(), steps, warmup)
             m, n, k = w[0], odims[0] * odims[2] * odims[3], w[1] * w[2] * w[3]
+            out_elems = int(np.prod(odims))
+            nbytes = 4 * (int(np.prod(x)) + int(np.prod(w)) + w[0] + out_elems * (2 if residual else 1))
             label = "Conv %dx%d s%d %d->%d @%dx%d%s" % (w[2], w[3], strides[0], x[1], w[0], x[2], x[3],
                                                          " +residual" if residual else "")
             for t in (X, W, B) + ((R,) if R is not None else ()):
@@ -312,17 +337,25 @@ def bench_resnet_layers(steps, warmup, batch=32):
             plan = ctx.last_plan()
             ms = timed_steps(ctx, lambda: H.gemm(ctx, A, Wt, Bv, trans_b=1).dispose(), steps, warmup)
             m, n, k = x[0], w[0], x[1]
+            nbytes = 4 * (x[0] * x[1] + w[0] * w[1] + w[0] + x[0] * w[0])
             label = "Gemm [%d,%d] x [%d,%d]^T" % (x[0], x[1], w[0], w[1])
             for t in (A, Wt, Bv):
                 t.dispose()
         flops = 2.0 * m * n * k
+        # the layer's own roofline: the larger of its matrix-core time and its HBM time at the two peaks
+        mfma_us = flops / PEAK_FP32_MFMA_TFLOPS / 1e6
+        hbm_us = nbytes / 8000.0 / 1e3
         rows.append({"layer": label, "count": info["count"], "m": m, "n": n, "k": k, "us": round(ms * 1e3, 1),
                      "tflops": round(flops / ms / 1e9, 1),
-                     "frac_mfma_peak": round(flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 3), **plan})
+                     "frac_mfma_peak": round(flops / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 3),
+                     "algorithmic_MB": round(nbytes / 1e6, 1),
+                     "bound": "mfma" if mfma_us >= hbm_us else "hbm",
+                     "frac_of_bound": round(max(mfma_us, hbm_us) / (ms * 1e3), 3), **plan})
     total_us = sum(r["us"] * r["count"] for r in rows)
     total_flops = sum(2.0 * r["m"] * r["n"] * r["k"] * r["count"] for r in rows)
     return {"note": "each distinct layer with its fused bias/residual/Relu epilogue and its K-split reduce pass, "
-                    "launches recorded into a HIP graph and replayed back to back; us = HIP events / launches",
+                    "launches recorded into a HIP graph and replayed back to back; us = HIP events / launches; "
+                    "bound / frac_of_bound: max(FLOP / 157.3 TFLOP/s, algorithmic bytes / 8 TB/s) over the time",
             "launches": sum(r["count"] for r in rows), "sum_us": round(total_us, 1),
             "tflops": round(total_flops / total_us / 1e6, 1), "layers": rows}
 
@@ -408,6 +441,7 @@ def main():
     with tempfile.TemporaryDirectory(prefix="webdnn_bench_") as workdir:
         resnet = bench_resnet(args.steps, args.warmup, workdir)
         report_only = bench_report_only(workdir, max(3, args.steps // 2), min(args.warmup, 3))
+        large_batch = bench_resnet_large_batch(max(3, args.steps // 3), 2, workdir)
         baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
     kernels = bench_kernels(args.steps, args.warmup)
     bandwidth = bench_bandwidth(args.steps, args.warmup)
@@ -471,6 +505,7 @@ def main():
                         "(runner.run([CPUTensor]), 19.3 MB over PCIe inside the timed region), graph replay",
                 "ms_per_step": round(resnet["ms_per_step_host_input_graph"], 4),
                 "images_per_s": round(resnet["batch"] / resnet["ms_per_step_host_input_graph"] * 1e3, 1)},
+            "resnet50_b128": large_batch,
             "resnet50_layers": layers,
             "device": resnet["device"],
         },
