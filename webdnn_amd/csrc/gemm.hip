@@ -568,22 +568,26 @@ __device__ __forceinline__ void finish_tile(const Params &p,
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
         const int rbase = __builtin_amdgcn_readfirstlane(row0 + wrow + mt * 32);
-        f32x4 cv[4], rv[4];
-        if (p.C) {
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
+        // Tiles with one or two blocks per wavefront have registers to spare and request the
+        // bias / residual values of all four row groups before the first is used; the
+        // 64-accumulator tiles request them row group by row group (anything else spills).
+        constexpr bool AHEAD = MT * NT <= 2;
+        f32x4 cv[AHEAD ? 4 : 1], rv[AHEAD ? 4 : 1];
+        auto request = [&](int i, int slot) {
+          if (p.C) {
             const int soff = (rbase + 8 * i) * cstride * 4;
             if (c_per_row) {
               const float c = buf_load(rsrc_c, voff_c, soff);
-              cv[i] = f32x4{c, c, c, c};
+              cv[slot] = f32x4{c, c, c, c};
             } else {
-              cv[i] = buf_load4(rsrc_c, voff_c, soff);
+              cv[slot] = buf_load4(rsrc_c, voff_c, soff);
             }
           }
-        }
-        if (p.R) {
+          if (p.R) rv[slot] = buf_load4(rsrc_r, voff_y, (rbase + 8 * i) * ystride * 4);
+        };
+        if constexpr (AHEAD) {
 #pragma unroll
-          for (int i = 0; i < 4; i++) rv[i] = buf_load4(rsrc_r, voff_y, (rbase + 8 * i) * ystride * 4);
+          for (int i = 0; i < 4; i++) request(i, i);
         }
         __builtin_amdgcn_wave_barrier();  // the previous block's reads come first
 #pragma unroll
@@ -592,13 +596,15 @@ __device__ __forceinline__ void finish_tile(const Params &p,
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int i = 0; i < 4; i++) {
+          const int slot = AHEAD ? i : 0;
+          if constexpr (!AHEAD) request(i, 0);
           const f32x4 v = *reinterpret_cast<const f32x4 *>(&st[(lr + 8 * i) * STAGE_LD + lc]);
           f32x4 y;
 #pragma unroll
           for (int e = 0; e < 4; e++) {
             float t = p.alpha * v[e];
-            if (p.C) t = __builtin_fmaf(cv[i][e], p.beta, t);
-            if (p.R) t = t + rv[i][e];
+            if (p.C) t = __builtin_fmaf(cv[slot][e], p.beta, t);
+            if (p.R) t = t + rv[slot][e];
             if (p.epilogue == WDH_EPI_RELU) t = relu_js(t);
             y[e] = t;
           }
