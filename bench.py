@@ -4,7 +4,7 @@
 
 Prints one JSON line.
 
-Workload of `value` (BASELINE config 4): ResNet-50 v1, batch 32, fp32, random-initialised weights
+Workload of `value` (benchmark config 4): ResNet-50 v1, batch 32, fp32, random-initialised weights
 (seeded), BatchNorm folded, run through the Node.js descriptor runner on the `hip` backend
 (WebDNN.load + runner.run) in strict mode — no CPU fallback.  A step is one runner.run() over one
 batch whose input tensor is already resident in HBM; the step ends when the logits are back on the
@@ -468,7 +468,7 @@ def main():
         "config": {"workload": "ResNet-50 v1 batch 32 [32,3,224,224] fp32, random init (seeded), BN folded, "
                                "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict, "
                                "runner.run(x, {graph: true}) replaying the step's captured HIP graph "
-                               "(BASELINE config 4)" % resnet["nodes"]},
+                               "(benchmark config 4)" % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
             "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3 and gathered forms; Gemm "

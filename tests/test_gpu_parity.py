@@ -1,6 +1,6 @@
 """Parity of the hip backend with the oracle, through the C ABI, on a real MI355X.
 
-Criteria (BASELINE.json north_star): bit-exact for indexing / layout / selection ops and for
+Criteria: bit-exact for indexing / layout / selection ops and for
 fp32 Add/Sub/Mul/Div/Relu; max|diff| <= 1e-4 * max|ref| for Gemm / MatMul / Conv.  Softmax and
 LayerNormalization, for which north_star names no figure, use 1e-6 and 1e-5 of max|ref| (the
 oracle evaluates exp in double and rounds once; the kernel evaluates it in fp32).
@@ -47,7 +47,7 @@ def hip_gemm(ctx, A, B, C=None, alpha=1.0, beta=1.0, ta=0, tb=0, epilogue=None):
 
 
 def test_gemm_config1(ctx):
-    """BASELINE config 1: A[256,512], B[1024,512] transB=1, C[1024], alpha=beta=1."""
+    """benchmark config 1: A[256,512], B[1024,512] transB=1, C[1024], alpha=beta=1."""
     A, B, C = uni(256, 512), uni(1024, 512), uni(1024)
     assert_close_max(hip_gemm(ctx, A, B, C, 1.0, 1.0, 0, 1), ref.gemm(A, B, C, 1.0, 1.0, 0, 1), GEMM_TOL, "C1")
 
@@ -129,7 +129,7 @@ def test_matmul_rejects_what_the_reference_rejects(ctx):
 
 
 def test_ffn_chain_config2(ctx):
-    """BASELINE config 2: X[8,512,768] -> MatMul W1 -> Add b1 -> Relu -> MatMul W2 -> Add X.
+    """benchmark config 2: X[8,512,768] -> MatMul W1 -> Add b1 -> Relu -> MatMul W2 -> Add X.
     Full size on the GPU; the oracle follows 64 sampled token rows (the chain is row-wise)."""
     X, W1, b1, W2 = nrm(8, 512, 768), nrm(768, 3072, std=0.02), np.zeros(3072, np.float32), nrm(3072, 768, std=0.02)
     tX, tW1, tb1, tW2 = (ctx.move_tensor(t) for t in (X, W1, b1, W2))
@@ -163,7 +163,7 @@ def he(cout, cin, k):
 
 
 def test_conv_config3_full(ctx):
-    """BASELINE config 3: X[32,64,56,56] U[0,1], W[64,64,3,3] He-normal, bias zeros, pad 1, then Relu."""
+    """benchmark config 3: X[32,64,56,56] U[0,1], W[64,64,3,3] He-normal, bias zeros, pad 1, then Relu."""
     X, W, B = uni(32, 64, 56, 56, lo=0), he(64, 64, 3), np.zeros(64, np.float32)
     want = ref.conv(X, W, B, pads=[1, 1, 1, 1])
     got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])

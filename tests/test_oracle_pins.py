@@ -64,7 +64,7 @@ def test_gemm_brute_force(ta, tb, cshape):
 
 
 def test_gemm_float64_closed_form_config1():
-    # BASELINE config 1: A[256,512] . B[1024,512]^T + C[1024]
+    # benchmark config 1: A[256,512] . B[1024,512]^T + C[1024]
     A, B, C = rnd(256, 512), rnd(1024, 512), rnd(1024)
     want = (A.astype(np.float64) @ B.astype(np.float64).T).astype(np.float32)
     want = (want.astype(np.float64) + C.astype(np.float64)).astype(np.float32)

@@ -1,4 +1,4 @@
-"""Writes the benchmark graphs (BASELINE configs 1-5) as model directories for the Node.js runner.
+"""Writes the benchmark graphs (benchmark configs 1-5) as model directories for the Node.js runner.
 
     python -m webdnn_amd.write_models OUT_DIR [gemm ffn conv resnet50 detr]
 
