@@ -566,6 +566,16 @@ def test_slice_ranks_ints_and_errors(ctx):
     big = nrm(32, 256, 56, 56)                                     # crop of a feature map, 100 MB in
     args = dict(starts=[4, 3], ends=[52, 53], axes=[2, 3])
     assert_bit_exact(H.slice_(ctx, ctx.move_tensor(big), **args).get_data(), ref.slice_(big, **args))
+    rows = nrm(2, 3, 200, 300)                                     # short odd rows gathered into a dense plane
+    tr = ctx.move_tensor(rows)
+    for args in (dict(starts=[5, 1], ends=[190, 52], axes=[2, 3]),                 # plane of 9435: several workgroups
+                 dict(starts=[199, 3], ends=[-500, 10], axes=[2, 3], steps=[-1, 1]),  # rows taken backwards
+                 dict(starts=[0, 250], ends=[200, 299], axes=[2, 3], steps=[3, 1]),   # every third row
+                 dict(starts=[1, 0, 17], ends=[3, 37, 50], axes=[1, 2, 3])):
+        assert_bit_exact(H.slice_(ctx, tr, **args).get_data(), ref.slice_(rows, **args), "slice %s" % args)
+    r5 = nrm(2, 3, 2, 40, 45)
+    args = dict(starts=[1, 2, 1], ends=[3, 40, 44], axes=[1, 3, 4])
+    assert_bit_exact(H.slice_(ctx, ctx.move_tensor(r5), **args).get_data(), ref.slice_(r5, **args))
     wide = nrm(6, 8, 4400)                                         # long rows: 16-byte pieces where alignment allows
     tw = ctx.move_tensor(wide)
     for args in (dict(starts=[7], ends=[-100], axes=[1], steps=[-1]), dict(starts=[4], ends=[4300], axes=[2]),

@@ -58,6 +58,7 @@
 #include <vector>
 
 #include "common.h"
+#include "fastdiv.h"
 
 // Workspace of wdh_gemm_static: the partial sums of tiles cut along K, held in the
 // library's own image instead of pool memory so that the call allocates nothing.
@@ -91,6 +92,10 @@ int init_static_scratch(int device) {
 
 namespace {
 
+using wdh::FastDiv;
+using wdh::make_fastdiv;
+using wdh::fdiv;
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -119,30 +124,6 @@ __device__ __forceinline__ void buf_store(rsrc_t r, float v, int voff, int soff)
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void buf_store4(rsrc_t r, f32x4 v, int voff, int soff) {
   __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
-}
-
-// Division of a non-negative 32-bit integer by a divisor fixed for the launch: the
-// host turns the divisor into a multiplier and a shift, the kernel pays one
-// multiply-high and one shift instead of the ~40 instructions of a hardware-less
-// integer division.  Exact for 0 <= n < 2^31.
-struct FastDiv {
-  unsigned mul;    // 0: the divisor is 1
-  unsigned shift;
-  int d;
-};
-inline FastDiv make_fastdiv(long long divisor) {
-  FastDiv f = {0u, 0u, (int)divisor};
-  if (divisor <= 1) return f;
-  unsigned lg = 0;
-  while ((1ll << lg) < divisor) lg++;
-  const unsigned pw = 31 + lg;
-  f.mul = (unsigned)((((unsigned long long)1 << pw) + (unsigned long long)divisor - 1) /
-                     (unsigned long long)divisor);
-  f.shift = pw - 32;
-  return f;
-}
-__device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
-  return f.mul ? (int)(__umulhi((unsigned)n, f.mul) >> f.shift) : n;
 }
 
 constexpr int BK = 16;
