@@ -243,7 +243,10 @@ def test_conv_1x1_equals_gemm(ctx):
                                    ((2, 1, 3, 1, 2, 1), (1, 2, 1, 2, 1, 3)), ((5, 7), (5, 1)), ((1, 3, 1, 12), (2, 3, 10, 12)),
                                    ((3, 1031), (3, 1031)), ((2, 64, 7, 7), (1, 64, 1, 1)), ((850, 1, 256), (850, 1, 1)),
                                    ((3, 5000), (3, 1)), ((2, 5, 4101), (5, 1)), ((4, 16, 28, 28), (16, 1, 1)),
-                                   ((16, 1, 1), (4, 16, 28, 28)), ((7, 300), (300,)), ((4100,), (1,))])
+                                   ((16, 1, 1), (4, 16, 28, 28)), ((7, 300), (300,)), ((4100,), (1,)),
+                                   # rows that fill power-of-two tiles badly: the flat walk, 16-byte and 4-byte units
+                                   ((3, 64, 56, 56), (64, 1, 1)), ((64, 1, 1), (3, 64, 56, 56)), ((2, 3, 37, 50), (3, 1, 50)),
+                                   ((2, 2, 3, 70, 50), (2, 1, 70, 1)), ((300, 50), (50,)), ((2, 40, 2500), (1, 40, 1))])
 def test_binary_bit_exact(ctx, op, sl, sr):
     L, R = uni(*sl, lo=-3, hi=3), uni(*sr, lo=-3, hi=3)
     got = H.binary(ctx, op, ctx.move_tensor(L), ctx.move_tensor(R))
@@ -263,6 +266,11 @@ def test_binary_special_values_int32_pow_and_errors(ctx):
     for op in ("Add", "Sub", "Mul", "Div"):
         got = H.binary(ctx, op, ctx.move_tensor(a), ctx.move_tensor(b)).get_data()
         assert_bit_exact(got, ref.binary(op, a, b), op + " int32")
+    ia = RNG.integers(-2 ** 31, 2 ** 31 - 1, (3, 37, 50)).astype(np.int32)    # int32 through the flat walk
+    ib = RNG.integers(-50000, 50000, (37, 1)).astype(np.int32)
+    for op in ("Add", "Mul"):
+        got = H.binary(ctx, op, ctx.move_tensor(ia), ctx.move_tensor(ib)).get_data()
+        assert_bit_exact(got, ref.binary(op, ia, ib), op + " int32, broadcast rows")
     base, ex = uni(4, 50, lo=0.1, hi=4), uni(50, lo=-3, hi=3)
     got = H.binary(ctx, "Pow", ctx.move_tensor(base), ctx.move_tensor(ex)).get_data()
     assert_close_max(got, ref.binary("Pow", base, ex), 1e-6, "Pow")

@@ -8,7 +8,10 @@
 // so those are single fp32 instructions here (compiled with contraction off).
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.h"
+#include "fastdiv.h"
 #include "plane_walk.h"
 
 namespace {
@@ -155,6 +158,67 @@ __global__ __launch_bounds__(256) void binary_plane(BinaryParams p, wdh::PlaneWa
   }
 }
 
+// The flat walk of plane_walk.h over the same views, for rows that fill the tiles above
+// badly (a bias added to planes of 56x56 = 784 units): consecutive threads take
+// consecutive units of the result whatever the row length.
+template <int OP, typename T, int UNIT>
+__global__ __launch_bounds__(256) void binary_flat(BinaryParams p, wdh::FlatWalk f, wdh::FastDiv fd_inner) {
+  const wdh::FlatPos q = wdh::flat_position(f);
+  long long bl = 0, br = 0;
+#pragma unroll
+  for (int d = 0; d < MAXD - 2; d++) {
+    if (d < f.n_outer) {
+      bl += (long long)q.oc[d] * p.sl[d];
+      br += (long long)q.oc[d] * p.sr[d];
+    }
+  }
+  const int nd = f.n_outer + 2;
+  const long long sl2 = p.sl[nd - 2], sr2 = p.sr[nd - 2];
+  const long long sl1 = p.sl[nd - 1] * UNIT, sr1 = p.sr[nd - 1] * UNIT;
+  const T *L = (const T *)p.L + bl, *R = (const T *)p.R + br;
+  T *Y = (T *)p.Y + (long long)q.outer_linear * f.plane * UNIT;
+  typedef typename std::conditional<UNIT == 4, f32x4, T>::type V;
+  for (unsigned u0 = q.begin + threadIdx.x; u0 < q.end; u0 += 1024) {
+    V a[4], b[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const unsigned u = u0 + 256 * k;
+      if (u < q.end) {
+        const unsigned row = (unsigned)wdh::fdiv((int)u, fd_inner), col = u - row * f.inner;
+        const T *l = L + (long long)row * sl2 + (long long)col * sl1;
+        const T *r = R + (long long)row * sr2 + (long long)col * sr1;
+        if constexpr (UNIT == 4) {
+          if (sl1) a[k] = *reinterpret_cast<const f32x4 *>(l);
+          else { const float s = *l; a[k] = f32x4{s, s, s, s}; }
+          if (sr1) b[k] = *reinterpret_cast<const f32x4 *>(r);
+          else { const float s = *r; b[k] = f32x4{s, s, s, s}; }
+        } else {
+          a[k] = *l;
+          b[k] = *r;
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const unsigned u = u0 + 256 * k;
+      if (u < q.end) {
+        if constexpr (UNIT == 4) {
+          f32x4 v;
+          v.x = apply_f<OP>(a[k].x, b[k].x);
+          v.y = apply_f<OP>(a[k].y, b[k].y);
+          v.z = apply_f<OP>(a[k].z, b[k].z);
+          v.w = apply_f<OP>(a[k].w, b[k].w);
+          *reinterpret_cast<f32x4 *>(Y + (long long)u * 4) = v;
+        } else if constexpr (__is_same(T, float)) {
+          Y[u] = apply_f<OP>(a[k], b[k]);
+        } else {
+          Y[u] = apply_i<OP>(a[k], b[k]);
+        }
+      }
+    }
+  }
+}
+
 // General path: one output element per thread per step, any strides.
 template <int OP, typename T, typename IDX>
 __global__ __launch_bounds__(256) void binary_general(BinaryParams p) {
@@ -204,10 +268,24 @@ int launch_binary(const BinaryParams &p, int dtype, bool dense, bool vec) {
   hipStream_t st = wdh::stream();
   const bool small = p.total <= 0xffffffffLL;
   wdh::PlaneWalk w;
+  wdh::FlatWalk fw;
+  const bool vec4 = dtype == 0 && vec;
+  const unsigned inner_units = vec4 ? p.shape[p.ndim - 1] / 4 : p.shape[p.ndim - 1];
   if (dtype == 0 && dense) {
     hipLaunchKernelGGL(binary_dense_f32<OP>, dim3(grid_for((p.total + 3) / 4, 256)),
                        dim3(256), 0, st, (const float *)p.L, (const float *)p.R,
                        (float *)p.Y, p.total);
+  } else if (p.ndim >= 2 &&
+             (!wdh::plan_plane_walk(&w, p.ndim, p.shape, inner_units) || wdh::plane_walk_fill(w) < 0.9) &&
+             wdh::plan_flat_walk(&fw, p.ndim, p.shape, inner_units)) {
+    const dim3 grid(fw.outer * fw.chunks);
+    const wdh::FastDiv fd = wdh::make_fastdiv(fw.inner);
+    if (vec4)
+      hipLaunchKernelGGL((binary_flat<OP, float, 4>), grid, dim3(256), 0, st, p, fw, fd);
+    else if (dtype == 0)
+      hipLaunchKernelGGL((binary_flat<OP, float, 1>), grid, dim3(256), 0, st, p, fw, fd);
+    else
+      hipLaunchKernelGGL((binary_flat<OP, int, 1>), grid, dim3(256), 0, st, p, fw, fd);
   } else if (dtype == 0 && vec &&
              wdh::plan_plane_walk(&w, p.ndim, p.shape, p.shape[p.ndim - 1] / 4)) {
     hipLaunchKernelGGL((binary_plane<OP, float, 4>), wdh::plane_grid(w), dim3(256), 0, st,

@@ -79,7 +79,74 @@ inline bool plan_plane_walk(PlaneWalk *w, int nd, const unsigned *shape, unsigne
   return true;
 }
 
+// Share of the walk's thread items that fall inside the plane of the last two axes.
+inline double plane_walk_fill(const PlaneWalk &w) {
+  const unsigned tx = 1u << w.tx_log2, ty = 256u >> w.tx_log2;
+  const double px = w.wide ? 4.0 * tx : tx, py = w.wide ? ty : 4.0 * ty;
+  return (double)w.shape[w.nd - 1] * w.shape[w.nd - 2] / ((double)w.xchunks * px * (double)w.ychunks * py);
+}
+
+// The other walk over the same view, for rows the tiles above fit badly (784 or 50 units
+// leave a quarter of a power-of-two tile empty): the plane of the last two axes is taken
+// as one run of second * inner units, cut into chunks of a workgroup each, thread t of
+// which takes units t, t + 256, ...; a unit's row is one multiply-high away.  Only a
+// plane's last wavefront is ragged.  The result must be dense over the plane.
+struct FlatWalk {
+  unsigned plane;    // second * inner, in units
+  unsigned inner;    // units per row
+  unsigned chunk;    // units per workgroup
+  unsigned chunks;   // workgroups per plane
+  unsigned outer;    // product of the outer extents
+  int n_outer;
+  unsigned oshape[WALK_MAXD];
+};
+
+inline bool plan_flat_walk(FlatWalk *f, int nd, const unsigned *shape, unsigned inner_units) {
+  if (nd < 2 || nd > WALK_MAXD || inner_units == 0) return false;
+  const unsigned long long plane = (unsigned long long)shape[nd - 2] * inner_units;
+  if (plane < 256 || plane >= 0x7fffffffULL) return false;
+  unsigned long long outer = 1;
+  for (int d = 0; d + 2 < nd; d++) {
+    outer *= shape[d];
+    if (outer > 0x7fffffffULL) return false;
+    f->oshape[d] = shape[d];
+  }
+  f->plane = (unsigned)plane;
+  f->inner = inner_units;
+  f->chunk = plane <= 8192 ? (unsigned)plane : 4096u;
+  f->chunks = (unsigned)((plane + f->chunk - 1) / f->chunk);
+  f->outer = (unsigned)outer;
+  f->n_outer = nd - 2;
+  return outer * f->chunks <= 0x7fffffffULL;
+}
+
 #ifdef __HIPCC__
+// Where a workgroup of a flat walk works: its coordinates on the outer axes, their linear
+// index, and the range [begin, end) of the plane's units it covers.
+struct FlatPos {
+  unsigned oc[WALK_MAXD];
+  unsigned outer_linear, begin, end;
+};
+__device__ __forceinline__ FlatPos flat_position(const FlatWalk &f) {
+  FlatPos q;
+  unsigned b = blockIdx.x;
+  const unsigned c = b % f.chunks;
+  b /= f.chunks;
+  q.outer_linear = b;
+#pragma unroll
+  for (int d = WALK_MAXD - 3; d >= 0; d--) {
+    q.oc[d] = 0;
+    if (d < f.n_outer) {
+      const unsigned t = b / f.oshape[d];
+      q.oc[d] = b - t * f.oshape[d];
+      b = t;
+    }
+  }
+  q.begin = c * f.chunk;
+  q.end = q.begin + f.chunk < f.plane ? q.begin + f.chunk : f.plane;
+  return q;
+}
+
 // The launch grid of a planned walk.  The three-axis form hands the kernel its
 // tile and outer index without any division; extents beyond a grid axis's
 // limit fall back to one folded axis.

@@ -261,49 +261,36 @@ __global__ __launch_bounds__(256) void copy_plane(StridedCopyParams p, wdh::Plan
 struct FlatCopyParams {
   const uint32_t *X;
   uint32_t *Y;
-  unsigned plane;       // elements of the result plane (second * inner)
-  unsigned inner;       // row length
-  unsigned chunk;       // elements per workgroup, a multiple of 1024 (or the whole plane)
-  unsigned chunks;      // workgroups per plane
   wdh::FastDiv fd_inner;
   long long sx2;        // input stride between rows
-  int n_outer;
-  unsigned oshape[MAXD];
   long long osx[MAXD], osy[MAXD];
 };
-__global__ __launch_bounds__(256) void copy_rows_flat(FlatCopyParams p) {
-  unsigned b = blockIdx.x;
-  const unsigned chunk_idx = b % p.chunks;
-  b /= p.chunks;
+__global__ __launch_bounds__(256) void copy_rows_flat(FlatCopyParams p, wdh::FlatWalk f) {
+  const wdh::FlatPos q = wdh::flat_position(f);
   long long bx = 0, by = 0;
 #pragma unroll
-  for (int d = MAXD - 1; d >= 0; d--) {
-    if (d < p.n_outer) {
-      const unsigned q = b / p.oshape[d];
-      const unsigned c = b - q * p.oshape[d];
-      b = q;
-      bx += (long long)c * p.osx[d];
-      by += (long long)c * p.osy[d];
+  for (int d = 0; d < MAXD - 2; d++) {
+    if (d < f.n_outer) {
+      bx += (long long)q.oc[d] * p.osx[d];
+      by += (long long)q.oc[d] * p.osy[d];
     }
   }
-  const unsigned begin = chunk_idx * p.chunk;
-  const unsigned end = begin + p.chunk < p.plane ? begin + p.chunk : p.plane;
   const uint32_t *x = p.X + bx;
   uint32_t *y = p.Y + by;
-  for (unsigned f0 = begin + threadIdx.x; f0 < end; f0 += 1024) {
+  for (unsigned f0 = q.begin + threadIdx.x; f0 < q.end; f0 += 1024) {
     uint32_t v[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const unsigned f = f0 + 256 * k;
-      if (f < end) {
-        const unsigned row = (unsigned)wdh::fdiv((int)f, p.fd_inner);
-        v[k] = x[(long long)row * p.sx2 + (f - row * p.inner)];
+      const unsigned u = f0 + 256 * k;
+      if (u < q.end) {
+        const unsigned row = (unsigned)wdh::fdiv((int)u, p.fd_inner);
+        v[k] = x[(long long)row * p.sx2 + (u - row * f.inner)];
       }
     }
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const unsigned f = f0 + 256 * k;
-      if (f < end) y[f] = v[k];
+      const unsigned u = f0 + 256 * k;
+      if (u < q.end) y[u] = v[k];
     }
   }
 }
@@ -459,32 +446,17 @@ int launch_strided_copy(const StridedCopyParams &g) {
   wdh::PlaneWalk w;
   const bool walk = wdh::plan_plane_walk(&w, nd, g.shape, vec ? g.shape[nd - 1] / 4 : g.shape[nd - 1]);
   // a dense result plane whose rows the tiled walk would cover badly: the flat walk
-  if (!vec && nd >= 2 && g.sx[nd - 1] == 1 && g.sy[nd - 1] == 1 && g.sy[nd - 2] == (long long)g.shape[nd - 1]) {
-    const unsigned long long plane = (unsigned long long)g.shape[nd - 2] * g.shape[nd - 1];
-    double eff = 0.0;
-    if (walk) {
-      const unsigned tx = 1u << w.tx_log2, ty = 256u >> w.tx_log2;
-      const double px = w.wide ? 4.0 * tx : tx, py = w.wide ? ty : 4.0 * ty;
-      eff = (double)plane / ((double)w.xchunks * px * (double)w.ychunks * py);
-    }
-    unsigned long long outer = 1;
-    for (int d = 0; d + 2 < nd; d++) outer *= g.shape[d];
-    if (eff < 0.9 && plane >= 256 && plane < 0x7fffffffULL) {
-      FlatCopyParams f = {};
-      f.X = g.X; f.Y = g.Y;
-      f.plane = (unsigned)plane; f.inner = g.shape[nd - 1];
-      f.chunk = plane <= 8192 ? (unsigned)plane : 4096u;
-      f.chunks = (unsigned)((plane + f.chunk - 1) / f.chunk);
-      f.fd_inner = wdh::make_fastdiv(f.inner);
-      f.sx2 = g.sx[nd - 2];
-      f.n_outer = nd - 2;
-      for (int d = 0; d < nd - 2; d++) { f.oshape[d] = g.shape[d]; f.osx[d] = g.sx[d]; f.osy[d] = g.sy[d]; }
-      if (outer * f.chunks <= 0x7fffffffULL) {
-        hipLaunchKernelGGL(copy_rows_flat, dim3((unsigned)(outer * f.chunks)), dim3(256), 0, st, f);
-        WDH_LAUNCH_CHECK();
-        return WDH_OK;
-      }
-    }
+  wdh::FlatWalk fw;
+  if (!vec && nd >= 2 && g.sx[nd - 1] == 1 && g.sy[nd - 1] == 1 && g.sy[nd - 2] == (long long)g.shape[nd - 1] &&
+      (!walk || wdh::plane_walk_fill(w) < 0.9) && wdh::plan_flat_walk(&fw, nd, g.shape, g.shape[nd - 1])) {
+    FlatCopyParams f = {};
+    f.X = g.X; f.Y = g.Y;
+    f.fd_inner = wdh::make_fastdiv(fw.inner);
+    f.sx2 = g.sx[nd - 2];
+    for (int d = 0; d < nd - 2; d++) { f.osx[d] = g.sx[d]; f.osy[d] = g.sy[d]; }
+    hipLaunchKernelGGL(copy_rows_flat, dim3(fw.outer * fw.chunks), dim3(256), 0, st, f, fw);
+    WDH_LAUNCH_CHECK();
+    return WDH_OK;
   }
   if (walk) {
     StridedCopyParams s = g;
