@@ -78,6 +78,11 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       input rows of a tile in LDS and read the taps from there;
  *                       0 = they gather taps from global memory like every other
  *                       geometry (both forms compute the same sums).
+ *   "conv_stem"         1 (default) = a 7x7, stride-2, undilated convolution from 3 to 64
+ *                       channels (the stem of an image network) runs in a kernel that keeps
+ *                       all weights and a tile's input patch in LDS; 0 = it gathers taps
+ *                       from global memory like every other geometry (same sums, added
+ *                       in another order).
  *   "gemm_wavesplit"    1 (default) = a Gemm / MatMul with few result tiles and K >= 128
  *                       runs as one launch of 32x32 blocks whose 16 wavefronts share K
  *                       among themselves; 0 = it takes the ordinary tiles (K cut across
@@ -109,6 +114,8 @@ int wdh_set_option(const char *name, int value);
 #define WDH_FORM_CONV_GATHER_FLAT 4 /* ... more taps or X of 2 GiB or more      */
 #define WDH_FORM_CONV_PIXELS 5    /* 1x1 stride 1: X read in place              */
 #define WDH_FORM_CONV3X3_LDS 6    /* 3x3 stride 1: taps read from an LDS tile   */
+#define WDH_FORM_CONV_STEM 7      /* 7x7 stride 2, 3 -> 64 channels: weights and the
+                                   * input patch of an 8x16-pixel tile in LDS   */
 int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles,
                   int64_t *split_tiles, int *split, int *form);
 

@@ -1001,6 +1001,60 @@ def test_conv3x3_lds_tile_kernel(ctx, shape):
     assert_close_max(got[1], got[0], 1e-5, "LDS-tile form vs gathered form")
 
 
+STEM_CONVS = [
+    # n, h, w, pads: 7x7 stride 2, 3 -> 64 channels -> the kernel with weights and patch in LDS
+    (2, 224, 224, [3, 3, 3, 3]),     # the ResNet stem: 14 x 7 whole tiles per image
+    (1, 64, 96, [3, 3, 3, 3]),
+    (3, 37, 53, [3, 3, 3, 3]),       # odd sizes: ragged tiles on both axes
+    (2, 40, 70, [2, 3, 3, 1]),       # unequal pads
+    (2, 45, 33, [0, 0, 0, 0]),       # no padding
+    (5, 7, 7, [0, 0, 0, 0]),         # one output pixel per image
+    (1, 9, 200, [5, 6, 4, 7]),       # pads wider than half the kernel
+]
+
+
+@pytest.mark.parametrize("shape", STEM_CONVS)
+def test_conv7x7_stem_kernel(ctx, shape):
+    n, h, w, pads = shape
+    X, W, B = uni(n, 3, h, w, lo=-1), he(64, 3, 7), nrm(64)
+    want = ref.conv(X, W, B, None, 1, None, pads, [2, 2])
+    R = nrm(*want.shape)
+    got = {}
+    for stem in (1, 0):
+        try:
+            ctx.set_option("conv_stem", stem)
+            got[stem] = hip_conv(ctx, X, W, B, None, 1, pads, [2, 2])
+            form = ctx.last_plan()["form"]
+            nobias = hip_conv(ctx, X, W, None, None, 1, pads, [2, 2])
+            fused = hip_conv(ctx, X, W, B, None, 1, pads, [2, 2], epilogue="relu", R=R)
+        finally:
+            ctx.set_option("conv_stem", 1)
+        assert ("stem" in form) == bool(stem), form
+        assert_close_max(got[stem], want, GEMM_TOL, "stem %d %s" % (stem, shape))
+        assert_close_max(nobias, want - B.reshape(1, 64, 1, 1), GEMM_TOL, "stem %d, no bias %s" % (stem, shape))
+        assert_bit_exact(fused, np.maximum(got[stem] + R, 0) + 0.0, "stem %d + residual + relu" % stem)
+    assert_close_max(got[1], got[0], 1e-5, "stem kernel vs gathered form")
+
+
+def test_conv7x7_stem_kernel_keeps_nan_and_inf_inside_their_receptive_fields(ctx):
+    """One step of the stem kernel's K order has no partner tap: what the idle half of the wavefront
+    multiplies must be a true zero, or an Inf elsewhere in the tile's patch would leak into every pixel."""
+    X, W = uni(1, 3, 40, 40, lo=-1), he(64, 3, 7)
+    X[0, 1, 20, 21] = np.inf
+    X[0, 2, 5, 30] = np.nan
+    got = {}
+    for stem in (1, 0):
+        try:
+            ctx.set_option("conv_stem", stem)
+            got[stem] = hip_conv(ctx, X, W, None, None, 1, [3, 3, 3, 3], [2, 2])
+        finally:
+            ctx.set_option("conv_stem", 1)
+    assert np.array_equal(np.isfinite(got[1]), np.isfinite(got[0]))
+    assert 0 < np.count_nonzero(~np.isfinite(got[1])) < got[1].size // 4
+    fin = np.isfinite(got[0])
+    assert_close_max(got[1][fin], got[0][fin], 1e-5, "finite outputs")
+
+
 @pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 def test_conv3x3_lds_tile_kernel_every_tile_shape(ctx, tile):
     """The LDS-tile kernel exists for the same five workgroup tiles as the gathered form."""

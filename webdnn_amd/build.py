@@ -17,7 +17,7 @@ LIB = os.path.join(LIBDIR, "libwebdnn_hip.so")
 ADDON_SRC = os.path.join(ROOT, "webdnn_amd", "napi", "addon.c")
 ADDON = os.path.join(LIBDIR, "webdnn_hip.node")
 
-HIP_SOURCES = ["runtime.hip", "gemm.hip", "elementwise.hip", "reduce.hip", "attention.hip", "pool_layout.hip"]
+HIP_SOURCES = ["runtime.hip", "gemm.hip", "conv_patch.hip", "elementwise.hip", "reduce.hip", "attention.hip", "pool_layout.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -33,6 +33,11 @@ void *resolve(wdh_buf h, size_t *bytes);
 // On failure returns false after recording the error (`what` names the operand).
 bool operand(wdh_buf h, size_t need, const char *what, void **out);
 
+// The stem convolution's own kernel (conv_patch.hip): whether a geometry qualifies, and the launch.
+bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group);
+int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
+                      int h, int w, int oh, int ow, int pt, int pl, int relu);
+
 // Frees the per-geometry tap tables of the conv kernel (called at shutdown).
 void release_conv_tables();
 

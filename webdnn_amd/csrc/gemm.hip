@@ -1419,6 +1419,7 @@ struct GroupQueue {
   long long blocks[16];
   int variant[16];  // 2 * B_IS_KC + VEC
 } g_group;
+int g_stem = 1;           // 0: the 7x7 stride-2 stem conv gathers its taps like any other geometry
 int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
 
 // Whether whole tiles may leave in 16-byte stores: Y (and the residual, which has Y's
@@ -1693,6 +1694,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: wide_stores %d (use 0 or 1)", value);
     g_wide_stores = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "conv_stem") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: conv_stem %d (use 0 or 1)", value);
+    g_stem = value;
     return WDH_OK;
   }
   if (strcmp(name, "conv3x3_halo") == 0) {
@@ -2023,6 +2030,12 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.fd_oh = make_fastdiv(oh);
   p.cv.fd_ohw = make_fastdiv((long long)oh * ow);
   p.cv.fd_plane = make_fastdiv((long long)h * w);
+
+  if (g_stem && wdh::conv_patch_applies(c, cout, kh, kw, sh, sw, dh, dw, group)) {
+    const long long tiles = (long long)n * ((oh + 7) / 8) * ((ow + 15) / 16);
+    g_last_plan = {64, 128, 1, WDH_FORM_CONV_STEM, tiles, 0};
+    return wdh::conv_patch_launch(p.B, p.A, p.C, p.R, p.Y, n, h, w, oh, ow, pt, pl, epilogue == WDH_EPI_RELU);
+  }
 
   const int ntaps = kh * kw;
   // Descriptor loads need every byte offset formed in the kernel (X, shifted up

@@ -153,7 +153,8 @@ class HipContext:
         call("wdh_set_option", name.encode(), int(value))
 
     FORMS = ("gemm, B k-contiguous", "gemm, B n-contiguous", "conv, gathered taps", "conv, gathered taps (32-63)",
-             "conv, gathered taps (flat loads)", "conv 1x1, X in place", "conv 3x3, LDS tile")
+             "conv, gathered taps (flat loads)", "conv 1x1, X in place", "conv 3x3, LDS tile",
+             "conv 7x7 s2 stem, weights and patch in LDS")
 
     def last_plan(self):
         """Layout of the most recent Gemm / Conv launch: tile, whole tiles, tiles cut along K, chunks, form."""
