@@ -34,7 +34,8 @@ void *resolve(wdh_buf h, size_t *bytes);
 bool operand(wdh_buf h, size_t need, const char *what, void **out);
 
 // The stem convolution's own kernel (conv_patch.hip): whether a geometry qualifies, and the launch.
-bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group);
+bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int oh,
+                        int ow);
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
                       int h, int w, int oh, int ow, int pt, int pl, int relu);
 

@@ -24,8 +24,12 @@
 // copied to LDS.  Sums therefore associate differently from the gathered form (as between
 // any two tile shapes); both are within the contraction tolerance of the oracle.
 #include "common.h"
+#include "fastdiv.h"
 
 namespace {
+
+using wdh::FastDiv;
+using wdh::fdiv;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -47,11 +51,23 @@ constexpr int LDW = 8 * STEP_GROUPS + 4;             // 164 floats per weight ro
 static_assert(STRIDE * ROWP % 32 == 16, "the two pixel rows of a block must land 16 banks apart");
 static_assert((LDW / 4) % 2 == 1, "weight rows must not line up on the banks");
 
+// Y and the residual are written and read through buffer descriptors that span one image's
+// 64 planes: the lane's part of the address is one byte offset per tile, the channel's part a
+// scalar offset, and a lane whose pixel lies outside the image carries an offset outside
+// every window, which the hardware drops: no address arithmetic and no branch per element.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int BUF_WORD3 = 0x00020000;
+constexpr int BUF_OUTSIDE = (int)0x80000000u;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, BUF_WORD3);
+}
+
 struct PatchParams {
   const float *X, *W, *Bias, *R;
   float *Y;
   int n, h, w, oh, ow, pt, pl;
   int tiles_x, tiles_y, ntiles;
+  FastDiv fd_per_image, fd_tiles_x;
   int relu;
 };
 
@@ -125,9 +141,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParam
   struct Origin { int img, oy0, ox0; };
   auto tile_origin = [&](int tile) {
     Origin o;
-    o.img = tile / per_image;
+    o.img = fdiv(tile, p.fd_per_image);
     const int r = tile - o.img * per_image;
-    const int ty = r / p.tiles_x;
+    const int ty = fdiv(r, p.fd_tiles_x);
     o.oy0 = ty * TH;
     o.ox0 = (r - ty * p.tiles_x) * TW;
     return o;
@@ -162,12 +178,42 @@ __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParam
   const int py = 2 * wave + (li >> 4), px = li & 15;
   const int corner = py * (STRIDE * ROWP) + px;
 
+  // ---- the epilogue of a tile, one element at a time ---------------------------------------
+  // It runs while the NEXT tile is multiplied: a few elements after each group of matrix-core
+  // instructions, whose 64 cycles apiece hide the additions and the stores.  (Run after the
+  // tile's own last product instead, it left the matrix cores idle a third of the time: the
+  // two workgroups of a CU fall into step, and then both are in their epilogue at once.)
+  const int plane = p.oh * p.ow;  // 64 planes of it stay below 2^29 elements (checked by the host)
+  struct Pending {
+    f32x16 sums[2];
+    rsrc_t y, r;
+    int lane_off;   // bytes from the image's first result to channel 4*half of the lane's pixel
+  };
+  auto open_pending = [&](Pending &d, const Origin &o, bool valid) {
+    const long long image = (long long)o.img * COUT * plane;
+    d.y = make_rsrc(p.Y + image, COUT * plane * 4);
+    d.r = make_rsrc((p.R ? p.R : p.Y) + image, COUT * plane * 4);
+    const int oy = o.oy0 + py, ox = o.ox0 + px;
+    d.lane_off = valid && oy < p.oh && ox < p.ow ? (4 * half * plane + oy * p.ow + ox) * 4 : BUF_OUTSIDE;
+  };
+  auto finish_element = [&](const Pending &d, int e) {  // e: compile-time 0..31
+    const int mt = e >> 4, r = e & 15;
+    const int soff = (32 * mt + 8 * (r >> 2) + (r & 3)) * plane * 4;
+    float v = d.sums[mt][r];
+    if (p.Bias) v = v + bias[mt][r];
+    if (p.R) v = v + __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(d.r, d.lane_off, soff, 0));
+    if (p.relu) v = relu_js(v);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), d.y, d.lane_off, soff, 0);
+  };
+
   int tile = blockIdx.x;  // the host launches at most ntiles workgroups
   Origin here = tile_origin(tile);
   fetch(here);
   stash(0);
   __syncthreads();
   int buf = 0;
+  Pending done;
+  open_pending(done, here, false);  // nothing to finish during the first tile
   for (;;) {
     const int next = tile + (int)gridDim.x;
     Origin there = here;
@@ -215,32 +261,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParam
         acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.a0[s], cur.b[s], acc[0], 0, 0, 0);
         acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.a1[s], cur.b[s], acc[1], 0, 0, 0);
       }
+      // two elements of the previous tile per group: 32 elements over the first 16 groups
+      if (g < 16) {
+        finish_element(done, 2 * g);
+        finish_element(done, 2 * g + 1);
+      }
       __builtin_amdgcn_sched_barrier(0);
       cur = nxt;
     }
-
-    // ---- bias, residual, Relu, store (a lane's 32 sums lie a channel plane apart in Y) ----
-    {
-      const int oy = here.oy0 + py, ox = here.ox0 + px;
-      if (oy < p.oh && ox < p.ow) {
-        const int plane = p.oh * p.ow;  // 64 planes stay below 2^31 elements (checked by the host)
-        const long long first = (long long)here.img * COUT * plane + (long long)(4 * half) * plane +
-                                (long long)oy * p.ow + ox;
-        float *y = p.Y + first;
-        const float *res = p.R ? p.R + first : nullptr;
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int off = (32 * mt + 8 * (r >> 2) + (r & 3)) * plane;
-            float v = acc[mt][r];
-            if (p.Bias) v = v + bias[mt][r];
-            if (res) v = v + res[off];
-            if (p.relu) v = relu_js(v);
-            y[off] = v;
-          }
-      }
-    }
+    done.sums[0] = acc[0];
+    done.sums[1] = acc[1];
+    open_pending(done, here, true);
     if (next >= p.ntiles) break;
     stash(buf ^ 1);   // nobody reads that buffer: its tile was finished before the last barrier
     __syncthreads();
@@ -248,15 +279,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParam
     tile = next;
     here = there;
   }
+  // the last tile has no successor to hide behind
+#pragma unroll
+  for (int e = 0; e < 32; e++) finish_element(done, e);
 }
 
 }  // namespace
 
 namespace wdh {
 
-bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group) {
+bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int oh,
+                        int ow) {
+  // (one image's results must fit a buffer descriptor's window: below 2 GiB)
   return group == 1 && c == CIN && cout == COUT && kh == KH && kw == KW && sh == STRIDE && sw == STRIDE &&
-         dh == 1 && dw == 1;
+         dh == 1 && dw == 1 && (long long)COUT * oh * ow * 4 < 0x7fffffffLL;
 }
 
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
@@ -268,8 +304,8 @@ int conv_patch_launch(const float *X, const float *W, const float *Bias, const f
   p.tiles_y = (oh + TH - 1) / TH;
   const long long ntiles = (long long)n * p.tiles_x * p.tiles_y;
   if (ntiles > 0x7fffffffLL) return fail(WDH_EINVAL, "wdh_conv2d: %lld output tiles exceed the grid limit", ntiles);
-  if ((long long)COUT * oh * ow > 0x7fffffffLL)
-    return fail(WDH_EINVAL, "wdh_conv2d: an image's %d x %d x %d results exceed 2^31", COUT, oh, ow);
+  p.fd_per_image = wdh::make_fastdiv((long long)p.tiles_x * p.tiles_y);
+  p.fd_tiles_x = wdh::make_fastdiv(p.tiles_x);
   p.ntiles = (int)ntiles;
   p.relu = relu;
   const long long cap = 2LL * compute_units();  // two workgroups fit a CU (62 KB of LDS each)
