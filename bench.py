@@ -49,7 +49,7 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 # passes included): rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB
 # device copy; recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read
 # counters itself).  The partial sums of tiles cut along K are in it (written once, read once).
-TRAFFIC_BYTES_PER_LAUNCH = 86.1e6  # (86.08 in the latest profile)
+TRAFFIC_BYTES_PER_LAUNCH = 86.8e6  # (86.81 in the latest profile)
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 
