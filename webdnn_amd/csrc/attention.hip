@@ -8,13 +8,13 @@
 // Softmax kernel of this library does), and the second product accumulated in fp32.
 // Only the order of the additions inside the two products and the row sum differs.
 //
-// A workgroup of eight wavefronts owns 32 query rows of one head:
+// A workgroup of eight or sixteen wavefronts owns 32 query rows of one head:
 //   1. scores: each wavefront takes 32-key column blocks in turn
 //      (v_mfma_f32_32x32x2_f32 over the head dimension) and writes alpha * S to LDS,
 //      the whole 32 x keys block (keys <= 1024: 129 KB of the CU's 160 KB);
-//   2. softmax: four rows per wavefront, in place in LDS;
+//   2. softmax: four (two) rows per wavefront, in place in LDS;
 //   3. output: the keys are cut across the wavefronts in blocks of 32, each wavefront
-//      accumulates its share of P V on the matrix cores, and the eight partial 32 x HD
+//      accumulates its share of P V on the matrix cores, and the partial 32 x HD
 //      blocks are added in wavefront order through LDS.
 // Within a block of 32 keys (or of the head dimension) the two halves of a wavefront
 // take the lower and the upper 16 indices, so that a lane reads 16 contiguous floats
@@ -32,7 +32,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int ATT_ROWS = 32;
-constexpr int ATT_WAVES = 8;
 constexpr int ATT_MAX_KEYS = 1024;
 
 struct AttParams {
@@ -45,9 +44,13 @@ struct AttParams {
   float alpha;
 };
 
-template <int HD>
+// ATT_WAVES wavefronts per workgroup: 16 for a head dimension of 32 (every phase is a chain of
+// dependent steps per wavefront; twice the wavefronts halve each chain), 8 where a wavefront's
+// registers hold less of K and V.
+template <int HD, int ATT_WAVES>
 __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParams p) {
   static_assert(HD % 32 == 0 && HD >= 32 && HD <= 128, "head dimension");
+  static_assert(ATT_WAVES == 8 || ATT_WAVES == 16, "32 rows and 32 key blocks are dealt over the wavefronts");
   constexpr int HALF = HD / 2;   // head-dimension indices per half wavefront
   constexpr int NB = HD / 32;    // 32-column blocks of the output
   extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -60,7 +63,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParam
   const float *V = p.V + (long long)b * p.sVb;
   const int ncb = (p.tk + 31) >> 5;  // blocks of 32 keys
 
-  // At most 1024 keys are 32 blocks of 32: four per wavefront.  Each phase issues the loads
+  // At most 1024 keys are 32 blocks of 32: four (two) per wavefront.  Each phase issues the loads
   // of all four before the first use, so a wavefront waits for memory once per phase.
   constexpr int PER_WAVE = ATT_MAX_KEYS / 32 / ATT_WAVES;
 
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParam
   __syncthreads();
 
   // ---- 2. softmax over each row, in place (softmax.ts:34-57) ------------------------
-  // Four rows per wavefront, taken through every step together: their reductions are
+  // The wavefront's four (two) rows are taken through every step together: their reductions are
   // independent, so the cross-lane exchanges of one row hide behind those of the others.
   {
     constexpr int RPW = ATT_ROWS / ATT_WAVES;
@@ -252,13 +255,13 @@ int lds_pitch(int tk) {
   return pitch;
 }
 
-template <int HD>
+template <int HD, int ATT_WAVES>
 int launch_attention(const AttParams &p, int batch) {
-  // the scores block, and later the eight partial outputs, whichever is larger
+  // the scores block, and later the wavefronts' partial outputs, whichever is larger
   size_t bytes = (size_t)ATT_ROWS * p.pitch * 4;
   const size_t partials = (size_t)ATT_WAVES * ATT_ROWS * (HD + 1) * 4;
   if (partials > bytes) bytes = partials;
-  hipLaunchKernelGGL(attention_rows_kernel<HD>, dim3((unsigned)((long long)batch * p.row_blocks)),
+  hipLaunchKernelGGL((attention_rows_kernel<HD, ATT_WAVES>), dim3((unsigned)((long long)batch * p.row_blocks)),
                      dim3(64 * ATT_WAVES), bytes, wdh::stream(), p);
   WDH_LAUNCH_CHECK();
   return WDH_OK;
@@ -271,11 +274,11 @@ namespace wdh {
 // wdh_init with the device current, so that no launch -- captured ones included -- has to).
 int init_attention() {
   const int limit = 160 * 1024;
-  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<32>),
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<32, 16>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, limit));
-  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<64>),
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<64, 8>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, limit));
-  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<128>),
+  WDH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(attention_rows_kernel<128, 8>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, limit));
   return WDH_OK;
 }
@@ -317,7 +320,7 @@ extern "C" int wdh_attention(wdh_buf hQ, wdh_buf hK, wdh_buf hV, wdh_buf hY, int
   p.tq = tq; p.tk = tk; p.pitch = lds_pitch(tk); p.row_blocks = (int)row_blocks;
   p.sQb = sQb; p.sQi = sQi; p.sKb = sKb; p.sKj = sKj; p.sVb = sVb; p.sVj = sVj; p.sYb = sYb; p.sYi = sYi;
   p.alpha = alpha;
-  if (d == 32) return launch_attention<32>(p, batch);
-  if (d == 64) return launch_attention<64>(p, batch);
-  return launch_attention<128>(p, batch);
+  if (d == 32) return launch_attention<32, 16>(p, batch);
+  if (d == 64) return launch_attention<64, 8>(p, batch);
+  return launch_attention<128, 8>(p, batch);
 }
