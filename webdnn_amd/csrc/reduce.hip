@@ -32,20 +32,31 @@ __device__ __forceinline__ double wave_sum_d(double v) {
   return v;
 }
 
-// Register-resident rows.  VEC: rows are 16-byte aligned and a multiple of 4
+// Register-resident rows.  VW = 4: rows are 16-byte aligned and a multiple of 4
 // long, and lane l holds elements 4l..4l+3 of every 256-element segment (one
-// 16-byte access each); otherwise lane l holds elements l, l+64, ...
+// 16-byte access each); VW = 2: the same with 8-byte pieces of every 128-element segment
+// (rows of an even length, 850 say, start on 8-byte boundaries); VW = 1: lane l holds
+// elements l, l+64, ...
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-template <bool VEC>
+template <int VW>
 __device__ __forceinline__ int elem_index(int lane, int i) {
-  return VEC ? lane * 4 + 256 * (i >> 2) + (i & 3) : lane + 64 * i;
+  return VW == 4 ? lane * 4 + 256 * (i >> 2) + (i & 3) : (VW == 2 ? lane * 2 + 128 * (i >> 1) + (i & 1) : lane + 64 * i);
 }
 
-template <int NV, bool VEC>
+template <int NV, int VW>
 __device__ __forceinline__ void load_row(const float *x, int len, int lane, float fill,
                                          float (&v)[NV]) {
-  if constexpr (VEC) {
+  if constexpr (VW == 2) {
+#pragma unroll
+    for (int i = 0; i < NV; i += 2) {
+      const int idx = lane * 2 + 64 * i;
+      f32x2 t = {fill, fill};
+      if (idx < len) t = *reinterpret_cast<const f32x2 *>(x + idx);
+      v[i] = t.x; v[i + 1] = t.y;
+    }
+  } else if constexpr (VW == 4) {
 #pragma unroll
     for (int i = 0; i < NV; i += 4) {
       const int idx = lane * 4 + 64 * i;
@@ -62,9 +73,15 @@ __device__ __forceinline__ void load_row(const float *x, int len, int lane, floa
   }
 }
 
-template <int NV, bool VEC>
+template <int NV, int VW>
 __device__ __forceinline__ void store_row(float *y, int len, int lane, const float (&v)[NV]) {
-  if constexpr (VEC) {
+  if constexpr (VW == 2) {
+#pragma unroll
+    for (int i = 0; i < NV; i += 2) {
+      const int idx = lane * 2 + 64 * i;
+      if (idx < len) *reinterpret_cast<f32x2 *>(y + idx) = f32x2{v[i], v[i + 1]};
+    }
+  } else if constexpr (VW == 4) {
 #pragma unroll
     for (int i = 0; i < NV; i += 4) {
       const int idx = lane * 4 + 64 * i;
@@ -80,14 +97,14 @@ __device__ __forceinline__ void store_row(float *y, int len, int lane, const flo
 }
 
 // ---- softmax ---------------------------------------------------------------
-template <int NV, bool VEC>
+template <int NV, int VW>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_reg(
     const float *__restrict__ X, float *__restrict__ Y, long long outer, int len) {
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
   float v[NV];
-  load_row<NV, VEC>(X + row * len, len, lane, -INFINITY, v);
+  load_row<NV, VW>(X + row * len, len, lane, -INFINITY, v);
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < NV; i++) mx = fmaxf(mx, v[i]);  // fmaxf skips NaN, like `if (v > max)`
@@ -95,7 +112,9 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_reg(
   float sum = 0.0f;
 #pragma unroll
   for (int i = 0; i < NV; i++) {
-    const float e = elem_index<VEC>(lane, i) < len ? exp_f32(v[i] - mx) : 0.0f;
+    // (cells past the row's end hold -inf: e^(-inf - max) is 0 for any finite or +inf max, and a
+    // row whose max is -inf sums to NaN with or without them)
+    const float e = exp_f32(v[i] - mx);
     v[i] = e;
     sum += e;
   }
@@ -104,7 +123,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_reg(
   const float inv = 1.0f / sum;
 #pragma unroll
   for (int i = 0; i < NV; i++) v[i] = v[i] * inv;
-  store_row<NV, VEC>(Y + row * len, len, lane, v);
+  store_row<NV, VW>(Y + row * len, len, lane, v);
 }
 
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void softmax_rows_stream(
@@ -137,9 +156,9 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
   const long long row = (long long)blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   if (row >= outer) return;
   float v[NV], g[NV], bt[NV];
-  load_row<NV, VEC>(X + row * len, len, lane, 0.0f, v);
-  if (G) load_row<NV, VEC>(G, len, lane, 0.0f, g);
-  if (Bt) load_row<NV, VEC>(Bt, len, lane, 0.0f, bt);
+  load_row<NV, VEC ? 4 : 1>(X + row * len, len, lane, 0.0f, v);
+  if (G) load_row<NV, VEC ? 4 : 1>(G, len, lane, 0.0f, g);
+  if (Bt) load_row<NV, VEC ? 4 : 1>(Bt, len, lane, 0.0f, bt);
   double s = 0.0;
 #pragma unroll
   for (int i = 0; i < NV; i++) s += (double)v[i];
@@ -150,7 +169,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
     const float d = v[i] - mean;
     v[i] = d;
     const float sq = d * d;
-    q += elem_index<VEC>(lane, i) < len ? (double)sq : 0.0;
+    q += elem_index<VEC ? 4 : 1>(lane, i) < len ? (double)sq : 0.0;
   }
   const float var = (float)(wave_sum_d(q) / (double)len);
   const float inv = 1.0f / (float)sqrt((double)(var + eps));
@@ -161,13 +180,13 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_reg(
     if (Bt) t = t + bt[i];
     v[i] = t;
   }
-  store_row<NV, VEC>(Y + row * len, len, lane, v);
+  store_row<NV, VEC ? 4 : 1>(Y + row * len, len, lane, v);
   if (P) {  // second output: the normalised row plus a row of P (the Add that follows in the graph)
     float pv[NV];
-    load_row<NV, VEC>(P + row * len, len, lane, 0.0f, pv);
+    load_row<NV, VEC ? 4 : 1>(P + row * len, len, lane, 0.0f, pv);
 #pragma unroll
     for (int i = 0; i < NV; i++) v[i] = v[i] + pv[i];
-    store_row<NV, VEC>(Y2 + row * len, len, lane, v);
+    store_row<NV, VEC ? 4 : 1>(Y2 + row * len, len, lane, v);
   }
 }
 
@@ -379,20 +398,27 @@ extern "C" int wdh_softmax(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   dim3 grid(row_blocks(outer)), block(64 * WAVES_PER_BLOCK);
   hipStream_t st = wdh::stream();
   const bool vec = len % 4 == 0 && (((uintptr_t)px | (uintptr_t)py) & 15) == 0;
+  const bool vec2 = !vec && len % 2 == 0 && (((uintptr_t)px | (uintptr_t)py) & 7) == 0;
   if (len <= 64 * 2)
-    hipLaunchKernelGGL((softmax_rows_reg<2, false>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<2, 1>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 8 && vec)
-    hipLaunchKernelGGL((softmax_rows_reg<8, true>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<8, 4>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 8 && vec2)
+    hipLaunchKernelGGL((softmax_rows_reg<8, 2>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 8)
-    hipLaunchKernelGGL((softmax_rows_reg<8, false>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<8, 1>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 16 && vec)
-    hipLaunchKernelGGL((softmax_rows_reg<16, true>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<16, 4>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 16 && vec2)
+    hipLaunchKernelGGL((softmax_rows_reg<16, 2>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 16)
-    hipLaunchKernelGGL((softmax_rows_reg<16, false>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<16, 1>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 32 && vec)
-    hipLaunchKernelGGL((softmax_rows_reg<32, true>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<32, 4>), grid, block, 0, st, X, Y, outer, len);
+  else if (len <= 64 * 32 && vec2)
+    hipLaunchKernelGGL((softmax_rows_reg<32, 2>), grid, block, 0, st, X, Y, outer, len);
   else if (len <= 64 * 32)
-    hipLaunchKernelGGL((softmax_rows_reg<32, false>), grid, block, 0, st, X, Y, outer, len);
+    hipLaunchKernelGGL((softmax_rows_reg<32, 1>), grid, block, 0, st, X, Y, outer, len);
   else
     hipLaunchKernelGGL(softmax_rows_stream, grid, block, 0, st, X, Y, outer, len);
   WDH_LAUNCH_CHECK();
