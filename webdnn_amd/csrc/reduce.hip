@@ -200,7 +200,8 @@ __device__ __forceinline__ double sub_sum_d(double v) {
   for (int off = SUB / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
   return v;
 }
-template <int SUB>
+// FULL: the rows are exactly 256 long, so no piece and no element needs a range test.
+template <int SUB, bool FULL>
 __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
     const float *__restrict__ X, const float *__restrict__ G,
     const float *__restrict__ Bt, float *__restrict__ Y, long long outer, int len,
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
 #pragma unroll
   for (int j = 0; j < NJ; j++) {
     const int idx = 4 * sub + SEG * j;
-    v[j] = idx < len ? *reinterpret_cast<const f32x4 *>(x + idx) : f32x4{0.f, 0.f, 0.f, 0.f};
+    v[j] = FULL || idx < len ? *reinterpret_cast<const f32x4 *>(x + idx) : f32x4{0.f, 0.f, 0.f, 0.f};
   }
   double s = 0.0;
 #pragma unroll
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
   double q = 0.0;
 #pragma unroll
   for (int j = 0; j < NJ; j++) {
-    const bool in = 4 * sub + SEG * j < len;
+    const bool in = FULL || 4 * sub + SEG * j < len;
 #pragma unroll
     for (int e = 0; e < 4; e++) {
       const float d = v[j][e] - mean;
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(64 * WAVES_PER_BLOCK) void layernorm_rows_part(
 #pragma unroll
   for (int j = 0; j < NJ; j++) {
     const int idx = 4 * sub + SEG * j;
-    if (!(live && idx < len)) continue;
+    if (!(live && (FULL || idx < len))) continue;
     f32x4 t = v[j];
 #pragma unroll
     for (int e = 0; e < 4; e++) t[e] = t[e] * inv;
@@ -452,7 +453,10 @@ int layernorm_launch(const char *who, wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_bu
     // (eight lanes per row measured slower: 12.4 us against 10.0 us on 27200 rows of 256)
     const long long per_block = WAVES_PER_BLOCK * 4;
     const dim3 g((unsigned)((outer + per_block - 1) / per_block));
-    hipLaunchKernelGGL(layernorm_rows_part<16>, g, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
+    if (len == 256)
+      hipLaunchKernelGGL((layernorm_rows_part<16, true>), g, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
+    else
+      hipLaunchKernelGGL((layernorm_rows_part<16, false>), g, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   } else if (len <= 64 * 4 && vec)
     hipLaunchKernelGGL((layernorm_rows_reg<4, true>), grid, block, 0, st, X, G, B, Y, outer, len, eps, P, Y2);
   else if (len <= 64 * 4)
