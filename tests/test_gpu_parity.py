@@ -1036,6 +1036,21 @@ def test_conv7x7_stem_kernel(ctx, shape):
     assert_close_max(got[1], got[0], 1e-5, "stem kernel vs gathered form")
 
 
+def test_conv7x7_stem_geometry_without_descriptors_takes_the_flat_gather(ctx):
+    """descriptor_loads = 0 stands for operands of 2 GiB and more: the stem's kernel addresses a whole
+    image's results through one descriptor, so it must step aside."""
+    X, W, B = uni(2, 3, 40, 56, lo=-1), he(64, 3, 7), nrm(64)
+    want = ref.conv(X, W, B, None, 1, None, [3, 3, 3, 3], [2, 2])
+    try:
+        ctx.set_option("descriptor_loads", 0)
+        got = hip_conv(ctx, X, W, B, None, 1, [3, 3, 3, 3], [2, 2])
+        form = ctx.last_plan()["form"]
+    finally:
+        ctx.set_option("descriptor_loads", 1)
+    assert form == "conv, gathered taps (flat loads)", form
+    assert_close_max(got, want, GEMM_TOL, "stem geometry, flat loads")
+
+
 def test_conv7x7_stem_kernel_keeps_nan_and_inf_inside_their_receptive_fields(ctx):
     """One step of the stem kernel's K order has no partner tap: what the idle half of the wavefront
     multiplies must be a true zero, or an Inf elsewhere in the tile's patch would leak into every pixel."""

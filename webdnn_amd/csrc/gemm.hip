@@ -2031,7 +2031,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.fd_ohw = make_fastdiv((long long)oh * ow);
   p.cv.fd_plane = make_fastdiv((long long)h * w);
 
-  if (g_stem && wdh::conv_patch_applies(c, cout, kh, kw, sh, sw, dh, dw, group, oh, ow)) {
+  if (g_stem && g_descriptors && wdh::conv_patch_applies(c, cout, kh, kw, sh, sw, dh, dw, group, oh, ow)) {
     const long long tiles = (long long)n * ((oh + 7) / 8) * ((ow + 15) / 16);
     g_last_plan = {64, 128, 1, WDH_FORM_CONV_STEM, tiles, 0};
     return wdh::conv_patch_launch(p.B, p.A, p.C, p.R, p.Y, n, h, w, oh, ow, pt, pl, epilogue == WDH_EPI_RELU);
