@@ -124,8 +124,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParam
   __syncthreads();
 
   // ---- 2. softmax over each row, in place (softmax.ts:34-57) ------------------------
-  // The wavefront's four (two) rows are taken through every step together: their reductions are
-  // independent, so the cross-lane exchanges of one row hide behind those of the others.
+  // The wavefront's four (two) rows are taken through every step together.
   {
     constexpr int RPW = ATT_ROWS / ATT_WAVES;
     const int ncols = ncb * 32;  // a multiple of 4; at most 1024: four 16-byte pieces per lane
@@ -145,9 +144,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParam
       }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-#pragma unroll
-      for (int j = 0; j < RPW; j++) mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], off, 64));
+    for (int j = 0; j < RPW; j++) mx[j] = wave_max(mx[j]);
 #pragma unroll
     for (int j = 0; j < RPW; j++) {
       sum[j] = 0.0f;
@@ -161,9 +158,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void attention_rows_kernel(AttParam
         }
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1)
-#pragma unroll
-      for (int j = 0; j < RPW; j++) sum[j] += __shfl_xor(sum[j], off, 64);
+    for (int j = 0; j < RPW; j++) sum[j] = wave_sum(sum[j]);
 #pragma unroll
     for (int j = 0; j < RPW; j++) {
       float *srow = lds + (wave + ATT_WAVES * j) * p.pitch;
