@@ -13,7 +13,8 @@
 //
 // One wavefront owns one row: lanes read consecutive floats (256-byte
 // coalesced requests), keep the row in registers when it fits (len <= 64*NV),
-// and reduce with cross-lane shuffles; no LDS, no barriers.  Rows longer than
+// and reduce across lanes (single-precision values through DPP operands, double-precision
+// sums through lane shuffles); no LDS tile, no barriers.  Rows longer than
 // the register budget are re-read from cache in further passes.
 #include <math.h>
 
