@@ -265,10 +265,11 @@ def bench_kernels(steps, warmup, calibrate_copy=False):
     }
 
 
-def bench_resnet_layers(steps, warmup, batch=32):
+def bench_resnet_layers(steps, warmup, batch=32, only=None):
     """Every distinct Conv / Gemm launch of the ResNet-50 step, through the C ABI with back-to-back
     launches (operands hot in the caches, unlike inside the graph): shape, how often the step runs
-    it, microseconds, TFLOP/s, and how the launch was laid out (tile, whole / K-split tiles, form)."""
+    it, microseconds, TFLOP/s, and how the launch was laid out (tile, whole / K-split tiles, form).
+    `only`: run just the layers whose label contains this text (one layer under a profiler)."""
     from webdnn_amd import hostops as H
     from webdnn_amd import modelgen
 
@@ -313,6 +314,13 @@ def bench_resnet_layers(steps, warmup, batch=32):
     rows = []
     for (x, w, pads, strides, residual), info in layers.items():
         if info["kind"] == "Conv":
+            label = "Conv %dx%d s%d %d->%d @%dx%d%s" % (w[2], w[3], strides[0], x[1], w[0], x[2], x[3],
+                                                         " +residual" if residual else "")
+        else:
+            label = "Gemm [%d,%d] x [%d,%d]^T" % (x[0], x[1], w[0], w[1])
+        if only and only not in label:
+            continue
+        if info["kind"] == "Conv":
             X = ctx.move_tensor(rng.uniform(0, 1, x).astype(np.float32))
             W = ctx.move_tensor((rng.standard_normal(w) * np.sqrt(2.0 / (w[1] * w[2] * w[3]))).astype(np.float32))
             B = ctx.move_tensor(np.zeros(w[0], np.float32))
@@ -325,8 +333,6 @@ def bench_resnet_layers(steps, warmup, batch=32):
             m, n, k = w[0], odims[0] * odims[2] * odims[3], w[1] * w[2] * w[3]
             out_elems = int(np.prod(odims))
             nbytes = 4 * (int(np.prod(x)) + int(np.prod(w)) + w[0] + out_elems * (2 if residual else 1))
-            label = "Conv %dx%d s%d %d->%d @%dx%d%s" % (w[2], w[3], strides[0], x[1], w[0], x[2], x[3],
-                                                         " +residual" if residual else "")
             for t in (X, W, B) + ((R,) if R is not None else ()):
                 t.dispose()
         else:
@@ -338,7 +344,6 @@ def bench_resnet_layers(steps, warmup, batch=32):
             ms = timed_steps(ctx, lambda: H.gemm(ctx, A, Wt, Bv, trans_b=1).dispose(), steps, warmup)
             m, n, k = x[0], w[0], x[1]
             nbytes = 4 * (x[0] * x[1] + w[0] * w[1] + w[0] + x[0] * w[0])
-            label = "Gemm [%d,%d] x [%d,%d]^T" % (x[0], x[1], w[0], w[1])
             for t in (A, Wt, Bv):
                 t.dispose()
         flops = 2.0 * m * n * k
@@ -419,6 +424,9 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--layer", default=None,
+                    help="with --only layers: run just the layers whose label contains this text, e.g. "
+                         "'1x1 s1 256->1024' (for per-layer profiler runs)")
     ap.add_argument("--only", choices=["all", "kernels", "bandwidth", "layers"], default="all",
                     help="kernels: only the in-process Gemm 4096 / Conv C3 launches plus one device-to-device "
                          "copy of known size (the unit for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -432,7 +440,7 @@ def main():
                           "unit": "GB/s of algorithmic bytes", "peak": 8000.0}))
         return
     if args.only == "layers":
-        print(json.dumps({"resnet50_layers": bench_resnet_layers(args.steps, args.warmup)}))
+        print(json.dumps({"resnet50_layers": bench_resnet_layers(args.steps, args.warmup, only=args.layer)}))
         return
     if args.only == "kernels":
         print(json.dumps({"kernels": bench_kernels(args.steps, args.warmup, calibrate_copy=True)}))

@@ -89,8 +89,8 @@ __host__ __device__ constexpr int step_offset(int t) {
 }
 
 __device__ __forceinline__ float relu_js(float v) {
-  // Math.max(v, 0): NaN stays NaN, -0 becomes +0.
-  return v > 0.0f ? v : (v != v ? v : 0.0f);
+  // Math.max(v, 0): NaN stays NaN (the comparison is false for it), -0 becomes +0.
+  return v <= 0.0f ? 0.0f : v;
 }
 
 __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParams p) {

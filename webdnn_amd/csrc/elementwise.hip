@@ -317,8 +317,8 @@ int launch_binary(const BinaryParams &p, int dtype, bool dense, bool vec) {
 // ---- unary ---------------------------------------------------------------
 
 __device__ __forceinline__ float relu_js(float v) {
-  // Math.max(v, 0): NaN stays NaN, -0 becomes +0.
-  return v > 0.0f ? v : (v != v ? v : 0.0f);
+  // Math.max(v, 0): NaN stays NaN (the comparison is false for it), -0 becomes +0.
+  return v <= 0.0f ? 0.0f : v;
 }
 
 template <int OP>

@@ -203,8 +203,8 @@ struct Params {
 };
 
 __device__ __forceinline__ float relu_js(float v) {
-  // Math.max(v, 0): NaN stays NaN, -0 becomes +0.
-  return v > 0.0f ? v : (v != v ? v : 0.0f);
+  // Math.max(v, 0): NaN stays NaN (the comparison is false for it), -0 becomes +0.
+  return v <= 0.0f ? 0.0f : v;
 }
 
 // Whole-tile workgroups: ids are dealt round-robin over the 8 XCDs by the
@@ -457,13 +457,13 @@ __device__ __forceinline__ void reduce_quad(const Params &p, int bm, int bn, int
   for (int i = 0; i < 4; i++) {
     const int col = tn * bn + lc + i;
     if (col >= p.n) break;
-    float y = p.alpha * acc[i];
+    float y = CONV ? acc[i] : p.alpha * acc[i];  // (a conv has alpha = beta = 1: the same bits, fewer instructions)
     long long off;
     if (CONV) {
       const int ohw = p.cv.oh * p.cv.ow;
       const int img = fdiv(col, p.cv.fd_ohw), q = col - img * ohw;
       off = ((long long)img * p.cv.cout_total + (long long)bz * p.cv.cout_g + row) * ohw + q;
-      if (p.C) y = __builtin_fmaf(p.C[bz * p.cv.cout_g + row], p.beta, y);
+      if (p.C) y = y + p.C[bz * p.cv.cout_g + row];
     } else {
       off = (long long)bz * p.sYb + (long long)row * p.sY0 + col;
       if (p.C) y = __builtin_fmaf(p.C[(long long)row * p.sC0 + (long long)col * p.sC1], p.beta, y);
@@ -583,8 +583,14 @@ __device__ __forceinline__ void finish_tile(const Params &p,
           f32x4 y;
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            float t = p.alpha * v[e];
-            if (p.C) t = __builtin_fmaf(cv[slot][e], p.beta, t);
+            float t;
+            if constexpr (CONV) {  // alpha = beta = 1: the same bits, two instructions fewer per element
+              t = v[e];
+              if (p.C) t = t + cv[slot][e];
+            } else {
+              t = p.alpha * v[e];
+              if (p.C) t = __builtin_fmaf(cv[slot][e], p.beta, t);
+            }
             if (p.R) t = t + rv[slot][e];
             if (p.epilogue == WDH_EPI_RELU) t = relu_js(t);
             y[e] = t;
@@ -646,8 +652,14 @@ __device__ __forceinline__ void finish_tile(const Params &p,
           }
 #pragma unroll
           for (int j = 0; j < 8; j++) {
-            float y = p.alpha * acc[mt][nt][8 * hb + j];
-            if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+            float y;
+            if constexpr (CONV) {
+              y = acc[mt][nt][8 * hb + j];
+              if (p.C) y = y + cv[j];
+            } else {
+              y = p.alpha * acc[mt][nt][8 * hb + j];
+              if (p.C) y = __builtin_fmaf(cv[j], p.beta, y);
+            }
             if (p.R) y = y + rv[j];
             if (p.epilogue == WDH_EPI_RELU) y = relu_js(y);
             buf_store(rsrc_y, y, voff_y, (rbase + 16 * hb + 8 * (j >> 2) + (j & 3)) * ystride * 4);
