@@ -29,10 +29,25 @@ def gemm_both(ctx, A, B, C, R, alpha, beta, epi):
                       0, 1, alpha, beta, epi, tr.handle)
     capi.call("wdh_gemm", *args(y0))
     ctx.sync()
+    # wdh_gemm left its partial-sum block in the pool's cache; with the cache emptied, a static call
+    # that took a block from the pool and gave it back would show up as cached bytes (or a new peak)
+    capi.call("wdh_trim", 0)
     before = mem_stats()
+    assert before[1] == 0, before
     capi.call("wdh_gemm_static", *args(y1))
     after = mem_stats()
     assert after == before, "the call took memory from the pool or the driver: %s -> %s" % (before, after)
+    # the callers it is for: a stream in capture mode (an allocation would fail the capture)
+    ctx.sync()
+    ctx.graph_begin()
+    try:
+        capi.call("wdh_gemm_static", *args(y1))
+    finally:
+        gid = ctx.graph_end()
+    assert mem_stats() == before
+    ctx.graph_launch(gid)
+    ctx.sync()
+    ctx.graph_destroy(gid)
     out = y0.get_data(), y1.get_data()
     for t in (ta, tb, tc, tr, y0, y1):
         t.dispose()

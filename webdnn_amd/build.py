@@ -41,20 +41,28 @@ def _run(cmd):
         print(out)
 
 
-def build_library(verbose=True):
+def build_library(verbose=True, only=None):
+    """Compiles the HIP sources (side by side, one hipcc each) and links them.  `only`: recompile
+    just these sources and reuse the other objects if they are still there (kernel work)."""
+    from concurrent.futures import ThreadPoolExecutor
+
     os.makedirs(LIBDIR, exist_ok=True)
-    objs = []
-    for src in HIP_SOURCES:
-        obj = os.path.join(LIBDIR, src.replace(".hip", ".o"))
-        cmd = ["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-               "-c", os.path.join(CSRC, src), "-o", obj]
+    objdir = os.path.join(LIBDIR, "obj")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        if only is not None and src not in only and os.path.exists(obj):
+            return obj
         if verbose:
             print("[build] hipcc", src)
-        _run(cmd)
-        objs.append(obj)
+        _run(["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+              "-c", os.path.join(CSRC, src), "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
-    for obj in objs:
-        os.remove(obj)
     return LIB
 
 
@@ -77,6 +85,10 @@ def build_all(verbose=True):
 
 
 if __name__ == "__main__":
-    build_all()
+    if len(sys.argv) > 1:      # python -m webdnn_amd.build gemm.hip ...: recompile these, relink
+        build_library(only=sys.argv[1:])
+        build_addon()
+    else:
+        build_all()
     print("built", LIB)
     sys.exit(0)

@@ -24,6 +24,9 @@ int device();           // the device wdh_init selected
 int init_static_scratch(int device);
 // Raises the dynamic LDS limit of the attention kernels on the current device (called by wdh_init).
 int init_attention();
+// Device resources of the contraction kernels that outlive a call (called by wdh_init / at shutdown).
+int init_contraction();
+void release_contraction();
 
 // Handle -> device pointer.  Returns nullptr (and records WDH_EINVAL) for an
 // unknown handle.  A zero-byte buffer resolves to a non-null dummy pointer.
@@ -34,8 +37,8 @@ void *resolve(wdh_buf h, size_t *bytes);
 bool operand(wdh_buf h, size_t need, const char *what, void **out);
 
 // The stem convolution's own kernel (conv_patch.hip): whether a geometry qualifies, and the launch.
-bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int oh,
-                        int ow);
+bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int h, int w,
+                        int pt, int pl, int oh, int ow);
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
                       int h, int w, int oh, int ow, int pt, int pl, int relu);
 

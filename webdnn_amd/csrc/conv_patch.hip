@@ -288,11 +288,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void conv7x7s2_patch_kernel(PatchParam
 
 namespace wdh {
 
-bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int oh,
-                        int ow) {
-  // (one image's results must fit a buffer descriptor's window: below 2 GiB)
+bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh, int dw, int group, int h, int w,
+                        int pt, int pl, int oh, int ow) {
+  // One image's results must fit a buffer descriptor's window (below 2 GiB), and the kernel
+  // indexes an image's input with 32-bit element offsets ((c * h + iy) * w + ix, shifted up by
+  // the padding): larger images are left to the gathered form and its 64-bit path.
   return group == 1 && c == CIN && cout == COUT && kh == KH && kw == KW && sh == STRIDE && sw == STRIDE &&
-         dh == 1 && dw == 1 && (long long)COUT * oh * ow * 4 < 0x7fffffffLL;
+         dh == 1 && dw == 1 && (long long)COUT * oh * ow * 4 < 0x7fffffffLL &&
+         (long long)CIN * h * w + (long long)pt * w + pl < 0x7fffffffLL / 4;
 }
 
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,

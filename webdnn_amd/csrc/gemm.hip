@@ -122,8 +122,13 @@ __device__ __forceinline__ void buf_store(rsrc_t r, float v, int voff, int soff)
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
 }
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void buf_store4(rsrc_t r, f32x4 v, int voff, int soff) {
-  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
+// No scalar-offset parameter on purpose: a buffer_store_dwordx4 whose scalar offset is a
+// register gets no wait states from the compiler before its data registers are written again,
+// and the chip then now and then stores the new values (seen in about one quad in a thousand).
+// Every term of the address goes into `voff`.  test_sixteen_byte_stores_hold_the_bits_of_four_byte_stores (tests/test_gpu_parity.py)
+// compares these stores with the 4-byte ones on every tile and must pass after a toolchain change.
+__device__ __forceinline__ void buf_store4(rsrc_t r, f32x4 v, int voff) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, 0, 0);
 }
 
 constexpr int BK = 16;
@@ -598,7 +603,7 @@ __device__ __forceinline__ void finish_tile(const Params &p,
           // (row offset in the vector register: a 16-byte store whose scalar offset is a
           // register gets no wait states from the compiler before its data registers are
           // written again, and this chip then now and then stores the new value)
-          buf_store4(rsrc_y, y, voff_y + (rbase + 8 * i) * ystride * 4, 0);
+          buf_store4(rsrc_y, y, voff_y + (rbase + 8 * i) * ystride * 4);
         }
       }
     }
@@ -1984,6 +1989,8 @@ void release_conv_tables() {
   }
   g_ktabs.clear();
 }
+int init_contraction() { return WDH_OK; }
+void release_contraction() {}
 }  // namespace wdh
 
 extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
@@ -2043,7 +2050,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   p.cv.fd_ohw = make_fastdiv((long long)oh * ow);
   p.cv.fd_plane = make_fastdiv((long long)h * w);
 
-  if (g_stem && g_descriptors && wdh::conv_patch_applies(c, cout, kh, kw, sh, sw, dh, dw, group, oh, ow)) {
+  if (g_stem && g_descriptors && wdh::conv_patch_applies(c, cout, kh, kw, sh, sw, dh, dw, group, h, w, pt, pl, oh, ow)) {
     const long long tiles = (long long)n * ((oh + 7) / 8) * ((ow + 15) / 16);
     g_last_plan = {64, 128, 1, WDH_FORM_CONV_STEM, tiles, 0};
     return wdh::conv_patch_launch(p.B, p.A, p.C, p.R, p.Y, n, h, w, oh, ow, pt, pl, epilogue == WDH_EPI_RELU);

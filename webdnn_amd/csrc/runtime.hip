@@ -11,6 +11,8 @@
 #include <string.h>
 
 #include <map>
+#include <string>
+#include <utility>
 #include <vector>
 
 #include "common.h"
@@ -158,12 +160,32 @@ extern "C" {
 
 const char *wdh_last_error(void) { return g_error; }
 
-int wdh_init(int device) {
-  if (g.ready) {
-    if (device == g.device) return WDH_OK;
-    return fail(WDH_EINVAL, "wdh_init: already initialised on device %d",
-                g.device);
+// WDH_OPTIONS="name=value,name=value": wdh_set_option calls made on behalf of a caller that
+// cannot make them itself (a model run through an unmodified host).  The whole string is
+// checked before anything is applied or any device resource exists, so a bad item leaves the
+// library uninitialised instead of half configured.
+static int parse_env_options(std::vector<std::pair<std::string, int>> *out) {
+  const char *env = getenv("WDH_OPTIONS");
+  if (!env) return WDH_OK;
+  if (strlen(env) > 511) return fail(WDH_EINVAL, "WDH_OPTIONS: longer than 511 characters");
+  char buf[512];
+  snprintf(buf, sizeof(buf), "%s", env);
+  for (char *item = strtok(buf, ","); item; item = strtok(nullptr, ",")) {
+    char *eq = strchr(item, '=');
+    if (!eq || eq == item) return fail(WDH_EINVAL, "WDH_OPTIONS: \"%s\" is not name=value", item);
+    *eq = '\0';
+    char *end = nullptr;
+    const long v = strtol(eq + 1, &end, 10);
+    if (end == eq + 1 || *end != '\0' || v < -0x7fffffffL || v > 0x7fffffffL)
+      return fail(WDH_EINVAL, "WDH_OPTIONS: value of \"%s\" is not an integer", item);
+    out->emplace_back(item, (int)v);
   }
+  return WDH_OK;
+}
+
+static void release_everything();
+
+static int init_device(int device) {
   int count = 0;
   hipError_t e = hipGetDeviceCount(&count);
   if (e != hipSuccess || count <= 0) {
@@ -190,43 +212,54 @@ int wdh_init(int device) {
     g.stage_busy[i] = false;
   }
   WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
-  {
-    int rc = wdh::init_static_scratch(device);
-    if (rc == WDH_OK) rc = wdh::init_attention();
-    if (rc != WDH_OK) return rc;
+  int rc = wdh::init_static_scratch(device);
+  if (rc == WDH_OK) rc = wdh::init_attention();
+  if (rc == WDH_OK) rc = wdh::init_contraction();
+  return rc;
+}
+
+int wdh_init(int device) {
+  if (g.ready) {
+    if (device == g.device) return WDH_OK;
+    return fail(WDH_EINVAL, "wdh_init: already initialised on device %d",
+                g.device);
+  }
+  // Options first: wdh_set_option checks names and ranges and touches plain variables only, so a
+  // bad WDH_OPTIONS fails here, before any device resource exists.
+  std::vector<std::pair<std::string, int>> options;
+  if (int rc = parse_env_options(&options)) return rc;
+  for (auto &kv : options)
+    if (int rc = wdh_set_option(kv.first.c_str(), kv.second)) return rc;
+  if (int rc = init_device(device)) {
+    release_everything();  // whatever was created before the failing step (the error text stays)
+    return rc;
   }
   g.device = device;
   g.ready = true;
-  // WDH_OPTIONS="name=value,name=value": wdh_set_option calls made on behalf of a caller that
-  // cannot make them itself (a model run through an unmodified host); unknown names are errors
-  if (const char *env = getenv("WDH_OPTIONS")) {
-    char buf[512];
-    snprintf(buf, sizeof(buf), "%s", env);
-    for (char *item = strtok(buf, ","); item; item = strtok(nullptr, ",")) {
-      char *eq = strchr(item, '=');
-      if (!eq) return fail(WDH_EINVAL, "WDH_OPTIONS: \"%s\" is not name=value", item);
-      *eq = '\0';
-      const int rc = wdh_set_option(item, atoi(eq + 1));
-      if (rc != WDH_OK) return rc;
-    }
-  }
   wdh::clear_error();
   return WDH_OK;
 }
 
 void wdh_shutdown(void) {
   if (!g.ready) return;
+  release_everything();
+}
+
+// Releases whatever exists (also after a wdh_init that failed half way): every step copes with
+// its resource missing.
+static void release_everything() {
   if (g.capturing) {
     hipGraph_t dropped = nullptr;
     (void)hipStreamEndCapture(g.stream, &dropped);
     if (dropped) (void)hipGraphDestroy(dropped);
     g.capturing = 0;
   }
-  (void)hipStreamSynchronize(g.stream);
+  if (g.stream) (void)hipStreamSynchronize(g.stream);
   for (size_t i = 0; i < g.graphs.size(); i++)
     if (g.graphs[i].live) dissolve_graph((int)i);
   g.graphs.clear();
   wdh::release_conv_tables();
+  wdh::release_contraction();
   for (auto &s : g.slots)
     if (s.ptr && s.ptr != g.dummy) (void)hipFree(s.ptr);
   g.slots.clear();
@@ -246,7 +279,7 @@ void wdh_shutdown(void) {
   }
   if (g.dummy) (void)hipFree(g.dummy);
   g.dummy = nullptr;
-  (void)hipStreamDestroy(g.stream);
+  if (g.stream) (void)hipStreamDestroy(g.stream);
   g.stream = nullptr;
   g.ready = false;
   g.device = -1;
