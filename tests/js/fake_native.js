@@ -390,6 +390,7 @@ native.free = function (h) {
   return undefined;
 };
 native.graphBegin = function () {
+  count("graphBegin");
   if (capture) throw new Error("wdh_graph_begin failed (-5): a capture is already open");
   capture = { ops: [], freed: [], failed: false };
 };

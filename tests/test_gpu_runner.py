@@ -178,14 +178,14 @@ def test_optimized_model_directory(tmp_path):
     assert_close_max(got8[0], ref8[out_name], 1e-3, "8-bit coded weights")
 
 
-def _graph_runs(tmp_path, data, a, b, runs, resident=False):
+def _graph_runs(tmp_path, data, a, b, runs, resident=False, flags=("--graph",)):
     alt = []
     for i, arr in enumerate(b):
         p = tmp_path / ("alt_%d.bin" % i)
         np.ascontiguousarray(arr).tofile(str(p))
         alt.append(str(p))
     return node_runner.run_model(str(tmp_path), a, "hip", strict=True, runs=runs,
-                                 extra=["--graph", "--alt-inputs", ",".join(alt)] + (["--resident-inputs"] if resident else []))
+                                 extra=list(flags) + ["--alt-inputs", ",".join(alt)] + (["--resident-inputs"] if resident else []))
 
 
 def test_graph_replay_equals_eager_runs(tmp_path):
@@ -203,6 +203,22 @@ def test_graph_replay_equals_eager_runs(tmp_path):
         assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
         assert rep["stats"]["graphReplay"] is True
         assert_bit_exact(got[0], want[0], "run %d of a graph-mode session" % runs)
+
+
+def test_runs_without_an_option_are_replayed_from_the_third_on(tmp_path):
+    """runner.run([CPUTensor]) with no option (graph "auto"): two eager runs, the third recorded, the rest
+    replayed; each compared run equals the eager run of the input it was given, bit for bit."""
+    data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    ea, _ = node_runner.run_model(str(tmp_path), [Xa], "hip", strict=True, extra=["--no-graph"])
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True, extra=["--no-graph"])
+    for runs, want, captured in ((2, eb, False), (3, ea, True), (4, eb, True), (7, ea, True)):
+        got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs, flags=())
+        assert rep["graph"]["captured"] is captured and rep["graph"]["unsupported"] is None, rep["graph"]
+        assert rep["stats"].get("graphReplay", False) is captured
+        assert_bit_exact(got[0], want[0], "run %d of a session without options" % runs)
 
 
 def test_graph_replay_with_two_resident_device_inputs(tmp_path):

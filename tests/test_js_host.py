@@ -59,7 +59,7 @@ def test_operator_instances_are_reused_across_runs(tmp_path):
     created = []
     outs = []
     for runs in (1, 2, 3, 4):
-        out, rep = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=runs)
+        out, rep = node_runner.run_model(str(tmp_path), [X], "hip", fake_native=True, runs=runs, extra=["--no-graph"])
         created.append(rep["stats"]["operatorsCreated"])
         outs.append(out[0])
         nodes = rep["stats"]["nodes"]
@@ -229,6 +229,36 @@ def test_attention_chain_becomes_one_node(tmp_path, hd, one_launch):
     np.testing.assert_allclose(outs[0], plain[0], rtol=0, atol=1e-6)
 
 
+def test_fused_matmul_keeps_the_broadcasting_of_the_nodes_it_absorbed(tmp_path):
+    """Two shapes where the absorbed Mul / Add broadcast differently from the kernel's alpha and C term:
+    a one-element constant of rank 4 (the Mul raises the result's rank: not absorbed) and a matrix-vector
+    product, whose result [m] gets a bias [m] (absorbed; the node then runs the Add separately).  The fused
+    graph gives the unfused graph's bits and shapes."""
+    g = modelgen.GraphBuilder(8)
+    m, k = 6, 10
+    rng = g.rng()
+    g.const("v", rng.standard_normal((k,)).astype(np.float32))
+    g.const("bm", rng.standard_normal((m,)).astype(np.float32))
+    g.const("W", rng.standard_normal((k, k)).astype(np.float32))
+    g.const("s4", np.full((1, 1, 1, 1), 0.5, np.float32))
+    g.const("s1", np.full((1,), 0.25, np.float32))
+    g.op("Relu", [g.op("Add", [g.op("MatMul", ["X", "v"], "xv"), "bm"], "xvb")], "Y1")      # [m,k] x [k] -> [m], + [m]
+    g.op("Mul", [g.op("MatMul", ["X", "W"], "xw"), "s4"], "Y2")                              # -> [1,1,m,k]
+    g.op("Mul", [g.op("MatMul", ["X", "W"], "xw2"), "s1"], "Y3")                             # -> [m,k], absorbed
+    data = g.finish([("X", [m, k])], [("Y1", [m]), ("Y2", [1, 1, m, k]), ("Y3", [m, k])], opset=13)
+    (tmp_path / "model.onnx").write_bytes(data)
+    X = np.random.default_rng(9).standard_normal((m, k)).astype(np.float32)
+    outs, rep = node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fake_native=True)
+    plain, rep_p = node_runner.run_model(str(tmp_path), [X], "hip", strict=True, fuse=False, fake_native=True)
+    assert rep["nodes"] < rep_p["nodes"]
+    for a, b, shape in zip(outs, plain, ((m,), (1, 1, m, k), (m, k))):
+        assert a.shape == b.shape == shape, (a.shape, b.shape)
+        assert_bit_exact(a, b, "fused vs unfused %s" % (shape,))
+    want = graph_ref.run_graph(modelgen.parse_model(data), {"X": X})
+    for got, name in zip(outs, ("Y1", "Y2", "Y3")):
+        np.testing.assert_allclose(got, want[name], rtol=0, atol=1e-5)
+
+
 def test_neighbouring_linear_layers_run_as_one_group(tmp_path):
     """Projections of one input and rank-3 MatMuls next to rank-2 ones:
     grouped into one node; the rank-2 ones take one native call, a group with the rank-3 product in it
@@ -332,9 +362,11 @@ def test_export_style_glue_graph(tmp_path, opset):
     assert rep["liveBuffers"] == rep["initializerCopies"]
 
 
-def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native):
+def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native, flags=("--graph",), runs=(3, 4)):
     """Runs 1..4 with {graph: true}: eager warm-up, capture + launch, replay, replay; even runs use
-    feeds_a, odd runs feeds_b.  Returns (outputs of run 3 (a), outputs of run 4 (b), eager a, eager b, report)."""
+    feeds_a, odd runs feeds_b.  Returns (outputs of run 3 (a), outputs of run 4 (b), eager a, eager b, report).
+    `flags`: what the CLI passes on to runner.run (nothing = the runner's default); `runs`: an odd and an
+    even session length to compare instead of 3 and 4."""
     (tmp_path / "model.onnx").write_bytes(data)
     model = modelgen.parse_model(data)
     a = [feeds_a[n] for n, _ in model["inputs"]]
@@ -347,8 +379,9 @@ def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native):
     kw = dict(strict=True, fake_native=fake_native)
     eager_a, _ = node_runner.run_model(str(tmp_path), a, "hip", **kw)
     eager_b, _ = node_runner.run_model(str(tmp_path), b, "hip", **kw)
-    g3, rep3 = node_runner.run_model(str(tmp_path), a, "hip", runs=3, extra=["--graph", "--alt-inputs", ",".join(alt)], **kw)
-    g4, rep4 = node_runner.run_model(str(tmp_path), a, "hip", runs=4, extra=["--graph", "--alt-inputs", ",".join(alt)], **kw)
+    extra = list(flags) + ["--alt-inputs", ",".join(alt)]
+    g3, rep3 = node_runner.run_model(str(tmp_path), a, "hip", runs=runs[0], extra=extra, **kw)
+    g4, rep4 = node_runner.run_model(str(tmp_path), a, "hip", runs=runs[1], extra=extra, **kw)
     return g3, g4, eager_a, eager_b, rep4
 
 
@@ -363,6 +396,26 @@ def test_graph_replay_on_the_host_path(tmp_path):
     assert_bit_exact(g4[0], eb[0], "fourth run (replay, second input)")
     assert rep["nativeCalls"]["graphLaunch"] == 3
     assert rep["liveBuffers"] == rep["initializerCopies"]          # the graph's buffers are gone after disposeGraph
+
+
+def test_a_caller_that_passes_no_option_gets_the_graph_after_two_runs(tmp_path):
+    """runner.run(inputs) as the reference's callers write it: runs 1 and 2 walk the node loop, run 3 is
+    recorded and launched, later runs replay -- with the bits of the eager runs of the same inputs.  Two
+    runs never record anything; {graph: false} keeps every run in the node loop."""
+    data, _ = modelgen.resnet50_model(batch=2, image=32, width=8, blocks=(1, 1, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    g5, g6, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"input": Xa}, {"input": Xb}, True, flags=(), runs=(5, 6))
+    assert rep["graph"] == {"captured": True, "unsupported": None}
+    assert rep["stats"]["graphReplay"] is True
+    assert_bit_exact(g5[0], ea[0], "fifth run (replay, first input)")
+    assert_bit_exact(g6[0], eb[0], "sixth run (replay, second input)")
+    assert rep["nativeCalls"]["graphLaunch"] == 4 and rep["nativeCalls"]["graphBegin"] == 1
+    assert rep["liveBuffers"] == rep["initializerCopies"]
+    _, rep2 = node_runner.run_model(str(tmp_path), [Xa], "hip", runs=2, fake_native=True)
+    assert rep2["graph"]["captured"] is False and "graphBegin" not in rep2["nativeCalls"]
+    _, rep_off = node_runner.run_model(str(tmp_path), [Xa], "hip", runs=5, fake_native=True, extra=["--no-graph"])
+    assert "graphBegin" not in rep_off["nativeCalls"] and "graphReplay" not in rep_off["stats"]
 
 
 def test_exporter_shaped_model_bytes_decode_and_run(tmp_path):

@@ -6,7 +6,7 @@
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
-//        [--graph] [--alt-inputs a2.bin[,b2.bin...]]
+//        [--graph | --no-graph] [--alt-inputs a2.bin[,b2.bin...]]
 //
 // Inputs are raw little-endian files (float32, or int32 where the graph input says
 // so) in the order of the graph's non-initializer inputs; outputs are written the same
@@ -17,7 +17,10 @@
 // reference operators that way, the product itself ships hot-path operators for hip only.
 //
 // --graph passes {graph: true} to runner.run: the second call records the run into a HIP graph,
-// later calls replay it.  --alt-inputs names a second set of input files used by every other
+// later calls replay it.  --no-graph passes {graph: false}: every run walks the node loop.  With
+// neither, runner.run gets no option, as from a caller written for the reference: the runner's
+// default ("auto") records the third run with inputs of one signature and replays it afterwards.
+// --alt-inputs names a second set of input files used by every other
 // run (odd run numbers), so that replays see changing data.
 //
 // Methodology follows the reference's harness (example/benchmark/runner/bench.js:130-167):
@@ -39,6 +42,7 @@ function parseArgs(argv) {
     else if (a === "--onnx") args.onnx = next();
     else if (a === "--optimized") args.optimized = true;
     else if (a === "--graph") args.graph = true;
+    else if (a === "--no-graph") args.graph = false;
     else if (a === "--alt-inputs") args.altInputs = next().split(",");
     else if (a === "--backend") args.backend = next();
     else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
@@ -109,7 +113,8 @@ async function main() {
     }
     runner.backendContexts.hip.sync();
   }
-  for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, { graph: !!args.graph });
+  const runOptions = (extra) => (args.graph === undefined ? extra : Object.assign({ graph: args.graph }, extra));
+  for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, runOptions({}));
   const times = [];
   let outputs = null;
   let queueAhead = null;
@@ -133,7 +138,7 @@ async function main() {
     }
     const t0 = process.hrtime.bigint();
     outputs = await runner.run(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs,
-      { measurePerformance: !!args.measureAll || (!!args.measure && i === args.runs - 1), graph: !!args.graph });
+      runOptions({ measurePerformance: !!args.measureAll || (!!args.measure && i === args.runs - 1) }));
     times.push(Number(process.hrtime.bigint() - t0) / 1e6);
     // --measure-all: device time of every timed run (HIP events on the library's stream; a replayed
     // graph is bracketed by one pair, an eager run has one event per node boundary)
@@ -157,7 +162,7 @@ async function main() {
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
     node: process.version,
-    graph: args.graph ? { captured: !!runner.graphState, unsupported: runner.graphUnsupported } : undefined,
+    graph: args.graph !== false ? { captured: !!runner.graphState, unsupported: runner.graphUnsupported } : undefined,
   };
   runner.disposeGraph();
   if (queueAhead) {
@@ -181,7 +186,11 @@ async function main() {
       report.initializerCopies = Array.from(runner.copiedInitializerTensors.get("hip").keys()).length;
     }
   }
-  process.stdout.write(JSON.stringify(report) + "\n");
+  // the library gives its device memory, stream and staging buffers back before the process ends
+  if (runner.backendContexts.hip && runner.backendContexts.hip.initialized && runner.backendContexts.hip.native.shutdown) {
+    runner.backendContexts.hip.native.shutdown();
+  }
+  process.stdout.write(JSON.stringify(report) + "\n", () => process.exit(0));
 }
 
 main().catch((e) => {

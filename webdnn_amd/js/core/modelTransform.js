@@ -88,10 +88,11 @@ function fuseForHip(model) {
     const attr = node.attribute.find((a) => a.name === "perm");
     return attr && attr.ints ? attr.ints.map(Number) : [];
   };
-  // value of a one-element float constant, or null
+  // value of a one-element float constant of rank 0 or 1, or null (a [1,1,1,1] constant would raise
+  // the rank of the product it multiplies, which the fused node does not)
   const scalarConstant = (name) => {
     const init = initializers.get(name);
-    if (!init) return null;
+    if (!init || init.dims.length > 1) return null;
     let t;
     try {
       t = tensorProtoToArray(init);

@@ -14,7 +14,13 @@
 //     (Date.now() only sees enqueue time there);
 //   * run(inputs, {graph: true}) records the device work of one run into a HIP graph
 //     and replays it on later calls with inputs of the same shapes: the node loop
-//     below (runnerImpl.ts:377-542 in the reference) then runs once, not per call.
+//     below (runnerImpl.ts:377-542 in the reference) then runs once, not per call;
+//   * callers that pass no option get the same thing by themselves (graph: "auto", the
+//     default of backendOptions.hip.graph): two eager runs with inputs of one signature,
+//     then the third is recorded and later ones replay it.  A model that cannot be
+//     recorded, a change of input shapes or a measurePerformance run falls back to the
+//     node loop exactly as {graph: true} does.  backendOptions.hip.graph = false or
+//     run(inputs, {graph: false}) keeps every run in the node loop.
 const fs = require("fs");
 const path = require("path");
 const { backends, backendsWithoutCPU } = require("../interface/constants");
@@ -27,8 +33,13 @@ const { getLogger } = require("../logging");
 
 const logger = getLogger("WebDNN.runner");
 
+// What a captured run is specific to: the types and shapes of the inputs.
+function inputSignature(inputs) {
+  return inputs.map((t) => `${t.dataType}[${t.dims.join(",")}]`).join(";");
+}
+
 class RunnerImpl {
-  // backendContexts: { cpu, hip? };  options: { strict?, fuse? }
+  // backendContexts: { cpu, hip? };  options: { strict?, fuse?, graph?: true | false | "auto" }
   constructor(backendOrder, backendContexts, options) {
     this.backendOrder = backendOrder;
     this.backendContexts = backendContexts;
@@ -45,6 +56,7 @@ class RunnerImpl {
     this.graphWarm = false;
     this.graphUnsupported = null; // reason, once a capture has failed for this model
     this.graphRetries = 0; // captures given up for a reason an eager run cures
+    this.autoSeen = { signature: null, runs: 0 }; // graph "auto": eager runs in a row with one input signature
     // Operator instances by node and by where its inputs live.  The reference builds
     // and initializes a new instance per node per run (runnerImpl.ts:441-452);
     // instances here keep no state beyond their attributes, so later runs reuse them.
@@ -140,9 +152,23 @@ class RunnerImpl {
     if (!this.model || !this.loaded) throw new Error("not initialized");
     if (!inputs) throw new Error("inputs are required");
     const hipContext = this.backendContexts.hip;
-    if (opts.graph && hipContext && hipContext.initialized && hipContext.native.graphBegin && !this.graphUnsupported) {
+    let mode = opts.graph !== undefined ? opts.graph : this.options.graph;
+    if (mode === undefined || mode === null) mode = "auto";
+    const available = hipContext && hipContext.initialized && hipContext.native.graphBegin && !this.graphUnsupported;
+    if (mode === "auto" && available) {
+      // Per-node timings need the node loop; so does anything seen fewer than twice.
+      if (opts.measurePerformance) return this.runEager(inputs, opts);
+      const signature = inputSignature(inputs);
+      if (this.autoSeen.signature !== signature) this.autoSeen = { signature, runs: 0 };
+      if (this.autoSeen.runs < 2) {
+        this.autoSeen.runs++;
+        this.graphWarm = !this.graphState || this.graphState.signature === signature;
+        if (this.graphState && this.graphState.signature !== signature) this.disposeGraph();
+        return this.runEager(inputs, opts);
+      }
       return this.runWithGraph(inputs, opts);
     }
+    if (mode === true && available) return this.runWithGraph(inputs, opts);
     return this.runEager(inputs, opts);
   }
 
@@ -170,7 +196,7 @@ class RunnerImpl {
     const hip = this.backendContexts.hip,
       cpu = this.backendContexts.cpu;
     if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
-    const signature = inputs.map((t) => `${t.dataType}[${t.dims.join(",")}]`).join(";");
+    const signature = inputSignature(inputs);
     if (this.graphState && this.graphState.signature !== signature) {
       // other shapes: other buffers, maybe conv geometries not seen yet -- warm up again
       this.disposeGraph();

@@ -15,7 +15,7 @@ const logger = Logging.getLogger("WebDNN.load");
 
 const defaultContexts = { cpu: null, hip: null };
 
-// options: { backendOrder?, backendOptions?: { hip?: {device, strict, fuse, contractionTile, splitK} },
+// options: { backendOrder?, backendOptions?: { hip?: {device, strict, fuse, graph, contractionTile, splitK} },
 //            onnxBaseName?, optimized? }
 async function load(directory, options) {
   const opts = options || {};
@@ -63,6 +63,7 @@ async function load(directory, options) {
   const runner = new RunnerImpl(actualBackendOrder, backendContexts, {
     strict: !!hipOption.strict,
     fuse: hipOption.fuse,
+    graph: hipOption.graph, // true | false | "auto" (default): see RunnerImpl.run
   });
   // An optimized-model directory holds one graph per backend, named after it, and keeps the
   // weights in WDN2 tensor files (separateBuild/coreOnly.ts:200-204).

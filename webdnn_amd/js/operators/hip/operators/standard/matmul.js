@@ -68,11 +68,20 @@ class HipMatMul extends MatMul {
     }
   }
 
-  product(context, tensorA, tensorB, viewA, viewB, bias, residual) {
+  product(context, tensorA, tensorB, viewA, viewB, bias, residual, activation = this.activation) {
     const plan = this.calcShape(viewA.dims, viewB.dims);
     const { resultDims, resultDimsAfterSqueeze, innerProductLength } = plan;
     const nd = resultDims.length;
     if (nd !== 2 && nd !== 3) throw new Error("MatMul: result rank >= 4 is not supported");
+    if (resultDimsAfterSqueeze.length !== nd && (bias || residual)) {
+      // A rank-1 operand: the Adds that were absorbed saw the squeezed result ([m] of a matrix-vector
+      // product, not [m, 1]), so their broadcasting is not that of the kernel's C term.  They run as
+      // the separate nodes they came from.
+      let output = this.product(context, tensorA, tensorB, viewA, viewB, null, null, "");
+      if (bias) output = addThenActivate(context, output, bias, residual ? "" : activation);
+      if (residual) output = addThenActivate(context, output, residual, activation);
+      return output;
+    }
     // strides of a permuted view replace the dense ones the plan assumes (same broadcasting rule:
     // a batch axis of extent 1 is re-read)
     const stridesOf = (view, planned) => {
@@ -104,7 +113,7 @@ class HipMatMul extends MatMul {
     const sameShape = residual && residual.ndim === resultDimsAfterSqueeze.length &&
       residual.dims.every((d, i) => d === resultDimsAfterSqueeze[i]);
     const inEpilogue = !residual || sameShape;
-    const epilogue = inEpilogue && this.activation === "Relu" ? 1 : 0;
+    const epilogue = inEpilogue && activation === "Relu" ? 1 : 0;
     if (mergeHeads) {
       // [batch, m, n] written as [m, batch, n]: what Transpose(1,0,2) would produce
       const output = context.emptyTensor([m, batch, n], "float32");
@@ -116,7 +125,7 @@ class HipMatMul extends MatMul {
     context.native.gemm(operandHandle(viewA, tensorA), operandHandle(viewB, tensorB), bias ? bias.handle : 0,
       output.handle, batch, m, n, innerProductLength, sAb, sA0, sA1, sBb, sB0, sB1, strideC[0], strideC[1],
       this.alpha, 1.0, epilogue, sameShape ? residual.handle : 0);
-    if (!inEpilogue) output = addThenActivate(context, output, residual, this.activation);
+    if (!inEpilogue) output = addThenActivate(context, output, residual, activation);
     if (this.permY.length) {
       // a result Transpose that could not be folded into the store (rank other than 3)
       const { outShape, inStrides } = permutedView(output.dims, denseStrides(output.dims), this.permY);
