@@ -10,22 +10,25 @@ Workload of `value` (benchmark config 4): ResNet-50 v1, batch 32, fp32, random-i
 batch whose input tensor is already resident in HBM; the step ends when the logits are back on the
 host (the run's only synchronisation).  Steps call runner.run(x, {graph: true}): the first warm-up
 run is eager, the second records the run's kernels into a HIP graph, every timed step launches that
-graph (same kernels, same order, one launch) and reads the logits; `extra.resnet50_ms_per_step_eager`
-is the same step through the node-by-node loop.  `value` = 32 * steps / total time.
+graph (same kernels, same order, one launch) and reads the logits.  `value` = 32 * steps / total time.
 
 `roofline` is for the dominant kernels of that workload, the implicit-GEMM contraction kernels (the
 1x1 convs read X in place, the 3x3 stride-1 convs stage input rows in LDS, the rest gather taps; all
 share one tile schedule and epilogue): their algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over the device time of
 the timed steps, measured with one HIP event pair on the library's stream around each graph replay
 (the step's three other kernels are inside that bracket, which makes the figure a lower bound).
-`roofline.eager_per_node_events` is the same sum from an eager run with an event at every node
-boundary (a run whose launches were all queued before the device reached them, so the events see
-no host gaps; the events themselves cost the stream a few microseconds each).
-`extra` carries the two single-kernel figures the metric names (Gemm 4096^3 and the config-3 Conv, each
-timed as replays of a HIP graph that holds the launches back to back, with the one-by-one launch time
-beside it), the same ResNet-50 step with the batch handed over as a host tensor on every run
-(`resnet50_host_input_graph`: H2D inside the timed region), configs 2 and 5 with their device time,
-the bandwidth-bound kernels and a per-layer table of the step's 54 contraction launches.
+Inside `roofline`, so that one record holds everything the metric names:
+  kernels        Gemm 4096^3 and the config-3 Conv as single-kernel figures (ms, GFLOP/s, fraction of the
+                 fp32 MFMA peak), each timed as replays of a HIP graph that holds the launches back to back,
+                 with the one-by-one launch time beside it;
+  end_to_end     the same ResNet-50 step with the batch handed over as a host tensor on every run
+                 (runner.run([CPUTensor]) with no option: H2D inside the timed region; the runner's
+                 default records the third run and replays it), the same through the node loop only
+                 ({graph: false}), and the network at batch 128;
+  other_configs  configs 2 and 5 with their device time;
+  bandwidth_kernels_frac_of_8TBps  the HBM-bound kernels at the configs' shapes.
+`python bench.py --only layers` prints the per-layer table of the step's 54 contraction launches,
+`--only bandwidth` the bandwidth kernels in full, `--only kernels` the two single kernels (for profiler runs).
 `cpu_baseline` times the JavaScript restatement of the reference's CPU operators (oracle/js) through
 the same runner with backendOrder ["cpu"] in Node.js on one host core, on three images of the batch (one per run, about 20 s).
 """
@@ -79,12 +82,12 @@ def bench_resnet(steps, warmup, workdir):
     assert timed["backend"] == "hip" and list(timed["stats"]["nodesByBackend"]) == ["hip"], timed["stats"]
     assert timed["graph"]["captured"], timed["graph"]
     total_ms = sum(timed["msPerRun"])
-    eager = node_run(workdir, inp, "hip", max(3, steps // 2), max(warmup, 2), ["--strict", "--resident-inputs"])
+    eager = node_run(workdir, inp, "hip", max(3, steps // 2), max(warmup, 2), ["--strict", "--resident-inputs", "--no-graph"])
     # one more run with per-node HIP events for the kernel-level figure.  The run is enqueued behind
     # a few milliseconds of queued streaming kernels, so that all of its launches are in the queue
     # before the device reaches them: the events then time the device, not the host's enqueue rate.
     eager_ms = sum(eager["msPerRun"]) / len(eager["msPerRun"])
-    prof = node_run(workdir, inp, "hip", 1, 2, ["--strict", "--resident-inputs", "--measure",
+    prof = node_run(workdir, inp, "hip", 1, 2, ["--strict", "--resident-inputs", "--no-graph", "--measure",
                                                 "--queue-ahead", "%.1f" % (2 * eager_ms + 2)])
     assert prof["queueAhead"]["deviceMs"] > prof["stats"]["enqueueMs"], (prof["queueAhead"], prof["stats"])
     contraction_ms = sum(p["deviceElapsed"] for p in prof["performance"]
@@ -93,16 +96,17 @@ def bench_resnet(steps, warmup, workdir):
     all_ms = sum(p["deviceElapsed"] or 0.0 for p in prof["performance"])
     # PCIe-inclusive: the input is a host tensor (runner.run([CPUTensor]), as in the reference), uploaded
     # by every run: 19.3 MB through the pinned staging buffers, then the same graph replay / node loop
-    host_in = node_run(workdir, inp, "hip", max(3, steps // 4), 2, ["--strict"])
-    host_in_graph = node_run(workdir, inp, "hip", steps, max(warmup, 2), ["--strict", "--graph"])
+    host_in = node_run(workdir, inp, "hip", max(3, steps // 4), 2, ["--strict", "--no-graph"])
+    # no option at all: what a caller written for the reference does (the runner records the third run)
+    host_in_graph = node_run(workdir, inp, "hip", steps, max(warmup, 3), ["--strict"])
     assert host_in_graph["graph"]["captured"], host_in_graph["graph"]
     return {
         "batch": batch, "flops": g.flops, "nodes": timed["nodes"], "ms_per_step": total_ms / steps,
         "images_per_s": batch * steps / total_ms * 1e3, "contraction_ms": contraction_ms,
         "contraction_launches": launches, "device_ms": all_ms,
         "graph_device_ms": sum(timed["deviceMsPerRun"]) / len(timed["deviceMsPerRun"]),
-        "images_per_s_host_input": batch / (sum(host_in["msPerRun"]) / len(host_in["msPerRun"])) * 1e3,
-        "ms_per_step_host_input_graph": sum(host_in_graph["msPerRun"]) / len(host_in_graph["msPerRun"]),
+        "ms_per_step_host_input_eager": sum(host_in["msPerRun"]) / len(host_in["msPerRun"]),
+        "ms_per_step_host_input": sum(host_in_graph["msPerRun"]) / len(host_in_graph["msPerRun"]),
         "ms_per_step_eager": sum(eager["msPerRun"]) / len(eager["msPerRun"]),
         "device": timed.get("device"), "node_version": timed["node"],
     }
@@ -152,7 +156,7 @@ def bench_report_only(workdir, steps, warmup):
         assert list(rep["stats"]["nodesByBackend"]) == ["hip"], rep["stats"]
         ms = sum(rep["msPerRun"]) / len(rep["msPerRun"])
         dev_ms = sum(rep["deviceMsPerRun"]) / len(rep["deviceMsPerRun"])
-        eager = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs"])
+        eager = node_run(d, inp, "hip", steps, max(warmup, 2), ["--strict", "--resident-inputs", "--no-graph"])
         out[key] = {"workload": label, "nodes": rep["nodes"], "ms_per_run": round(ms, 4),
                     "graph_replay": bool(rep["graph"]["captured"]),
                     "ms_per_run_eager": round(sum(eager["msPerRun"]) / len(eager["msPerRun"]), 4),
@@ -453,13 +457,14 @@ def main():
         baseline = None if args.no_cpu_baseline else cpu_baseline_resnet(workdir)
     kernels = bench_kernels(args.steps, args.warmup)
     bandwidth = bench_bandwidth(args.steps, args.warmup)
-    layers = bench_resnet_layers(args.steps, min(args.warmup, 5))
 
     # The timed steps are graph replays: one HIP event pair brackets each replay on the library's
-    # stream.  That device time covers the 54 contraction launches with their reduce passes plus the
-    # step's three other kernels (MaxPool, GlobalAveragePool, one copy: about 1 % of it), so
-    # FLOPs over it is a lower bound for the contraction kernel alone.
+    # stream.  That device time covers the 54 contraction launches plus the step's three other kernels
+    # (MaxPool, GlobalAveragePool, one copy: about 1 % of it), so FLOPs over it is a lower bound for
+    # the contraction kernels alone.
     achieved = resnet["flops"] / resnet["graph_device_ms"] / 1e9
+    batch = resnet["batch"]
+    pick = lambda d, *keys: {k: d[k] for k in keys}
     line = {
         "metric": METRIC,
         "value": round(resnet["images_per_s"], 1),
@@ -474,15 +479,15 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "ResNet-50 v1 batch 32 [32,3,224,224] fp32, random init (seeded), BN folded, "
-                               "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict, "
-                               "runner.run(x, {graph: true}) replaying the step's captured HIP graph "
-                               "(benchmark config 4)" % resnet["nodes"]},
+                               "%d nodes after Conv+Add+Relu fusion, Node.js runner on the hip backend, strict; "
+                               "a step = runner.run(x) with x resident in HBM, ending with the logits on the host "
+                               "(benchmark config 4); the same step fed a host tensor is in roofline.end_to_end"
+                               % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
-            "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3 and gathered forms; Gemm "
+            "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3, gathered forms, stem; Gemm "
                       "head), %d launches per step; device time = HIP events around each timed graph replay "
-                      "(whole step: includes MaxPool, GlobalAveragePool and the K-split reduce passes)"
-                      % resnet["contraction_launches"],
+                      "(whole step, MaxPool and GlobalAveragePool included)" % resnet["contraction_launches"],
             "achieved": round(achieved, 2),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
@@ -492,35 +497,45 @@ def main():
             "flops_per_step": resnet["flops"],
             "avg_launch_ms": round(resnet["graph_device_ms"] / resnet["contraction_launches"], 5),
             "step_device_ms": round(resnet["graph_device_ms"], 4),
-            "eager_per_node_events": {
-                "note": "same nodes timed one by one (an event per node boundary, each costing the stream a "
-                        "bubble of a few microseconds) in an eager run queued behind other work",
-                "contraction_ms": round(resnet["contraction_ms"], 4),
-                "tflops": round(resnet["flops"] / resnet["contraction_ms"] / 1e9, 2)},
+            # the two single-kernel figures the metric names (graph replays of back-to-back launches)
+            "kernels": {
+                "gemm_4096": pick(kernels["gemm_4096"], "ms", "gflops", "frac_mfma_peak", "ms_launched_one_by_one"),
+                "conv_c3": pick(kernels["conv_c3"], "ms", "gflops", "frac_mfma_peak", "ms_launched_one_by_one"),
+            },
+            # ResNet-50 b32 images/s by how the batch reaches the device and how runner.run is called
+            "end_to_end": {
+                "resident_input_images_per_s": round(resnet["images_per_s"], 1),
+                "host_input_images_per_s": round(batch / resnet["ms_per_step_host_input"] * 1e3, 1),
+                "host_input_ms_per_step": round(resnet["ms_per_step_host_input"], 4),
+                "host_input_note": "runner.run([CPUTensor]) with no option, as the reference's callers write it: "
+                                   "19.3 MB over PCIe inside every timed step; the runner records the third run "
+                                   "and replays it (graph \"auto\")",
+                "host_input_node_loop_images_per_s": round(batch / resnet["ms_per_step_host_input_eager"] * 1e3, 1),
+                "resident_input_node_loop_ms_per_step": round(resnet["ms_per_step_eager"], 4),
+                "batch128_device_frac_mfma_peak": large_batch["device_frac_mfma_peak"],
+                "batch128_images_per_s": large_batch["images_per_s"],
+            },
+            "other_configs": {
+                "ffn_c2_device_ms": report_only["ffn_c2"]["device_ms"],
+                "ffn_c2_device_frac_mfma_peak": report_only["ffn_c2"]["device_frac_mfma_peak"],
+                "detr_r50_b1_ms_per_run": report_only["detr_r50_b1"]["ms_per_run"],
+                "detr_r50_b1_device_ms": report_only["detr_r50_b1"]["device_ms"],
+                "detr_r50_b1_device_frac_mfma_peak": report_only["detr_r50_b1"]["device_frac_mfma_peak"],
+            },
+            "bandwidth_kernels_frac_of_8TBps": {k: v["frac_hbm_peak"] for k, v in bandwidth.items()},
         },
-        "extra": {
-            "gemm_4096": kernels["gemm_4096"],
-            "conv_c3": kernels["conv_c3"],
-            "ffn_c2": report_only["ffn_c2"],
-            "detr_r50_b1": report_only["detr_r50_b1"],
-            "bandwidth_kernels": {"unit": "GB/s of algorithmic bytes (HIP events around back-to-back launches)",
-                                  "peak": 8000.0, "kernels": bandwidth},
-            "resnet50_device_ms_per_step": round(resnet["device_ms"], 4),
-            "resnet50_ms_per_step_eager": round(resnet["ms_per_step_eager"], 4),
-            "resnet50_images_per_s_host_input": round(resnet["images_per_s_host_input"], 1),
-            "resnet50_host_input_graph": {
-                "note": "the same step with the batch handed over as a host tensor on every run "
-                        "(runner.run([CPUTensor]), 19.3 MB over PCIe inside the timed region), graph replay",
-                "ms_per_step": round(resnet["ms_per_step_host_input_graph"], 4),
-                "images_per_s": round(resnet["batch"] / resnet["ms_per_step_host_input_graph"] * 1e3, 1)},
-            "resnet50_b128": large_batch,
-            "resnet50_layers": layers,
-            "device": resnet["device"],
-        },
+        # the same figures once more as plain scalars
+        "gemm_4096_frac_mfma_peak": kernels["gemm_4096"]["frac_mfma_peak"],
+        "conv_c3_frac_mfma_peak": kernels["conv_c3"]["frac_mfma_peak"],
+        "host_input_images_per_s": round(batch / resnet["ms_per_step_host_input"] * 1e3, 1),
+        "host_input_node_loop_images_per_s": round(batch / resnet["ms_per_step_host_input_eager"] * 1e3, 1),
+        "device": resnet["device"],
     }
     if baseline is not None:
         line["cpu_baseline"] = baseline
-    print(json.dumps(line))
+    text = json.dumps(line)
+    assert len(text) < 8000, "the bench line must stay under 8 KB (%d)" % len(text)
+    print(text)
 
 
 if __name__ == "__main__":

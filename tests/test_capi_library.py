@@ -109,3 +109,23 @@ def test_stem_kernel_steps_aside_for_images_beyond_its_32_bit_indexing():
     assert applies(224, 224) and applies(800, 1088)
     assert not applies(14000, 14000)        # an image (and its results) beyond 2 GiB
     assert not fn(4, 64, 7, 7, 2, 2, 1, 1, 1, 224, 224, 3, 3, 112, 112)
+
+
+def test_typed_surface_lists_every_addon_function_with_its_argument_count():
+    """interface/backend/hip/hipNative.d.ts is written by hand: it must name exactly the functions the
+    addon exports, each with as many parameters as the addon's ARGS() check demands."""
+    addon = open(os.path.join(ROOT, "webdnn_amd", "napi", "addon.c")).read()
+    exported = dict(re.findall(r'\{"(\w+)",\s*(js_\w+)\}', addon))
+    argc = {}
+    for js_name, c_name in exported.items():
+        body = addon[addon.index("FN(%s)" % c_name):]
+        m = re.search(r'ARGS\("\w+",\s*(\d+)\)', body[:body.index("\n}\n")])
+        argc[js_name] = int(m.group(1)) if m else 0          # js_shutdown takes none and has no ARGS()
+    text = open(os.path.join(ROOT, "webdnn_amd", "js", "interface", "backend", "hip", "hipNative.d.ts")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    iface = text[text.index("export interface HipNative {"):]
+    declared = {}
+    for name, params in re.findall(r"^\s{2}(\w+)\(([^)]*)\)\s*:", iface, flags=re.M | re.S):
+        declared[name] = 0 if not params.strip() else params.count(",") + 1
+    assert declared == argc

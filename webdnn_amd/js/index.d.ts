@@ -1,0 +1,45 @@
+// Entry points of the package (index.js).  Reference: src/descriptor_runner/index.ts:23-149 and
+// interface/core/runner.ts; `backendOptions.hip` and the `graph` run option are the additions.
+import { Backend } from "./interface/core/constants";
+import { Tensor } from "./interface/core/tensor";
+import { WebDNNHipContext, WebDNNHipContextOption } from "./interface/backend/hip/hipContext";
+
+export interface InitOption {
+  backendOrder?: Backend[];
+  backendOptions?: { hip?: WebDNNHipContextOption };
+  /** file name of the graph inside the directory (default model.onnx, or model-<backend>.onnx with `optimized`) */
+  onnxBaseName?: string | null;
+  /** the directory is an optimized-model directory (graph per backend, WDN2 weight files) */
+  optimized?: boolean;
+}
+
+export interface RunOption {
+  measurePerformance?: boolean;
+  graph?: boolean | "auto";
+}
+
+export interface RunStats {
+  nodesByBackend: Record<string, number>;
+  retriedOnCpu: string[];
+  nodes: number;
+  operatorsCreated: number;
+  enqueueMs?: number;
+  graphReplay?: boolean;
+}
+
+export interface Runner {
+  readonly backendName: Backend;
+  readonly backendContexts: { cpu: unknown; hip?: WebDNNHipContext };
+  lastRunStats: RunStats | null;
+  lastPerformance: Array<{ name: string; opType: string; backend: Backend; elapsed?: number; deviceElapsed?: number }> | null;
+  graphUnsupported: string | null;
+  getInputNames(): string[];
+  getOutputNames(): string[];
+  /** outputs come back as CPU tensors, as in the reference */
+  run(inputs?: Tensor[], options?: RunOption): Promise<Tensor[]>;
+  disposeGraph(): void;
+}
+
+export function load(directory: string, options?: InitOption): Promise<Runner>;
+export const CPUTensor: new (dims: ReadonlyArray<number>, dataType?: "float32" | "int32" | "bool",
+                             data?: Float32Array | Int32Array | Uint8Array) => Tensor;

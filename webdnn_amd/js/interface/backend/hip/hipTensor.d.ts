@@ -1,0 +1,13 @@
+// Device tensor of the hip backend (backend/hip/hipTensorImpl.js).  Shaped after
+// src/descriptor_runner/interface/backend/wasm/wasmTensor.ts; `handle` and `alias` are what the hip
+// operators use beyond the Tensor contract.
+import { Tensor } from "../../core/tensor";
+
+export interface HipTensor extends Tensor {
+  readonly backend: "hip";
+  /** Buffer handle of libwebdnn_hip.so (a wdh_buf, > 0).  Throws after dispose(). */
+  readonly handle: number;
+  /** Another view of the same device buffer with other dims (Reshape, Flatten, Squeeze, Unsqueeze);
+   *  the buffer is freed when the last view is disposed. */
+  alias(dims: ReadonlyArray<number>): HipTensor;
+}
