@@ -92,6 +92,19 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       batch strides of Y that are multiples of four) are turned through
  *                       LDS and stored 16 bytes per lane; 0 = every lane stores single
  *                       elements (same arithmetic, same bits).
+ *   "stream_k"          how wdh_gemm / wdh_conv2d launches whose tiles do not fill the chip in
+ *                       whole rounds are scheduled: 1 (default) = such launches keep a fixed
+ *                       grid of resident workgroups, each of which multiplies an equal,
+ *                       contiguous share of all K slabs of the launch, tile borders or not;
+ *                       a tile shared by neighbouring workgroups is added up in K order by
+ *                       the one that holds its last slabs (one launch, no second pass);
+ *                       2 = every launch that can; 0 = none (one tile or K chunk per
+ *                       workgroup, chunks added by a second kernel).  The sums of a tile are
+ *                       added in another order than with 0; both orders are fixed.
+ *   "stream_wgs"        1..8 (default 4) = resident workgroups per CU of such a launch.
+ *   "stream_spin"       how often a workgroup polls for a neighbour's partial tile before it
+ *                       gives up (the next wdh_sync / wdh_read then fails with WDH_EHIP); a
+ *                       test hook.
  *   "descriptor_loads"  1 (default) = operands below 2 GiB are read and written
  *                       through buffer descriptors with 32-bit offsets; 0 = every
  *                       operand is treated as if it spanned 2 GiB or more (64-bit
@@ -106,7 +119,9 @@ int wdh_set_option(const char *name, int value);
  * reports; cf. the per-node records of measurePerformance,
  * core/runnerImpl.ts:533-541): workgroup tile, the number of tiles computed whole
  * and of tiles cut along K, chunks per cut tile (1 = none), and which form of the
- * kernel ran: WDH_FORM_* below.  Any pointer may be NULL. */
+ * kernel ran: WDH_FORM_* below.  A launch scheduled as a stream of K slabs ("stream_k")
+ * reports split = 0, all its tiles as whole_tiles and its workgroup count as split_tiles.
+ * Any pointer may be NULL. */
 #define WDH_FORM_GEMM_KC 0        /* B k-contiguous (transB)                    */
 #define WDH_FORM_GEMM_MC 1        /* B n-contiguous                             */
 #define WDH_FORM_CONV_GATHER32 2  /* taps gathered from X, at most 31 taps      */
@@ -239,7 +254,7 @@ int wdh_linear_group(int count, const wdh_buf *A, const wdh_buf *W, const wdh_bu
  * they later read, so nothing has to be cleared, but two such calls that overlap
  * on one GPU (other streams, other threads) race; the library's single stream
  * orders them. */
-#define WDH_STATIC_SCRATCH_BYTES (16u << 20)
+#define WDH_STATIC_SCRATCH_BYTES ((32u << 20) + (160u << 10))
 int wdh_gemm_static(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
                     int n, int k, int64_t sAb, int64_t sA0, int64_t sA1,
                     int64_t sBb, int64_t sB0, int64_t sB1, int64_t sC0,

@@ -1183,10 +1183,11 @@ def test_small_products_cut_k_across_the_wavefronts_of_a_workgroup(ctx, batch, m
 
 def test_few_blocks_with_a_long_k_keep_the_ordinary_tiles(ctx):
     """The ResNet classifier head, [32,2048] x [1000,2048]^T: 32 blocks of 32x32 would leave the 8 MB of
-    weights to 32 workgroups; it stays with 64x64 tiles cut along K."""
+    weights to 32 workgroups; it stays with 64x64 tiles whose K is shared out (as a stream of K slabs,
+    or in chunks with a reduce pass when that schedule is switched off)."""
     A, B, C = uni(32, 2048), uni(1000, 2048), uni(1000)
     got = hip_gemm(ctx, A, B, C, 1.0, 1.0, 0, 1)
-    assert ctx.last_plan()["tile"] == "64x64" and ctx.last_plan()["split"] > 1
+    assert ctx.last_plan()["tile"] == "64x64" and ctx.last_plan()["split"] != 1
     assert_close_max(got, ref.gemm(A, B, C, 1.0, 1.0, 0, 1), GEMM_TOL, "classifier head")
 
 

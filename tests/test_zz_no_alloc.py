@@ -90,7 +90,7 @@ def test_static_workspace_rejects_what_does_not_fit(ctx):
     y = ctx.empty_tensor([m, n])
     args = (ta.handle, tb.handle, 0, y.handle, 1, m, n, k, 0, k, 1, 0, n, 1, 0, 0, 1.0, 1.0, 0, 0)
     try:
-        ctx.set_option("split_k", 8)      # 256 tiles x 8 chunks x 16 KiB = 32 MiB of partial sums
+        ctx.set_option("split_k", 16)     # 256 tiles x 16 chunks x 16 KiB = 64 MiB of partial sums
         with pytest.raises(capi.HipError) as err:
             capi.call("wdh_gemm_static", *args)
         assert err.value.code == -2 and "static workspace" in str(err.value)

@@ -27,6 +27,8 @@ int init_attention();
 // Device resources of the contraction kernels that outlive a call (called by wdh_init / at shutdown).
 int init_contraction();
 void release_contraction();
+// After a synchronisation: fails if a contraction kernel reported that it gave up a wait.
+int contraction_check();
 
 // Handle -> device pointer.  Returns nullptr (and records WDH_EINVAL) for an
 // unknown handle.  A zero-byte buffer resolves to a non-null dummy pointer.

@@ -535,7 +535,7 @@ int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
     copied += chunk_of[which];
     which = next;
   }
-  return WDH_OK;
+  return wdh::contraction_check();  // (the stream has drained up to the data just read)
 }
 
 int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
@@ -559,7 +559,7 @@ int wdh_sync(void) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_sync");
   WDH_HIP_CHECK(hipStreamSynchronize(g.stream));
-  return WDH_OK;
+  return wdh::contraction_check();
 }
 
 int wdh_mem_stats(uint64_t *in_use, uint64_t *cached, uint64_t *peak) {
