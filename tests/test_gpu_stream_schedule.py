@@ -63,7 +63,8 @@ def test_gemm_as_a_stream(stream_always, m, n, k, tile):
         plan = ctx.last_plan()
         want = ref.unary("Relu", ref.gemm(A, B, C, 0.75, -1.25, 0, 1))
         assert_close_max(got, want, TOL, "stream gemm %s tile %d (%s)" % ((m, n, k), tile, plan))
-        assert plan["split"] == 0, plan            # the stream schedule did run
+        # the stream schedule did run (operand rows that are not 16-byte aligned have no stream form)
+        assert plan["split"] == (0 if k % 4 == 0 else 1), plan
         again = gemm(ctx, A, B, C, 0.75, -1.25, 0, 1, "relu")
         assert_bit_exact(again, got, "the same launch twice")
     finally:
@@ -119,7 +120,7 @@ def test_conv_as_a_stream(stream_always, shape, tile):
     plan = ctx.last_plan()
     want = ref.unary("Relu", ref.binary("Add", ref.conv(X, W, B, pads=[p] * 4, strides=[s, s], group=g), R))
     assert_close_max(got, want, TOL, "stream conv %s tile %d (%s)" % (shape, tile, plan))
-    assert plan["split"] == 0, plan
+    assert plan["split"] == (0 if (cin // g * k * k) % 4 == 0 else 1), plan
     again = conv(ctx, X, W, B, pads=[p] * 4, strides=[s, s], group=g, epilogue="relu", R=R)
     assert_bit_exact(again, got, "the same launch twice")
 

@@ -25,7 +25,7 @@ int init_static_scratch(int device);
 // Raises the dynamic LDS limit of the attention kernels on the current device (called by wdh_init).
 int init_attention();
 // Device resources of the contraction kernels that outlive a call (called by wdh_init / at shutdown).
-int init_contraction();
+int init_contraction(int device);
 void release_contraction();
 // After a synchronisation: fails if a contraction kernel reported that it gave up a wait.
 int contraction_check();

@@ -904,138 +904,147 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
   const int li = lane & 31, half = lane >> 5;
   const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
 
-  // A stream launch walks the segments of this workgroup's slab range (see stream_next);
-  // any other launch has one tile, or one chunk of a tile, per workgroup.
-  StreamPos pos = {};
-  if (STREAM) pos = stream_begin(p);
-  for (bool again = false;; again = true) {
-  // which tile, and which part of K
-  bool whole = true;
-  int lin, chunk = 0, bz, tm, tn, kbeg, kend;
-  Segment sg = {};
-  if (STREAM) {
-    if (pos.cur_end <= pos.u0) break;
-    if (again) __syncthreads();  // the previous segment's epilogue has finished with the LDS
-    sg = stream_next(p, pos);
-    lin = sg.lin;
-    kbeg = sg.sbeg * BK;
-    kend = sg.send * BK < p.k ? sg.send * BK : p.k;
-    const int tiles_per_z = p.tiles_m * p.tiles_n;
-    bz = fdiv(lin, p.fd_tiles_per_z);
-    tile_coords(p, lin - bz * tiles_per_z, &tm, &tn);
-  } else {
-    if (again) break;
-    const TileWork tw = decode_work(p);
-    whole = tw.whole;
-    lin = tw.lin; chunk = tw.chunk; bz = tw.bz; tm = tw.tm; tn = tw.tn;
-    // this workgroup's share of K
-    kbeg = whole ? 0 : chunk * p.kchunk;
-    kend = whole ? p.k : (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k);
-  }
-  const int row0 = tm * BM, col0 = tn * BN;
+  // Everything the loops need to know about one segment of work: the tile, the part of K, and
+  // this thread's fetch plan (one byte offset per 16-byte piece, every address term folded in
+  // before the K loop starts).
+  struct Ctx {
+    bool whole, first, last;
+    int lin, chunk, bz, row0, col0, kbeg, kend;
+    const float *A, *B;
+    long long lda, ldb;
+    int voff_a[BM / 64], voff_b[BN / 64];
+    rsrc_t rsrc_a, rsrc_b;
+    PixelCtx px;
+    PixelFast pf;
+    int kgroup0;   // first of the L consecutive k rows this wavefront gathers in each slab
+    int tile_begin;
+  };
+  const bool a_fast = p.fast;
+  const bool b_fast = p.fast && BMODE_ != B_IM2COL_BIG;
 
-  const float *A = p.A + (long long)bz * p.sAb;
-  const float *B = p.B + (long long)bz * p.sBb;
-  const long long lda = A_KC ? p.sA0 : p.sA1;
-  const long long ldb = B_IS_KC ? p.sB1 : p.sB0;
-
-  // ---- descriptor fetch plans: one byte offset per 16-byte piece -------------
+  // ---- descriptor fetch plans --------------------------------------------------------
   // Every operand below 2 GiB takes this path, edge tiles included.  Rows of a
   // row-major-in-K operand past the edge are clamped; an operand that is
   // contiguous along M or N simply reads on past its last row or column, into
   // the next k row (or, past the end of the matrix, zeros from the descriptor's
   // bounds check).  Either way the surplus rows and columns only feed products
   // that are never stored.
-  const bool a_fast = p.fast;
-  const bool b_fast = p.fast && BMODE_ != B_IM2COL_BIG;
-  int voff_a[BM / 64], voff_b[BN / 64];
-  if (A_KC) {
+  auto setup = [&](Ctx &c, int tm, int tn) {
+    const int bz = c.bz;
+    const int row0 = c.row0 = tm * BM, col0 = c.col0 = tn * BN;
+    c.A = p.A + (long long)bz * p.sAb;
+    c.B = p.B + (long long)bz * p.sBb;
+    const long long lda = c.lda = A_KC ? p.sA0 : p.sA1;
+    const long long ldb = c.ldb = B_IS_KC ? p.sB1 : p.sB0;
+    if (A_KC) {
 #pragma unroll
-    for (int i = 0; i < BM / 64; i++) {
-      int r = row0 + (tid >> 2) + i * 64;
-      r = r < p.m ? r : p.m - 1;
-      voff_a[i] = (int)(((long long)r * lda + (tid & 3) * 4) * 4);
+      for (int i = 0; i < BM / 64; i++) {
+        int r = row0 + (tid >> 2) + i * 64;
+        r = r < p.m ? r : p.m - 1;
+        c.voff_a[i] = (int)(((long long)r * lda + (tid & 3) * 4) * 4);
+      }
+    } else {
+      constexpr int TPR = BM / 4, RPP = NTHREADS / TPR;
+#pragma unroll
+      for (int i = 0; i < BM / 64; i++)
+        c.voff_a[i] = (int)(((long long)(tid / TPR + i * RPP) * lda + row0 + (tid % TPR) * 4) * 4);
     }
-  } else {
-    constexpr int TPR = BM / 4, RPP = NTHREADS / TPR;
+    if (B_IS_KC) {
 #pragma unroll
-    for (int i = 0; i < BM / 64; i++)
-      voff_a[i] = (int)(((long long)(tid / TPR + i * RPP) * lda + row0 + (tid % TPR) * 4) * 4);
-  }
-  if (B_IS_KC) {
+      for (int i = 0; i < BN / 64; i++) {
+        int cc = col0 + (tid >> 2) + i * 64;
+        cc = cc < p.n ? cc : p.n - 1;
+        c.voff_b[i] = (int)(((long long)cc * ldb + (tid & 3) * 4) * 4);
+      }
+    } else if (!IM2COL) {
+      constexpr int TPR = BN / 4, RPP = NTHREADS / TPR;
+      // B_PIXELS: column = pixel index over the batch; its four pixels share an image
+      long long colpos = col0 + (tid % TPR) * 4;
+      if (PIXELS) {
+        const unsigned plane = (unsigned)(p.cv.h * p.cv.w);
+        const unsigned img = (unsigned)fdiv((int)colpos, p.cv.fd_plane);
+        colpos = (long long)img * p.cv.c_total * plane + ((unsigned)colpos - img * plane);
+      }
 #pragma unroll
-    for (int i = 0; i < BN / 64; i++) {
-      int c = col0 + (tid >> 2) + i * 64;
-      c = c < p.n ? c : p.n - 1;
-      voff_b[i] = (int)(((long long)c * ldb + (tid & 3) * 4) * 4);
+      for (int i = 0; i < BN / 64; i++)
+        c.voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + colpos) * 4);
     }
-  } else if (!IM2COL) {
-    constexpr int TPR = BN / 4, RPP = NTHREADS / TPR;
-    // B_PIXELS: column = pixel index over the batch; its four pixels share an image
-    long long colpos = col0 + (tid % TPR) * 4;
-    if (PIXELS) {
-      const unsigned plane = (unsigned)(p.cv.h * p.cv.w);
-      const unsigned img = (unsigned)fdiv((int)colpos, p.cv.fd_plane);
-      colpos = (long long)img * p.cv.c_total * plane + ((unsigned)colpos - img * plane);
-    }
-#pragma unroll
-    for (int i = 0; i < BN / 64; i++)
-      voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + colpos) * 4);
-  }
-  const rsrc_t rsrc_a = make_rsrc(A, p.a_bytes);
+    c.rsrc_a = make_rsrc(c.A, p.a_bytes);
 
-  // ---- im2col: what this thread's pixel looks like ----------------------------
-  PixelCtx px = {p.B, 0, 0, 0, 0ull};
-  PixelFast pf = {0, 0xffffffffu, 0xffffffffu};
-  const float *bbase = B;  // base of the B descriptor
-  if (IM2COL) {
-    const unsigned P = (unsigned)col0 + (unsigned)(tid % BN);  // npix < 2^31
-    const long long plane = (long long)p.cv.h * p.cv.w;
-    const int bias = p.cv.pt * p.cv.w + p.cv.pl;  // makes every corner offset >= 0
-    px.xbase = p.B + (long long)bz * p.cv.c_in_g * plane;
-    bbase = px.xbase - bias;
-    if (P < (unsigned)p.cv.npix) {
-      const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
-      const unsigned img = (unsigned)fdiv((int)P, p.cv.fd_ohw);
-      const unsigned q = P - img * ohw;
-      const int oy = fdiv((int)q, p.cv.fd_ow), ox = (int)q - oy * p.cv.ow;
-      const long long img_off = (long long)img * p.cv.c_total * plane;
-      px.iy0 = oy * p.cv.sh - p.cv.pt;
-      px.ix0 = ox * p.cv.sw - p.cv.pl;
-      px.pbase = px.iy0 * p.cv.w + px.ix0;
-      if (IM2COL_FAST) {
-        pf.valid = (int)((img_off + px.pbase + bias) * 4);
-        // which taps of this pixel fall inside the input: rows first, then columns
-        unsigned long long inside = 0;
-        int t = 0;
-        for (int ky = 0; ky < p.cv.kh; ky++) {
-          const bool row_in = (unsigned)(px.iy0 + ky * p.cv.dh) < (unsigned)p.cv.h;
-          for (int kx = 0; kx < p.cv.kw; kx++, t++)
-            if (row_in && (unsigned)(px.ix0 + kx * p.cv.dw) < (unsigned)p.cv.w)
-              inside |= 1ull << t;
+    // ---- im2col: what this thread's pixel looks like ----------------------------
+    c.px = PixelCtx{p.B, 0, 0, 0, 0ull};
+    c.pf = PixelFast{0, 0xffffffffu, 0xffffffffu};
+    const float *bbase = c.B;  // base of the B descriptor
+    if (IM2COL) {
+      const unsigned P = (unsigned)col0 + (unsigned)(tid % BN);  // npix < 2^31
+      const long long plane = (long long)p.cv.h * p.cv.w;
+      const int bias = p.cv.pt * p.cv.w + p.cv.pl;  // makes every corner offset >= 0
+      c.px.xbase = p.B + (long long)bz * p.cv.c_in_g * plane;
+      bbase = c.px.xbase - bias;
+      if (P < (unsigned)p.cv.npix) {
+        const unsigned ohw = (unsigned)(p.cv.oh * p.cv.ow);
+        const unsigned img = (unsigned)fdiv((int)P, p.cv.fd_ohw);
+        const unsigned q = P - img * ohw;
+        const int oy = fdiv((int)q, p.cv.fd_ow), ox = (int)q - oy * p.cv.ow;
+        const long long img_off = (long long)img * p.cv.c_total * plane;
+        c.px.iy0 = oy * p.cv.sh - p.cv.pt;
+        c.px.ix0 = ox * p.cv.sw - p.cv.pl;
+        c.px.pbase = c.px.iy0 * p.cv.w + c.px.ix0;
+        if (IM2COL_FAST) {
+          c.pf.valid = (int)((img_off + c.px.pbase + bias) * 4);
+          // which taps of this pixel fall inside the input: rows first, then columns
+          unsigned long long inside = 0;
+          int t = 0;
+          for (int ky = 0; ky < p.cv.kh; ky++) {
+            const bool row_in = (unsigned)(c.px.iy0 + ky * p.cv.dh) < (unsigned)p.cv.h;
+            for (int kx = 0; kx < p.cv.kw; kx++, t++)
+              if (row_in && (unsigned)(c.px.ix0 + kx * p.cv.dw) < (unsigned)p.cv.w)
+                inside |= 1ull << t;
+          }
+          c.pf.pad_lo = ~(unsigned)inside;
+          c.pf.pad_hi = ~(unsigned)(inside >> 32);
+        } else {
+          c.px.xbase += img_off;
+          c.px.mask = 1ull;
         }
-        pf.pad_lo = ~(unsigned)inside;
-        pf.pad_hi = ~(unsigned)(inside >> 32);
-      } else {
-        px.xbase += img_off;
-        px.mask = 1ull;
       }
     }
-  }
-  // conv: p.b_bytes is group 0's window, later groups start further into X
-  const int b_window =
-      CONV ? p.b_bytes - (int)((long long)bz * p.cv.c_in_g * p.cv.h * p.cv.w * 4) : p.b_bytes;
-  const rsrc_t rsrc_b = make_rsrc(bbase, b_window);
-  // first of the L consecutive k rows this wavefront gathers in each slab
-  const int kgroup0 = IM2COL ? __builtin_amdgcn_readfirstlane(tid / BN) * (BK / (NTHREADS / BN)) : 0;
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int a = 0; a < MT; a++)
-#pragma unroll
-    for (int b = 0; b < NT; b++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+    // conv: p.b_bytes is group 0's window, later groups start further into X
+    const int b_window =
+        CONV ? p.b_bytes - (int)((long long)bz * p.cv.c_in_g * p.cv.h * p.cv.w * 4) : p.b_bytes;
+    c.rsrc_b = make_rsrc(bbase, b_window);
+    c.kgroup0 = IM2COL ? __builtin_amdgcn_readfirstlane(tid / BN) * (BK / (NTHREADS / BN)) : 0;
+  };
+  // A stream launch walks the segments of this workgroup's slab range (see stream_next);
+  // any other launch has one tile, or one chunk of a tile, per workgroup.
+  StreamPos pos = {};
+  if (STREAM) pos = stream_begin(p);
+  auto next_segment = [&](Ctx &c) {
+    int tm, tn;
+    if (STREAM) {
+      const Segment sg = stream_next(p, pos);
+      c.whole = true;
+      c.first = sg.first;
+      c.last = sg.last;
+      c.tile_begin = sg.tile_begin;
+      c.lin = sg.lin;
+      c.chunk = 0;
+      c.kbeg = sg.sbeg * BK;
+      c.kend = sg.send * BK < p.k ? sg.send * BK : p.k;
+      c.bz = fdiv(c.lin, p.fd_tiles_per_z);
+      tile_coords(p, c.lin - c.bz * (p.tiles_m * p.tiles_n), &tm, &tn);
+    } else {
+      const TileWork tw = decode_work(p);
+      c.whole = tw.whole;
+      c.first = c.last = true;
+      c.tile_begin = 0;
+      c.lin = tw.lin; c.chunk = tw.chunk; c.bz = tw.bz; tm = tw.tm; tn = tw.tn;
+      // this workgroup's share of K
+      c.kbeg = c.whole ? 0 : c.chunk * p.kchunk;
+      c.kend = c.whole ? p.k : (c.kbeg + p.kchunk < p.k ? c.kbeg + p.kchunk : p.k);
+    }
+    setup(c, tm, tn);
+  };
 
   // Registers that carry one fetched K slab from global memory to LDS.
   struct Staged {
@@ -1044,34 +1053,34 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
   };
   // Descriptor-only fetch: legal for a slab that lies fully inside K when
   // both operands qualify (all_fast).
-  auto fetch_fast = [&](int k0, Staged &st) {
-    fetch_rows_fast<BM, VEC>(rsrc_a, voff_a, A_KC ? k0 * 4 : (int)(k0 * lda * 4), st.a);
+  auto fetch_fast = [&](const Ctx &c, int k0, Staged &st) {
+    fetch_rows_fast<BM, VEC>(c.rsrc_a, c.voff_a, A_KC ? k0 * 4 : (int)(k0 * c.lda * 4), st.a);
     if (IM2COL_FAST)
-      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(rsrc_b, p.cv.ktab, pf, k0 + kgroup0, st.b);
+      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(c.rsrc_b, p.cv.ktab, c.pf, k0 + c.kgroup0, st.b);
     else if (!IM2COL)
-      fetch_rows_fast<BN, VEC>(rsrc_b, voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * ldb * 4), st.b);
+      fetch_rows_fast<BN, VEC>(c.rsrc_b, c.voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * c.ldb * 4), st.b);
   };
   // Fetch that copes with everything: ragged last slab, edge tiles, huge operands.
-  auto fetch_any = [&](int k0, Staged &st) {
-    const bool full = k0 + BK <= kend;
+  auto fetch_any = [&](const Ctx &c, int k0, Staged &st) {
+    const bool full = k0 + BK <= c.kend;
     if (a_fast && full) {
-      fetch_rows_fast<BM, VEC>(rsrc_a, voff_a, A_KC ? k0 * 4 : (int)(k0 * lda * 4), st.a);
+      fetch_rows_fast<BM, VEC>(c.rsrc_a, c.voff_a, A_KC ? k0 * 4 : (int)(k0 * c.lda * 4), st.a);
     } else if (A_KC) {
-      fetch_kc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
+      fetch_kc<BM, VEC>(c.A, c.lda, c.row0, p.m, k0, c.kend, tid, st.a);
     } else {
-      fetch_mc<BM, VEC>(A, lda, row0, p.m, k0, kend, tid, st.a);
+      fetch_mc<BM, VEC>(c.A, c.lda, c.row0, p.m, k0, c.kend, tid, st.a);
     }
     if (IM2COL_FAST) {
       // padding entries of the tap table read as 0, so a ragged K needs no care
-      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(rsrc_b, p.cv.ktab, pf, k0 + kgroup0, st.b);
+      fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(c.rsrc_b, p.cv.ktab, c.pf, k0 + c.kgroup0, st.b);
     } else if (IM2COL) {
-      st.ok = fetch_im2col<BN>(p.cv, px, k0, kend, tid, st.b);
+      st.ok = fetch_im2col<BN>(p.cv, c.px, k0, c.kend, tid, st.b);
     } else if ((b_fast && full) || PIXELS) {
-      fetch_rows_fast<BN, VEC>(rsrc_b, voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * ldb * 4), st.b);
+      fetch_rows_fast<BN, VEC>(c.rsrc_b, c.voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * c.ldb * 4), st.b);
     } else if (B_IS_KC) {
-      fetch_kc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
+      fetch_kc<BN, VEC>(c.B, c.ldb, c.col0, p.n, k0, c.kend, tid, st.b);
     } else {
-      fetch_mc<BN, VEC>(B, ldb, col0, p.n, k0, kend, tid, st.b);
+      fetch_mc<BN, VEC>(c.B, c.ldb, c.col0, p.n, k0, c.kend, tid, st.b);
     }
   };
   auto stash = [&](int buf, const Staged &st) {
@@ -1088,6 +1097,8 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
     else
       stash_mc<BN>(lds_b[buf], tid, st.b);
   };
+
+  f32x16 acc[MT][NT];
   // One K slab from LDS buffer `cur` through the matrix cores.
   auto compute = [&](int cur) {
     const float *ta = lds_a[cur];
@@ -1128,51 +1139,76 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
     }
   };
 
-  // Slab s+1 travels global -> registers while slab s runs through the matrix
-  // cores, then goes to the other LDS buffer.  (A second slab in flight was
-  // measured and bought nothing.)  The main loop takes two slabs per trip, so
-  // that LDS buffer indices are compile-time constants, and contains
-  // descriptor fetches only; the few slabs it leaves over (and every slab of a
-  // workgroup that cannot use descriptors) run in the general loop below it.
-  const int nslabs = (kend - kbeg + BK - 1) / BK;
-  const int nfull = (kend - kbeg) / BK;
-  const bool all_fast = a_fast && b_fast && !(IM2COL && !IM2COL_FAST);
-  const int nfast = all_fast ? nfull - 1 : 0;  // steps whose next slab is a full one
+  Ctx c;
   Staged st0;
-  fetch_any(kbeg, st0);
-  stash(0, st0);
-  __syncthreads();
-  int s = 0;
-  // The scheduling fences keep the compiler from sinking the loads below the
-  // matrix-core work they are meant to overlap.
-  for (; s + 2 <= nfast; s += 2) {
-    fetch_fast(kbeg + (s + 1) * BK, st0);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(0);
-    stash(1, st0);
-    __syncthreads();
-    fetch_fast(kbeg + (s + 2) * BK, st0);
-    __builtin_amdgcn_sched_barrier(0);
-    compute(1);
+  if (STREAM && pos.cur_end <= pos.u0) return;  // (an XCD without tiles)
+  next_segment(c);
+  fetch_any(c, c.kbeg, st0);
+  for (;;) {
+#pragma unroll
+    for (int a = 0; a < MT; a++)
+#pragma unroll
+      for (int b = 0; b < NT; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+
+    // Slab s+1 travels global -> registers while slab s runs through the matrix
+    // cores, then goes to the other LDS buffer.  (A second slab in flight was
+    // measured and bought nothing.)  The main loop takes two slabs per trip, so
+    // that LDS buffer indices are compile-time constants, and contains
+    // descriptor fetches only; the few slabs it leaves over (and every slab of a
+    // workgroup that cannot use descriptors) run in the general loop below it.
+    const int kbeg = c.kbeg;
+    const int nslabs = (c.kend - kbeg + BK - 1) / BK;
+    const int nfull = (c.kend - kbeg) / BK;
+    const bool all_fast = a_fast && b_fast && !(IM2COL && !IM2COL_FAST);
+    const int nfast = all_fast ? nfull - 1 : 0;  // steps whose next slab is a full one
     stash(0, st0);
     __syncthreads();
-  }
-  for (; s < nslabs; s++) {
-    const int cur = s & 1;
-    if (s + 1 < nslabs) fetch_any(kbeg + (s + 1) * BK, st0);
-    compute(cur);
-    if (s + 1 < nslabs) stash(cur ^ 1, st0);
-    __syncthreads();
-  }
+    int s = 0;
+    // The scheduling fences keep the compiler from sinking the loads below the
+    // matrix-core work they are meant to overlap.
+    for (; s + 2 <= nfast; s += 2) {
+      fetch_fast(c, kbeg + (s + 1) * BK, st0);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(0);
+      stash(1, st0);
+      __syncthreads();
+      fetch_fast(c, kbeg + (s + 2) * BK, st0);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(1);
+      stash(0, st0);
+      __syncthreads();
+    }
+    for (; s < nslabs; s++) {
+      const int cur = s & 1;
+      if (s + 1 < nslabs) fetch_any(c, kbeg + (s + 1) * BK, st0);
+      compute(cur);
+      if (s + 1 < nslabs) stash(cur ^ 1, st0);
+      __syncthreads();
+    }
 
-  static_assert(2 * A_FLOATS >= 2 * STAGE_FLOATS && 2 * B_FLOATS >= 2 * STAGE_FLOATS, "epilogue staging");
-  if (STREAM && !sg.last) {
-    stream_hand_on<MT, NT>(p, acc);
-    continue;
-  }
-  if (STREAM && !sg.first) stream_collect<MT, NT>(p, pos, sg, acc);
-  finish_tile<BM, BN, WM, WN, CONV>(p, acc, whole, lin, chunk, bz, row0, col0,
-                                    (wave < 2 ? &lds_a[0][0] : &lds_b[0][0]) + (wave & 1) * STAGE_FLOATS);
+    // what the epilogue needs of this segment; c moves on to the next one, whose first slab
+    // is requested before the epilogue so that it travels while the results are stored
+    const bool whole = c.whole, first = c.first, last = c.last;
+    const int lin = c.lin, chunk = c.chunk, bz = c.bz, row0 = c.row0, col0 = c.col0;
+    Segment sg;
+    sg.tile_begin = c.tile_begin;
+    const bool more = STREAM && pos.cur_end > pos.u0;
+    if (more) {
+      next_segment(c);
+      fetch_any(c, c.kbeg, st0);
+    }
+    static_assert(2 * A_FLOATS >= 2 * STAGE_FLOATS && 2 * B_FLOATS >= 2 * STAGE_FLOATS, "epilogue staging");
+    if (STREAM && !last) {
+      stream_hand_on<MT, NT>(p, acc);
+    } else {
+      if (STREAM && !first) stream_collect<MT, NT>(p, pos, sg, acc);
+      finish_tile<BM, BN, WM, WN, CONV>(p, acc, whole, lin, chunk, bz, row0, col0,
+                                        (wave < 2 ? &lds_a[0][0] : &lds_b[0][0]) + (wave & 1) * STAGE_FLOATS);
+    }
+    if (!more) break;
+    __syncthreads();  // the epilogue has finished with the LDS
   }
 }
 
@@ -1251,122 +1287,135 @@ __global__ __launch_bounds__(NTHREADS, halo_blocks(BM, BN)) void conv3x3_halo_ke
   const int li = lane & 31, half = lane >> 5;
   const int wrow = wm * (MT * 32), wcol = wn * (NT * 32);
 
-  // (a stream launch walks the segments of this workgroup's range of K blocks: see stream_next)
-  StreamPos pos = {};
-  if (STREAM) pos = stream_begin(p);
-  for (bool again = false;; again = true) {
-  TileWork t;
-  int kbeg, kend;
-  Segment sg = {};
-  if (STREAM) {
-    if (pos.cur_end <= pos.u0) break;
-    if (again) __syncthreads();  // the previous segment's epilogue has finished with the LDS
-    sg = stream_next(p, pos);
-    t.whole = true;
-    t.lin = sg.lin;
-    t.chunk = 0;
-    t.bz = fdiv(t.lin, p.fd_tiles_per_z);
-    tile_coords(p, t.lin - t.bz * (p.tiles_m * p.tiles_n), &t.tm, &t.tn);
-    kbeg = sg.sbeg * HALO_KB;
-    kend = sg.send * HALO_KB < p.k ? sg.send * HALO_KB : p.k;
-  } else {
-    if (again) break;
-    t = decode_work(p);
-    kbeg = t.whole ? 0 : t.chunk * p.kchunk;
-    kend = t.whole ? p.k : (kbeg + p.kchunk < p.k ? kbeg + p.kchunk : p.k);
-  }
-  const int row0 = t.tm * BM, col0 = t.tn * BN;
-
   const ConvGeom &cv = p.cv;
   const int plane_in = cv.h * cv.w;
-  // first output row of the tile (rows numbered through the batch) and its image
-  const int R0 = fdiv(col0, cv.fd_ow);
-  const int img0 = fdiv(R0, cv.fd_oh);
+  const int pg = cv.pitch / VECW;       // pieces per row
+  const int upc = cv.slots * pg;        // pieces per channel
+  const int xu = cv.units;              // pieces per thread this geometry needs (<= XU)
 
   // ---- weights: piece (row r0 + 14 i, k 4q .. 4q+3) of the block -----------------
   // (threads 252..255 repeat pieces of row 13: same values to the same cells)
   const int q = tid % 18, r0 = tid / 18 < HALO_AROWS ? tid / 18 : HALO_AROWS - 1;
-  int voff_a[AU];
-#pragma unroll
-  for (int i = 0; i < AU; i++) {
-    int r = row0 + r0 + HALO_AROWS * i;
-    r = r < p.m ? r : p.m - 1;  // rows past the edge are never stored
-    voff_a[i] = (r * p.k + 4 * q) * 4;
-  }
   const int lds_a_w = (r0 * HALO_ROWA + 4 * q) * 4;
-  const rsrc_t rsrc_a = make_rsrc(p.A + (long long)t.bz * p.sAb, p.a_bytes);
-
-  // ---- input rows: piece u = tid + 256 i -> (channel, slot, column group) ---------
-  const int pg = cv.pitch / VECW;       // pieces per row
-  const int upc = cv.slots * pg;        // pieces per channel
-  const int first_rows = (img0 + 1) * cv.oh - R0;  // output rows from R0 to the end of its image
-  const int xu = cv.units;  // pieces per thread this geometry needs (<= XU)
-  int voff_x[XU], lds_x_w[XU];
-#pragma unroll
-  for (int i = 0; i < XU; i++) {
-    const int u = tid + NTHREADS * i;
-    const int c = fdiv(u, cv.fd_upc), rem = u - c * upc;
-    const int slot = fdiv(rem, cv.fd_pg), cg = rem - slot * pg;
-    // which input row the slot holds
-    int d, iy;
-    if (slot < first_rows + 2) {
-      d = 0;
-      iy = (R0 - img0 * cv.oh) - cv.pt + slot;
-    } else {
-      const int s2 = slot - first_rows - 2;
-      const int dd = fdiv(s2, cv.fd_oh2);
-      d = 1 + dd;
-      iy = s2 - dd * (cv.oh + 2) - cv.pt;
-    }
-    const int img = img0 + d;
-    const int ix = cg * VECW - cv.col0;
-    const bool live = c < HALO_CB;
-    const bool data = live && (long long)img * cv.oh * cv.ow < cv.npix && iy >= 0 && iy < cv.h &&
-                      ix >= 0 && ix + VECW <= cv.w;
-    voff_x[i] = data ? (((img * cv.c_total + c) * cv.h + iy) * cv.w + ix) * 4 : BUF_OOB;
-    lds_x_w[i] = live ? (c * PLANE + slot * cv.pitch + cg * VECW) * 4 : HALO_CB * PLANE * 4;
-  }
-  const long long group_off = (long long)t.bz * cv.c_in_g * plane_in;
-  const rsrc_t rsrc_x = make_rsrc(p.B + group_off, p.b_bytes - (int)(group_off * 4));
-
-  // ---- where a lane finds its operands in LDS -------------------------------------
+  // ---- where a lane finds its weights in LDS --------------------------------------
   int lds_a_r[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; mt++)
     lds_a_r[mt] = ((wrow + mt * 32 + li) * HALO_ROWA + 36 * half) * 4;
-  int lds_b_r[NT][9];
+
+  // What the loops need to know about one segment of work (a tile, a range of K blocks).
+  struct Ctx {
+    TileWork t;
+    bool first, last;
+    int tile_begin, row0, col0, kbeg, kend;
+    int voff_a[AU], voff_x[XU], lds_x_w[XU];
+    rsrc_t rsrc_a, rsrc_x;
+    int lds_b_r[NT][9];   // where a lane finds tap t of its pixel of block nt in LDS
+  };
+  // (a stream launch walks the segments of this workgroup's range of K blocks: see stream_next)
+  StreamPos pos = {};
+  if (STREAM) pos = stream_begin(p);
+  auto next_segment = [&](Ctx &c) {
+    TileWork &t = c.t;
+    if (STREAM) {
+      const Segment sg = stream_next(p, pos);
+      c.first = sg.first;
+      c.last = sg.last;
+      c.tile_begin = sg.tile_begin;
+      t.whole = true;
+      t.lin = sg.lin;
+      t.chunk = 0;
+      t.bz = fdiv(t.lin, p.fd_tiles_per_z);
+      tile_coords(p, t.lin - t.bz * (p.tiles_m * p.tiles_n), &t.tm, &t.tn);
+      c.kbeg = sg.sbeg * HALO_KB;
+      c.kend = sg.send * HALO_KB < p.k ? sg.send * HALO_KB : p.k;
+    } else {
+      t = decode_work(p);
+      c.first = c.last = true;
+      c.tile_begin = 0;
+      c.kbeg = t.whole ? 0 : t.chunk * p.kchunk;
+      c.kend = t.whole ? p.k : (c.kbeg + p.kchunk < p.k ? c.kbeg + p.kchunk : p.k);
+    }
+    const int row0 = c.row0 = t.tm * BM, col0 = c.col0 = t.tn * BN;
+    // first output row of the tile (rows numbered through the batch) and its image
+    const int R0 = fdiv(col0, cv.fd_ow);
+    const int img0 = fdiv(R0, cv.fd_oh);
 #pragma unroll
-  for (int nt = 0; nt < NT; nt++) {
-    int P = col0 + wcol + nt * 32 + li;
-    P = P < (int)cv.npix ? P : (int)cv.npix - 1;  // lanes past the edge are never stored
-    const int R = fdiv(P, cv.fd_ow), ox = P - R * cv.ow;
-    const int slot0 = (R - R0) + 2 * (fdiv(R, cv.fd_oh) - img0);
-    const int corner = (4 * half * PLANE + slot0 * cv.pitch + cv.col0 - cv.pl + ox) * 4;
+    for (int i = 0; i < AU; i++) {
+      int r = row0 + r0 + HALO_AROWS * i;
+      r = r < p.m ? r : p.m - 1;  // rows past the edge are never stored
+      c.voff_a[i] = (r * p.k + 4 * q) * 4;
+    }
+    c.rsrc_a = make_rsrc(p.A + (long long)t.bz * p.sAb, p.a_bytes);
+
+    // ---- input rows: piece u = tid + 256 i -> (channel, slot, column group) ---------
+    const int first_rows = (img0 + 1) * cv.oh - R0;  // output rows from R0 to the end of its image
 #pragma unroll
-    for (int tap = 0; tap < 9; tap++)
-      lds_b_r[nt][tap] = corner + ((tap / 3) * cv.pitch + tap % 3) * 4;
-  }
+    for (int i = 0; i < XU; i++) {
+      const int u = tid + NTHREADS * i;
+      const int ch = fdiv(u, cv.fd_upc), rem = u - ch * upc;
+      const int slot = fdiv(rem, cv.fd_pg), cg = rem - slot * pg;
+      // which input row the slot holds
+      int d, iy;
+      if (slot < first_rows + 2) {
+        d = 0;
+        iy = (R0 - img0 * cv.oh) - cv.pt + slot;
+      } else {
+        const int s2 = slot - first_rows - 2;
+        const int dd = fdiv(s2, cv.fd_oh2);
+        d = 1 + dd;
+        iy = s2 - dd * (cv.oh + 2) - cv.pt;
+      }
+      const int img = img0 + d;
+      const int ix = cg * VECW - cv.col0;
+      const bool live = ch < HALO_CB;
+      const bool data = live && (long long)img * cv.oh * cv.ow < cv.npix && iy >= 0 && iy < cv.h &&
+                        ix >= 0 && ix + VECW <= cv.w;
+      c.voff_x[i] = data ? (((img * cv.c_total + ch) * cv.h + iy) * cv.w + ix) * 4 : BUF_OOB;
+    }
+    const long long group_off = (long long)t.bz * cv.c_in_g * plane_in;
+    c.rsrc_x = make_rsrc(p.B + group_off, p.b_bytes - (int)(group_off * 4));
+  };
+  // The LDS side of a segment's plan: where the fetched pieces go and where a lane finds its
+  // taps.  Computed after the previous segment's epilogue (it is not needed to request the
+  // first block, and the epilogue needs the registers).
+  auto lds_plan = [&](Ctx &c) {
+    const int col0 = c.col0;
+    const int R0 = fdiv(col0, cv.fd_ow);
+    const int img0 = fdiv(R0, cv.fd_oh);
+#pragma unroll
+    for (int i = 0; i < XU; i++) {
+      const int u = tid + NTHREADS * i;
+      const int ch = fdiv(u, cv.fd_upc), rem = u - ch * upc;
+      const int slot = fdiv(rem, cv.fd_pg), cg = rem - slot * pg;
+      c.lds_x_w[i] = ch < HALO_CB ? (ch * PLANE + slot * cv.pitch + cg * VECW) * 4 : HALO_CB * PLANE * 4;
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++) {
+      int P = col0 + wcol + nt * 32 + li;
+      P = P < (int)cv.npix ? P : (int)cv.npix - 1;  // lanes past the edge are never stored
+      const int R = fdiv(P, cv.fd_ow), ox = P - R * cv.ow;
+      const int slot0 = (R - R0) + 2 * (fdiv(R, cv.fd_oh) - img0);
+      const int corner = (4 * half * PLANE + slot0 * cv.pitch + cv.col0 - cv.pl + ox) * 4;
+#pragma unroll
+      for (int tap = 0; tap < 9; tap++)
+        c.lds_b_r[nt][tap] = corner + ((tap / 3) * cv.pitch + tap % 3) * 4;
+    }
+  };
 
   f32x16 acc[MT][NT];
-#pragma unroll
-  for (int a = 0; a < MT; a++)
-#pragma unroll
-    for (int b = 0; b < NT; b++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
-
   f32x4 ra[AU];
   xpiece rx[XU];
-  auto fetch = [&](int k0) {
+  auto fetch = [&](const Ctx &c, int k0) {
     const int soff_a = k0 * 4;
     const int soff_x = (k0 / 9) * plane_in * 4;
 #pragma unroll
-    for (int i = 0; i < AU; i++) ra[i] = buf_load4(rsrc_a, voff_a[i], soff_a);
+    for (int i = 0; i < AU; i++) ra[i] = buf_load4(c.rsrc_a, c.voff_a[i], soff_a);
 #pragma unroll
     for (int i = 0; i < XU; i++)
-      if (i < xu) rx[i] = HaloPiece<VECW>::load(rsrc_x, voff_x[i], soff_x);
+      if (i < xu) rx[i] = HaloPiece<VECW>::load(c.rsrc_x, c.voff_x[i], soff_x);
   };
-  auto stash = [&]() {
+  auto stash = [&](const Ctx &c) {
     char *const as_b = reinterpret_cast<char *>(as);
     char *const xs_b = reinterpret_cast<char *>(xs);
 #pragma unroll
@@ -1374,9 +1423,9 @@ __global__ __launch_bounds__(NTHREADS, halo_blocks(BM, BN)) void conv3x3_halo_ke
       *reinterpret_cast<f32x4 *>(as_b + lds_a_w + i * (HALO_AROWS * HALO_ROWA * 4)) = ra[i];
 #pragma unroll
     for (int i = 0; i < XU; i++)
-      if (i < xu) *reinterpret_cast<xpiece *>(xs_b + lds_x_w[i]) = rx[i];
+      if (i < xu) *reinterpret_cast<xpiece *>(xs_b + c.lds_x_w[i]) = rx[i];
   };
-  auto compute = [&]() {
+  auto compute = [&](const Ctx &c) {
     const char *const as_b = reinterpret_cast<const char *>(as);
     const char *const xs_b = reinterpret_cast<const char *>(xs);
 #pragma unroll
@@ -1387,11 +1436,11 @@ __global__ __launch_bounds__(NTHREADS, halo_blocks(BM, BN)) void conv3x3_halo_ke
         av[mt] = *reinterpret_cast<const f32x4 *>(as_b + lds_a_r[mt] + 16 * j);
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        const int kk = 4 * j + e, c = kk / 9, tap = kk % 9;
+        const int kk = 4 * j + e, ch = kk / 9, tap = kk % 9;
         float b_el[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; nt++)
-          b_el[nt] = *reinterpret_cast<const float *>(xs_b + lds_b_r[nt][tap] + c * (PLANE * 4));
+          b_el[nt] = *reinterpret_cast<const float *>(xs_b + c.lds_b_r[nt][tap] + ch * (PLANE * 4));
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -1401,25 +1450,51 @@ __global__ __launch_bounds__(NTHREADS, halo_blocks(BM, BN)) void conv3x3_halo_ke
     }
   };
 
-  // One LDS buffer: block b+1 travels global -> registers while block b runs through
-  // the matrix cores, and is written to LDS once every wavefront has finished reading.
-  fetch(kbeg);
-  for (int k0 = kbeg; k0 < kend; k0 += HALO_KB) {
-    if (k0 != kbeg) __syncthreads();
-    stash();
-    __syncthreads();
-    if (k0 + HALO_KB < kend) fetch(k0 + HALO_KB);
-    __builtin_amdgcn_sched_barrier(0);
-    compute();
-  }
-  static_assert(AU * HALO_AROWS * HALO_ROWA >= 4 * STAGE_FLOATS, "epilogue staging");
-  if (STREAM && !sg.last) {
-    stream_hand_on<MT, NT>(p, acc);
-    continue;
-  }
-  if (STREAM && !sg.first) stream_collect<MT, NT>(p, pos, sg, acc);
-  finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0,
-                                    as + (threadIdx.x >> 6) * STAGE_FLOATS);
+  if (STREAM && pos.cur_end <= pos.u0) return;  // (an XCD without tiles)
+  Ctx c;
+  next_segment(c);
+  fetch(c, c.kbeg);
+  for (;;) {
+    lds_plan(c);
+#pragma unroll
+    for (int a = 0; a < MT; a++)
+#pragma unroll
+      for (int b = 0; b < NT; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+
+    // One LDS buffer: block b+1 travels global -> registers while block b runs through
+    // the matrix cores, and is written to LDS once every wavefront has finished reading.
+    for (int k0 = c.kbeg; k0 < c.kend; k0 += HALO_KB) {
+      if (k0 != c.kbeg) __syncthreads();
+      stash(c);
+      __syncthreads();
+      if (k0 + HALO_KB < c.kend) fetch(c, k0 + HALO_KB);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(c);
+    }
+    // what the epilogue needs of this segment; c moves on to the next one, whose first block
+    // is requested before the epilogue so that it travels while the results are stored
+    const TileWork t = c.t;
+    const bool first = c.first, last = c.last;
+    const int row0 = c.row0, col0 = c.col0;
+    Segment sg;
+    sg.tile_begin = c.tile_begin;
+    const bool more = STREAM && pos.cur_end > pos.u0;
+    if (more) {
+      next_segment(c);
+      fetch(c, c.kbeg);
+    }
+    static_assert(AU * HALO_AROWS * HALO_ROWA >= 4 * STAGE_FLOATS, "epilogue staging");
+    if (STREAM && !last) {
+      stream_hand_on<MT, NT>(p, acc);
+    } else {
+      if (STREAM && !first) stream_collect<MT, NT>(p, pos, sg, acc);
+      finish_tile<BM, BN, WM, WN, true>(p, acc, t.whole, t.lin, t.chunk, t.bz, row0, col0,
+                                        as + (threadIdx.x >> 6) * STAGE_FLOATS);
+    }
+    if (!more) break;
+    __syncthreads();  // the epilogue has finished with the LDS
   }
 }
 

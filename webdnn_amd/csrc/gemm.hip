@@ -233,11 +233,14 @@ int stream_width(long long tiles, int slabs, int kgran, const WorkPlan &w, int t
   if (!g_stream || g_forced_split >= 1 || !g_scratch_ptr[wdh::device()] || !g_stream_error_dev || tiles <= 0 || slabs <= 0) return 0;
   const long long cus = wdh::compute_units();
   if (g_stream == 1) {
-    // worth it when the plain plan would cut tiles across workgroups (a second launch to add
-    // them up) or would leave a good part of its last round of tiles idle
-    const double rounds = (double)tiles / (double)cus;
-    const double up = (double)((tiles + cus - 1) / cus);
-    if (w.tail == 0 && (rounds >= 8.0 || up / rounds < 1.04)) return 0;
+    // Measured on the ResNet-50 and DETR layer shapes: resident workgroups that walk segments
+    // lose to one short-lived workgroup per tile wherever the plain plan needs no cut (more
+    // wavefronts in flight hide the start and the end of a tile better than a longer-lived
+    // workgroup does), and they win where it would cut every tile of a launch that has at
+    // least a tile per CU (392 tiles of K 1024 or 2304: 45 -> 40 us, 83 -> 81 us): there the
+    // stream saves the reduce pass and evens out the 1.5 tiles per CU.  With fewer tiles than
+    // CUs each tile is shared by many workgroups and the chunk plan's parallel reduce wins.
+    if (!(w.tail == tiles && tiles >= cus)) return 0;
   }
   int per_cu = g_stream_wgs < max_wgs_per_cu ? g_stream_wgs : max_wgs_per_cu;
   if (per_cu < 1) per_cu = 1;
@@ -606,7 +609,7 @@ void release_conv_tables() {
 // The word a stream launch sets when one of its workgroups gave up waiting for a partial tile
 // lives in pinned host memory the device writes to directly, so the host can look at it after
 // any synchronisation without a copy.
-int init_contraction() {
+int init_contraction(int device) {
   if (g_stream_error) return WDH_OK;
   void *host = nullptr, *dev = nullptr;
   if (hipHostMalloc(&host, 64, hipHostMallocMapped) != hipSuccess ||
@@ -620,7 +623,7 @@ int init_contraction() {
   g_stream_error_dev = static_cast<unsigned *>(dev);
   // the flags of the static workspace start at zero and are left at zero by every launch; a
   // launch that was cut short (a failed run before a new wdh_init) may have left some raised
-  float *base = g_scratch_ptr[device()];
+  float *base = device >= 0 && device < kMaxDevices ? g_scratch_ptr[device] : nullptr;
   if (base && hipMemset(base + SK_PARTIAL_FLOATS, 0, (size_t)SK_FLAG_WORDS * 4) != hipSuccess) {
     (void)hipGetLastError();
     return fail(WDH_EHIP, "wdh_init: clearing the workspace flags");

@@ -214,7 +214,7 @@ static int init_device(int device) {
   WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
   int rc = wdh::init_static_scratch(device);
   if (rc == WDH_OK) rc = wdh::init_attention();
-  if (rc == WDH_OK) rc = wdh::init_contraction();
+  if (rc == WDH_OK) rc = wdh::init_contraction(device);
   return rc;
 }
 
