@@ -92,6 +92,10 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       batch strides of Y that are multiples of four) are turned through
  *                       LDS and stored 16 bytes per lane; 0 = every lane stores single
  *                       elements (same arithmetic, same bits).
+ *   "conv1x1_stride2_in_place"  1 (default) = an unpadded 1x1 convolution with a column stride of
+ *                       2 whose output rows hold an even number of pixels (input rows a multiple
+ *                       of four) reads X in place (16-byte pieces, every other element kept); 0 = it gathers its
+ *                       taps from global memory like every other strided geometry.
  *   "stream_k"          how wdh_gemm / wdh_conv2d launches whose tiles do not fill the chip in
  *                       whole rounds are scheduled: 1 (default) = such launches keep a fixed
  *                       grid of resident workgroups, each of which multiplies an equal,
@@ -131,6 +135,8 @@ int wdh_set_option(const char *name, int value);
 #define WDH_FORM_CONV3X3_LDS 6    /* 3x3 stride 1: taps read from an LDS tile   */
 #define WDH_FORM_CONV_STEM 7      /* 7x7 stride 2, 3 -> 64 channels: weights and the
                                    * input patch of an 8x16-pixel tile in LDS   */
+#define WDH_FORM_CONV_PIXELS_S2 8 /* 1x1 with column stride 2: X read in place,
+                                   * every other pixel of a row kept            */
 int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles,
                   int64_t *split_tiles, int *split, int *form);
 

@@ -1146,6 +1146,45 @@ def test_conv_1x1_in_place_with_a_ragged_last_tile(ctx, n, cin, h, w, cout, grou
     assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "ragged in-place 1x1 + residual + relu")
 
 
+@pytest.mark.parametrize("n,cin,h,w,cout,sh,group", [
+    (4, 256, 56, 56, 128, 2, 1),       # the stride-2 1x1 convs that open ResNet-50's stages 2 and 3
+    (4, 512, 28, 28, 1024, 2, 1),
+    (3, 32, 10, 24, 40, 2, 1),         # ragged last tile, rows of 12 output pixels
+    (3, 32, 12, 20, 40, 2, 1),         # rows of 10 output pixels: a thread's two pixel pairs lie in different rows
+    (2, 32, 9, 16, 24, 1, 1),          # column stride only
+    (2, 32, 13, 8, 24, 3, 2),          # row stride 3, two groups
+    (1, 16, 4, 8, 8, 2, 1),            # fewer pixels than a tile
+])
+def test_conv_1x1_column_stride_2_in_place(ctx, n, cin, h, w, cout, sh, group):
+    """An unpadded 1x1 conv with column stride 2 whose output rows hold an even number of pixels reads X
+    in place (two 16-byte pieces per four output pixels, every other element kept).  Against the oracle, and
+    bit for bit against the gathered form of the same geometry (the same products added in the same order)."""
+    X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin // group, 1), nrm(cout)
+    oh, ow = (h - 1) // sh + 1, (w - 1) // 2 + 1
+    R = nrm(n, cout, oh, ow)
+    got = hip_conv(ctx, X, W, B, None, group, None, [sh, 2], epilogue="relu", R=R)
+    assert ctx.last_plan()["form"] == "conv 1x1 stride 2, X in place", ctx.last_plan()
+    want = ref.unary("Relu", ref.binary("Add", ref.conv(X, W, B, None, group, None, None, [sh, 2]), R))
+    assert_close_max(got, want, GEMM_TOL, "1x1 column stride 2 in place")
+    try:
+        ctx.set_option("conv1x1_stride2_in_place", 0)
+        gathered = hip_conv(ctx, X, W, B, None, group, None, [sh, 2], epilogue="relu", R=R)
+        assert ctx.last_plan()["form"] == "conv, gathered taps"
+    finally:
+        ctx.set_option("conv1x1_stride2_in_place", 1)
+    assert_close_max(gathered, want, GEMM_TOL, "gathered")
+
+
+def test_conv_1x1_column_stride_2_falls_back_where_rows_do_not_fit(ctx):
+    """Output rows with an odd number of pixels (7 of 14), padding, or a column stride of 3: gathered."""
+    for shape, strides, pads in (((2, 64, 14, 14), [2, 2], None), ((2, 32, 16, 16), [2, 2], [1, 1, 1, 1]),
+                                 ((2, 32, 16, 24), [2, 3], None)):
+        X, W = uni(*shape, lo=0), he(24, shape[1], 1)
+        got = hip_conv(ctx, X, W, None, None, 1, pads, strides)
+        assert ctx.last_plan()["form"] == "conv, gathered taps", (shape, ctx.last_plan())
+        assert_close_max(got, ref.conv(X, W, None, None, 1, None, pads, strides), GEMM_TOL, "fallback %s" % (shape,))
+
+
 @pytest.mark.parametrize("batch,m,n,k,tb", [(1, 850, 256, 256, 0), (1, 850, 256, 2048, 0), (8, 850, 32, 850, 0),
                                             (1, 200, 1000, 256, 1), (3, 70, 45, 333, 1), (1, 100, 92, 256, 0),
                                             (8, 100, 100, 128, 1), (2, 33, 31, 500, 0)])

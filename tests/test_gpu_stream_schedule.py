@@ -101,7 +101,8 @@ CONVS = [
     (8, 1024, 14, 14, 256, 1, 1, 0, 1),     # 1x1 in place
     (8, 256, 14, 14, 1024, 1, 1, 0, 1),
     (4, 2048, 7, 7, 512, 1, 1, 0, 1),       # 7x7 planes
-    (4, 512, 28, 28, 256, 1, 2, 0, 1),      # stride-2 1x1: gathered
+    (4, 512, 28, 28, 256, 1, 2, 0, 1),      # stride-2 1x1: in place, every other pixel
+    (4, 512, 14, 14, 256, 1, 2, 0, 1),      # stride-2 1x1 onto 7x7 planes: gathered
     (2, 24, 17, 19, 40, 5, 2, 2, 1),        # gathered, 25 taps, ragged K
     (1, 16, 30, 30, 8, 7, 1, 3, 1),         # 49 taps
 ]
@@ -141,7 +142,7 @@ def test_any_number_of_resident_workgroups(stream_always, wgs):
 def test_stream_and_tile_per_workgroup_schedules_agree(ctx):
     """The default plan picks the stream schedule for the deep, small-plane layers; switched off, the
     same layers are cut into chunks with a reduce pass.  Two summation orders of the same products."""
-    X, W, B = uni(8, 256, 14, 14, lo=0.0), he(256, 256, 3), uni(256)
+    X, W, B = uni(32, 256, 14, 14, lo=0.0), he(256, 256, 3), uni(256)     # 392 tiles: more than one per CU
     want = ref.conv(X, W, B, pads=[1] * 4)
     try:
         outs = {}

@@ -121,7 +121,11 @@ constexpr int MC_PAD = 8;    // MC tile row stride = extent + 8 (floats)
 // h*w contiguous pixels per image, so it is fetched like B_MC (16-byte pieces)
 // with the image jump folded into each thread's column offset; the host picks it
 // only when every tile and K slab is whole (n % BN == 0, k % BK == 0, h*w % 4 == 0).
-enum BMode { B_KC = 0, B_MC = 1, B_IM2COL32 = 2, B_IM2COL64 = 3, B_IM2COL_BIG = 4, B_PIXELS = 5 };
+// B_PIXELS_S2: a 1x1 unpadded conv with column stride 2 (any row stride) whose output rows hold an
+// even number of pixels: two neighbouring output pixels are elements 0 and 2 of four consecutive
+// input floats, so a thread's four pixels arrive as two 16-byte pieces (each with its own offset:
+// the two pairs may lie in different rows) of which every other element is kept.
+enum BMode { B_KC = 0, B_MC = 1, B_IM2COL32 = 2, B_IM2COL64 = 3, B_IM2COL_BIG = 4, B_PIXELS = 5, B_PIXELS_S2 = 8 };
 
 struct ConvGeom {
   int c_in_g;        // input channels per group
@@ -882,7 +886,8 @@ template <int BM, int BN, int WM, int WN, bool A_KC, int BMODE_, bool VEC, bool 
 __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_blocks(BM, BN)) void contraction_kernel(Params p) {
   constexpr bool IM2COL_FAST = BMODE_ == B_IM2COL32 || BMODE_ == B_IM2COL64;
   constexpr bool IM2COL = IM2COL_FAST || BMODE_ == B_IM2COL_BIG;
-  constexpr bool PIXELS = BMODE_ == B_PIXELS;
+  constexpr bool PIX_S2 = BMODE_ == B_PIXELS_S2;
+  constexpr bool PIXELS = BMODE_ == B_PIXELS || PIX_S2;
   constexpr bool CONV = IM2COL || PIXELS;  // Y is NCHW, the bias is per row
   constexpr bool B_IS_KC = BMODE_ == B_KC;
   // layout of the B tile in LDS: tile[column][k] for a k-contiguous B and for the
@@ -913,6 +918,7 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
     const float *A, *B;
     long long lda, ldb;
     int voff_a[BM / 64], voff_b[BN / 64];
+    int voff_b2[BMODE_ == B_PIXELS_S2 ? BN / 64 : 1];  // B_PIXELS_S2: the piece of the second pixel pair
     rsrc_t rsrc_a, rsrc_b;
     PixelCtx px;
     PixelFast pf;
@@ -960,14 +966,28 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
       constexpr int TPR = BN / 4, RPP = NTHREADS / TPR;
       // B_PIXELS: column = pixel index over the batch; its four pixels share an image
       long long colpos = col0 + (tid % TPR) * 4;
-      if (PIXELS) {
+      long long colpos2 = 0;
+      if (PIX_S2) {
+        // output pixel -> (image, row, column) -> offset of its input pixel; pixels 0,1 and 2,3 of the
+        // thread's four are neighbours in a row (rows hold an even number of pixels)
+        const unsigned plane = (unsigned)(p.cv.h * p.cv.w), ohw = (unsigned)(p.cv.oh * p.cv.ow);
+        auto input_offset = [&](unsigned P) {
+          const unsigned img = (unsigned)fdiv((int)P, p.cv.fd_ohw), q = P - img * ohw;
+          const unsigned oy = (unsigned)fdiv((int)q, p.cv.fd_ow), ox = q - oy * (unsigned)p.cv.ow;
+          return (long long)img * p.cv.c_total * plane + (long long)oy * p.cv.sh * p.cv.w + 2 * ox;
+        };
+        colpos2 = input_offset((unsigned)colpos + 2);
+        colpos = input_offset((unsigned)colpos);
+      } else if (PIXELS) {
         const unsigned plane = (unsigned)(p.cv.h * p.cv.w);
         const unsigned img = (unsigned)fdiv((int)colpos, p.cv.fd_plane);
         colpos = (long long)img * p.cv.c_total * plane + ((unsigned)colpos - img * plane);
       }
 #pragma unroll
-      for (int i = 0; i < BN / 64; i++)
+      for (int i = 0; i < BN / 64; i++) {
         c.voff_b[i] = (int)(((long long)(tid / TPR + i * RPP) * ldb + colpos) * 4);
+        if (PIX_S2) c.voff_b2[PIX_S2 ? i : 0] = (int)(((long long)(tid / TPR + i * RPP) * ldb + colpos2) * 4);
+      }
     }
     c.rsrc_a = make_rsrc(c.A, p.a_bytes);
 
@@ -1049,7 +1069,17 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
   // Registers that carry one fetched K slab from global memory to LDS.
   struct Staged {
     f32x4 a[BM / 64], b[BN / 64];
+    f32x4 b2[PIX_S2 ? BN / 64 : 1];  // B_PIXELS_S2: the second 16 bytes of each piece
     unsigned ok;  // flat im2col only: which fetched taps lie inside the input
+  };
+  // B_PIXELS_S2: two pieces of four consecutive input floats, of which elements 0 and 2 are pixels
+  auto fetch_b_s2 = [&](const Ctx &c, int k0, Staged &st) {
+    const int soff = (int)(k0 * c.ldb * 4);
+#pragma unroll
+    for (int i = 0; i < BN / 64; i++) {
+      st.b[i] = buf_load4(c.rsrc_b, c.voff_b[i], soff);
+      st.b2[PIX_S2 ? i : 0] = buf_load4(c.rsrc_b, c.voff_b2[PIX_S2 ? i : 0], soff);
+    }
   };
   // Descriptor-only fetch: legal for a slab that lies fully inside K when
   // both operands qualify (all_fast).
@@ -1057,6 +1087,8 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
     fetch_rows_fast<BM, VEC>(c.rsrc_a, c.voff_a, A_KC ? k0 * 4 : (int)(k0 * c.lda * 4), st.a);
     if (IM2COL_FAST)
       fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(c.rsrc_b, p.cv.ktab, c.pf, k0 + c.kgroup0, st.b);
+    else if (PIX_S2)
+      fetch_b_s2(c, k0, st);
     else if (!IM2COL)
       fetch_rows_fast<BN, VEC>(c.rsrc_b, c.voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * c.ldb * 4), st.b);
   };
@@ -1075,6 +1107,8 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
       fetch_im2col_fast<BN, BMODE_ == B_IM2COL64>(c.rsrc_b, p.cv.ktab, c.pf, k0 + c.kgroup0, st.b);
     } else if (IM2COL) {
       st.ok = fetch_im2col<BN>(p.cv, c.px, k0, c.kend, tid, st.b);
+    } else if (PIX_S2) {
+      fetch_b_s2(c, k0, st);
     } else if ((b_fast && full) || PIXELS) {
       fetch_rows_fast<BN, VEC>(c.rsrc_b, c.voff_b, B_IS_KC ? k0 * 4 : (int)(k0 * c.ldb * 4), st.b);
     } else if (B_IS_KC) {
@@ -1094,7 +1128,13 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
       stash_im2col_fast<BN>(lds_b[buf], tid, st.b);
     else if (IM2COL)
       stash_im2col<BN>(lds_b[buf], tid, st.b, st.ok);
-    else
+    else if (PIX_S2) {
+      f32x4 even[BN / 64];
+#pragma unroll
+      for (int i = 0; i < BN / 64; i++)
+        even[i] = f32x4{st.b[i].x, st.b[i].z, st.b2[PIX_S2 ? i : 0].x, st.b2[PIX_S2 ? i : 0].z};
+      stash_mc<BN>(lds_b[buf], tid, even);
+    } else
       stash_mc<BN>(lds_b[buf], tid, st.b);
   };
 
@@ -1852,7 +1892,7 @@ int launch(Params &p, int nz, bool vec) {
 int launch_gemm_a_kc(bool b_kc, Params &p, int nz, bool vec);     // contraction_gemm_akc.hip
 int launch_gemm_a_mc(bool b_kc, Params &p, int nz, bool vec);     // contraction_gemm_amc.hip
 int launch_conv_gather(int mode, Params &p, int nz, bool vec);    // contraction_conv_gather.hip
-int launch_conv_pixels(Params &p, int nz, bool vec);              // contraction_conv_pixels.hip
+int launch_conv_pixels(Params &p, int nz, bool vec, bool stride2);  // contraction_conv_pixels.hip
 int launch_conv3x3(int tile, Params &p, int nz, int vecw);        // contraction_conv3x3.hip
 
 }  // namespace wdhc

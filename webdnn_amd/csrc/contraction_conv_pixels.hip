@@ -3,6 +3,8 @@
 #include "contraction.h"
 
 namespace wdhc {
-// 1x1 stride-1 Conv reading X in place
-int launch_conv_pixels(Params &p, int nz, bool vec) { return launch<true, B_PIXELS>(p, nz, vec); }
+// 1x1 unpadded Conv reading X in place: every pixel (stride 1), or every other pixel of a row
+int launch_conv_pixels(Params &p, int nz, bool vec, bool stride2) {
+  return stride2 ? launch<true, B_PIXELS_S2>(p, nz, vec) : launch<true, B_PIXELS>(p, nz, vec);
+}
 }  // namespace wdhc

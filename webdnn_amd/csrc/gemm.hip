@@ -130,6 +130,7 @@ struct GroupQueue {
   int variant[16];  // 2 * B_IS_KC + VEC
 } g_group;
 int g_stem = 1;           // 0: the 7x7 stride-2 stem conv gathers its taps like any other geometry
+int g_pixels_s2 = 1;      // 0: 1x1 convs with a column stride of 2 gather their taps like any other geometry
 int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
 int g_stream = 1;         // launches scheduled as streams of K slabs: 0 never, 1 where the plan below gains, 2 wherever legal
 int g_stream_wgs = 4;     // workgroups per CU of a stream launch (at most what the kernel's resources allow)
@@ -322,6 +323,12 @@ extern "C" int wdh_set_option(const char *name, int value) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: conv_stem %d (use 0 or 1)", value);
     g_stem = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "conv1x1_stride2_in_place") == 0) {
+    if (value != 0 && value != 1)
+      return fail(WDH_EINVAL, "wdh_set_option: conv1x1_stride2_in_place %d (use 0 or 1)", value);
+    g_pixels_s2 = value;
     return WDH_OK;
   }
   if (strcmp(name, "stream_k") == 0) {
@@ -720,14 +727,21 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   // over the end of the pixels: its surplus columns read the next k row or, past the last
   // image, the zeros the descriptor returns, and are never stored.
   const long long plane = (long long)h * w;
-  if (small && vec && ntaps == 1 && sh == 1 && sw == 1 && pt == 0 && pl == 0 && pb == 0 && pr == 0 &&
-      plane % 4 == 0 && kdim % BK == 0 && aligned16(p.B)) {
+  // The same with a column stride of 2 (the stride-2 1x1 convs that open a ResNet stage), when output
+  // rows hold an even number of pixels: two neighbouring output pixels are elements 0 and 2 of four
+  // consecutive input floats (B_PIXELS_S2).
+  const bool unpadded_1x1 = small && vec && ntaps == 1 && pt == 0 && pl == 0 && pb == 0 && pr == 0 &&
+                            plane % 4 == 0 && kdim % BK == 0 && aligned16(p.B);
+  const bool in_place = unpadded_1x1 && sh == 1 && sw == 1;
+  const bool in_place_s2 = unpadded_1x1 && g_pixels_s2 && sw == 2 && ow % 2 == 0 && ((long long)sh * w) % 4 == 0 && w % 4 == 0;
+  if (in_place || in_place_s2) {
     p.m = cout_g; p.n = (int)npix; p.k = (int)kdim;
     p.sAb = (long long)cout_g * kdim; p.sA0 = kdim; p.sA1 = 1;
     p.sBb = (long long)c_in_g * plane; p.sB0 = plane; p.sB1 = 1;
     p.alpha = 1.0f; p.beta = 1.0f; p.epilogue = epilogue;
     p.cv.c_in_g = c_in_g; p.cv.h = h; p.cv.w = w; p.cv.oh = oh; p.cv.ow = ow;
-    p.cv.sh = p.cv.sw = p.cv.kh = p.cv.kw = p.cv.dh = p.cv.dw = 1;
+    p.cv.sh = sh; p.cv.sw = sw;
+    p.cv.kh = p.cv.kw = p.cv.dh = p.cv.dw = 1;
     p.cv.c_total = c; p.cv.cout_total = cout; p.cv.cout_g = cout_g;
     p.cv.ntaps = 1; p.cv.npix = npix;
     p.fast = 1;
@@ -736,7 +750,7 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.y_bytes = g_descriptors && out_bytes < 0x7fffffffULL ? (int)out_bytes : 0;
     p.c_bytes = cout * 4;
     set_wide(p, true);
-    return launch_conv_pixels(p, group, true);
+    return launch_conv_pixels(p, group, true, in_place_s2);
   }
   // 3x3, stride 1, no dilation, input channels in blocks of 8: taps read from an input
   // tile staged in LDS (conv3x3_halo_kernel)
