@@ -57,6 +57,7 @@
 #pragma once
 #include <string.h>
 
+
 #include "common.h"
 #include "fastdiv.h"
 
@@ -1197,7 +1198,9 @@ __global__ __launch_bounds__(NTHREADS, STREAM ? stream_blocks(BM, BN) : min_bloc
     // measured and bought nothing.)  The main loop takes two slabs per trip, so
     // that LDS buffer indices are compile-time constants, and contains
     // descriptor fetches only; the few slabs it leaves over (and every slab of a
-    // workgroup that cannot use descriptors) run in the general loop below it.
+    // workgroup that cannot use descriptors) run in the general loop below it.  (Two slabs
+    // in flight, requested two trips ahead, were measured again on the ResNet-50 layers, same box,
+    // alternating builds: 2966 against 2957 us over the 54 launches -- nothing.)
     const int kbeg = c.kbeg;
     const int nslabs = (c.kend - kbeg + BK - 1) / BK;
     const int nfull = (c.kend - kbeg) / BK;

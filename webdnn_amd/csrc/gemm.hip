@@ -237,11 +237,13 @@ int stream_width(long long tiles, int slabs, int kgran, const WorkPlan &w, int t
     // Measured on the ResNet-50 and DETR layer shapes: resident workgroups that walk segments
     // lose to one short-lived workgroup per tile wherever the plain plan needs no cut (more
     // wavefronts in flight hide the start and the end of a tile better than a longer-lived
-    // workgroup does), and they win where it would cut every tile of a launch that has at
-    // least a tile per CU (392 tiles of K 1024 or 2304: 45 -> 40 us, 83 -> 81 us): there the
-    // stream saves the reduce pass and evens out the 1.5 tiles per CU.  With fewer tiles than
-    // CUs each tile is shared by many workgroups and the chunk plan's parallel reduce wins.
-    if (!(w.tail == tiles && tiles >= cus)) return 0;
+    // workgroup does), and they win for 1x1 convs that read X in place where the plain plan
+    // would cut every tile of a launch that has at least a tile per CU (392 tiles of K 1024:
+    // 45 -> 40 us; 850 tiles of K 256 on a 50x68 plane: 31 -> 27 us): there the stream saves
+    // the reduce pass and evens out the 1.5 tiles per CU.  With fewer tiles than CUs each tile
+    // is shared by many workgroups and the chunk plan's parallel reduce wins; 3x3 convs gain 2 %
+    // on ResNet-50's 14x14 planes and lose 8-10 % on DETR's 100x136 and 25x34 planes.
+    if (!(w.tail == tiles && tiles >= cus && (g_last_form == B_PIXELS || g_last_form == B_PIXELS_S2))) return 0;
   }
   int per_cu = g_stream_wgs < max_wgs_per_cu ? g_stream_wgs : max_wgs_per_cu;
   if (per_cu < 1) per_cu = 1;

@@ -20,6 +20,10 @@
 namespace {
 
 constexpr size_t kStagingBytes = 32u << 20;  // per pinned buffer, two of them
+// Uploads go through the staging buffers in pieces of kUploadPiece, each with an event of its
+// own, so that the host's copy of piece i+1 into pinned memory overlaps the DMA of piece i.
+constexpr size_t kUploadPiece = 4u << 20;
+constexpr int kUploadSlots = (int)(2 * kStagingBytes / kUploadPiece);
 constexpr size_t kSmallGranule = 512;        // allocation rounding below 1 MiB
 constexpr size_t kLargeGranule = 1u << 20;   // and above
 
@@ -56,8 +60,10 @@ struct Runtime {
   uint64_t in_use = 0, cached = 0, reserved = 0, peak = 0;
   // pinned staging, ping-pong
   void *stage[2] = {nullptr, nullptr};
-  hipEvent_t stage_done[2] = {nullptr, nullptr};
-  bool stage_busy[2] = {false, false};
+  hipEvent_t stage_done[2] = {nullptr, nullptr};   // downloads: one event per buffer
+  hipEvent_t up_done[kUploadSlots] = {};            // uploads: one event per piece
+  bool up_busy[kUploadSlots] = {};
+  int up_next = 0;
   // timing events, created lazily
   hipEvent_t events[WDH_MAX_EVENTS] = {};
   // one-element dummy so that zero-byte buffers have a valid address
@@ -209,8 +215,12 @@ static int init_device(int device) {
       return fail(WDH_ENOMEM, "wdh_init: pinned staging allocation failed");
     WDH_HIP_CHECK(
         hipEventCreateWithFlags(&g.stage_done[i], hipEventDisableTiming));
-    g.stage_busy[i] = false;
   }
+  for (int i = 0; i < kUploadSlots; i++) {
+    WDH_HIP_CHECK(hipEventCreateWithFlags(&g.up_done[i], hipEventDisableTiming));
+    g.up_busy[i] = false;
+  }
+  g.up_next = 0;
   WDH_HIP_CHECK(hipMalloc(&g.dummy, 256));
   int rc = wdh::init_static_scratch(device);
   if (rc == WDH_OK) rc = wdh::init_attention();
@@ -272,6 +282,11 @@ static void release_everything() {
     if (g.stage_done[i]) (void)hipEventDestroy(g.stage_done[i]);
     g.stage[i] = nullptr;
     g.stage_done[i] = nullptr;
+  }
+  for (int i = 0; i < kUploadSlots; i++) {
+    if (g.up_done[i]) (void)hipEventDestroy(g.up_done[i]);
+    g.up_done[i] = nullptr;
+    g.up_busy[i] = false;
   }
   for (auto &ev : g.events) {
     if (ev) (void)hipEventDestroy(ev);
@@ -393,14 +408,20 @@ int wdh_free(wdh_buf h) {
     }                                                                             \
   } while (0)
 
+// Blocks until no upload piece is still on its way out of the staging buffers.
+static int wait_for_uploads() {
+  for (int i = 0; i < kUploadSlots; i++)
+    if (g.up_busy[i]) {
+      WDH_HIP_CHECK(hipEventSynchronize(g.up_done[i]));
+      g.up_busy[i] = false;
+    }
+  return WDH_OK;
+}
+
 int wdh_graph_begin(void) {
   WDH_REQUIRE_INIT();
   if (g.capturing) return fail(WDH_ESTATE, "wdh_graph_begin: a capture is already open");
-  for (int i = 0; i < 2; i++)
-    if (g.stage_busy[i]) {
-      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[i]));
-      g.stage_busy[i] = false;
-    }
+  if (int rc = wait_for_uploads()) return rc;
   int id = -1;
   for (size_t i = 0; i < g.graphs.size(); i++)
     if (!g.graphs[i].live) id = (int)i;
@@ -471,20 +492,21 @@ int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
   if (bytes && !src) return fail(WDH_EINVAL, "wdh_write: src is NULL");
   const char *s = (const char *)src;
   size_t done = 0;
-  int which = 0;
   while (done < bytes) {
-    size_t chunk = bytes - done < kStagingBytes ? bytes - done : kStagingBytes;
-    if (g.stage_busy[which]) {
-      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[which]));
-      g.stage_busy[which] = false;
+    const size_t chunk = bytes - done < kUploadPiece ? bytes - done : kUploadPiece;
+    const int slot = g.up_next;
+    g.up_next = (g.up_next + 1) % kUploadSlots;
+    if (g.up_busy[slot]) {
+      WDH_HIP_CHECK(hipEventSynchronize(g.up_done[slot]));
+      g.up_busy[slot] = false;
     }
-    memcpy(g.stage[which], s + done, chunk);
-    WDH_HIP_CHECK(hipMemcpyAsync(dst + dst_offset + done, g.stage[which], chunk,
-                                 hipMemcpyHostToDevice, g.stream));
-    WDH_HIP_CHECK(hipEventRecord(g.stage_done[which], g.stream));
-    g.stage_busy[which] = true;
+    const size_t per_buffer = kStagingBytes / kUploadPiece;
+    char *piece = (char *)g.stage[slot / per_buffer] + (slot % per_buffer) * kUploadPiece;
+    memcpy(piece, s + done, chunk);
+    WDH_HIP_CHECK(hipMemcpyAsync(dst + dst_offset + done, piece, chunk, hipMemcpyHostToDevice, g.stream));
+    WDH_HIP_CHECK(hipEventRecord(g.up_done[slot], g.stream));
+    g.up_busy[slot] = true;
     done += chunk;
-    which ^= 1;
   }
   return WDH_OK;
 }
@@ -500,11 +522,7 @@ int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
                 bytes, src_offset, have);
   if (bytes && !dst) return fail(WDH_EINVAL, "wdh_read: dst is NULL");
   // staging buffers may still carry an in-flight upload
-  for (int i = 0; i < 2; i++)
-    if (g.stage_busy[i]) {
-      WDH_HIP_CHECK(hipEventSynchronize(g.stage_done[i]));
-      g.stage_busy[i] = false;
-    }
+  if (int rc = wait_for_uploads()) return rc;
   char *d = (char *)dst;
   size_t issued = 0, copied = 0;
   size_t chunk_of[2] = {0, 0};
