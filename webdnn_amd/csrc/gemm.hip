@@ -288,6 +288,16 @@ long long span(long long nb, long long sb, long long n0, long long s0,
 
 using wdh::fail;
 
+// Whether a product is one for gemm_wavesplit_kernel: few result blocks and a K worth cutting.
+static bool wavesplit_suits(int batch, int m, int n, int k) {
+  if (!g_wavesplit || g_forced_tile >= 0 || g_forced_split >= 0 || k < 128) return false;
+  const long long blocks32 = (long long)((m + 31) / 32) * ((n + 31) / 32) * batch;
+  const long long tiles64 = (long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
+  // (few blocks each streaming a long K would leave the weights to a handful of CUs)
+  return blocks32 <= 4LL * wdh::compute_units() && tiles64 < 2LL * wdh::compute_units() &&
+         (blocks32 * 2 >= wdh::compute_units() || k <= 512);
+}
+
 extern "C" int wdh_set_option(const char *name, int value) {
   if (!name) return fail(WDH_EINVAL, "wdh_set_option: name is NULL");
   if (strcmp(name, "contraction_tile") == 0) {
@@ -491,13 +501,9 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
   }
   // Few result tiles and a K worth cutting: one launch with K cut across the wavefronts of a
   // workgroup (gemm_wavesplit_kernel) instead of chunks in a workspace and a reduce pass
-  if (g_wavesplit && g_forced_tile < 0 && g_forced_split < 0 && useA_kc && p.fast && k >= 128) {
+  if (useA_kc && p.fast && wavesplit_suits(batch, m, n, k)) {
     const long long blocks32 = (long long)((m + 31) / 32) * ((n + 31) / 32) * batch;
-    const long long tiles64 = (long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
-    // (few blocks each streaming a long K would leave the weights to a handful of CUs)
-    if (blocks32 <= 4LL * wdh::compute_units() && tiles64 < 2LL * wdh::compute_units() &&
-        (blocks32 * 2 >= wdh::compute_units() || k <= 512) &&
-        (useB_kc || (long long)(k - 1) * p.sB0 * 4 < 0x7fffffffLL)) {
+    if (useB_kc || (long long)(k - 1) * p.sB0 * 4 < 0x7fffffffLL) {
       p.tiles_m = (m + 31) / 32;
       p.tiles_n = (n + 31) / 32;
       p.nz = batch;
