@@ -328,12 +328,13 @@ def bench_resnet_layers(steps, warmup, batch=32, only=None):
             X = ctx.move_tensor(rng.uniform(0, 1, x).astype(np.float32))
             W = ctx.move_tensor((rng.standard_normal(w) * np.sqrt(2.0 / (w[1] * w[2] * w[3]))).astype(np.float32))
             B = ctx.move_tensor(np.zeros(w[0], np.float32))
-            probe = H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu")
+            # (constant_weights: what the runner passes for an initializer's device copy)
+            probe = H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu", constant_weights=True)
             plan, odims = ctx.last_plan(), probe.dims
             R = ctx.move_tensor(rng.uniform(0, 1, odims).astype(np.float32)) if residual else None
             probe.dispose()
             ms = timed_steps(ctx, lambda: H.conv(ctx, X, W, B, pads=list(pads), strides=list(strides), epilogue="relu",
-                                                 residual=R).dispose(), steps, warmup)
+                                                 residual=R, constant_weights=True).dispose(), steps, warmup)
             m, n, k = w[0], odims[0] * odims[2] * odims[3], w[1] * w[2] * w[3]
             out_elems = int(np.prod(odims))
             nbytes = 4 * (int(np.prod(x)) + int(np.prod(w)) + w[0] + out_elems * (2 if residual else 1))

@@ -78,6 +78,13 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *                       input rows of a tile in LDS and read the taps from there;
  *                       0 = they gather taps from global memory like every other
  *                       geometry (both forms compute the same sums).
+ *   "conv3x3_winograd"  how 3x3, stride-1, undilated, ungrouped convolutions whose channel count is a
+ *                       multiple of 16 are computed: 1 (default) = those with at least 128 input and
+ *                       128 output channels by the minimal-filtering algorithm F(2x2, 3x3) (filters
+ *                       and 4x4 input patches transformed, 16 batched matrix products with 4/9 of the
+ *                       multiplications, results transformed back under the epilogue); 2 = all of
+ *                       them; 0 = none (the direct forms below).  Not the direct form's sums: results
+ *                       agree within the Gemm/Conv tolerance, not bit for bit.
  *   "conv_stem"         1 (default) = a 7x7, stride-2, undilated convolution from 3 to 64
  *                       channels (the stem of an image network) runs in a kernel that keeps
  *                       all weights and a tile's input patch in LDS; 0 = it gathers taps
@@ -137,6 +144,8 @@ int wdh_set_option(const char *name, int value);
                                    * input patch of an 8x16-pixel tile in LDS   */
 #define WDH_FORM_CONV_PIXELS_S2 8 /* 1x1 with column stride 2: X read in place,
                                    * every other pixel of a row kept            */
+#define WDH_FORM_CONV3X3_WINOGRAD 9 /* 3x3 stride 1 as F(2x2, 3x3): transforms around a
+                                   * batched product (tile and split are the product's) */
 int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles,
                   int64_t *split_tiles, int *split, int *form);
 
@@ -277,6 +286,17 @@ int wdh_conv2d(wdh_buf X, wdh_buf W, wdh_buf Bias, wdh_buf Y, int n, int c,
                int h, int w, int cout, int kh, int kw, int pt, int pl, int pb,
                int pr, int sh, int sw, int dh, int dw, int group, int epilogue,
                wdh_buf R);
+/* wdh_conv2d with promises about the operands.  WDH_CONV_CONSTANT_WEIGHTS: nobody writes to W
+ * while its handle lives -- what holds for the device copy of an initializer, which the runner
+ * uploads once and keeps across runs (copiedInitializerTensors, core/runnerImpl.ts:323-351).
+ * The library may then keep data derived from W (the transformed filters of the F(2x2, 3x3)
+ * form) from one call to the next; it is dropped when W is freed, written to through wdh_write
+ * or wdh_copy, or at wdh_shutdown.  Results are those of wdh_conv2d. */
+#define WDH_CONV_CONSTANT_WEIGHTS 1
+int wdh_conv2d_ex(wdh_buf X, wdh_buf W, wdh_buf Bias, wdh_buf Y, int n, int c,
+                  int h, int w, int cout, int kh, int kw, int pt, int pl, int pb,
+                  int pr, int sh, int sw, int dh, int dw, int group, int epilogue,
+                  wdh_buf R, int flags);
 
 /* ---- elementwise -------------------------------------------------------
  * Replaces Binary7 (operators/cpu/operators/standard/binary7.ts:16-68) and

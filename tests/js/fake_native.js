@@ -136,6 +136,12 @@ const native = {
     }
   },
 
+  // (flags: promises about the operands that let the library keep derived data; nothing to do here)
+  conv2dEx(X, W, Bias, Y, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epi, R, flags) {
+    if (flags !== 0 && flags !== 1) throw new Error("wdh_conv2d_ex failed (-2): unknown flags");
+    return this.conv2d(X, W, Bias, Y, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epi, R);
+  },
+
   conv2d(X, W, Bias, Y, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epi, R) {
     count("conv2d");
     if (c % group || cout % group) throw new Error("wdh_conv2d failed (-2): channels not divisible by group");
@@ -356,7 +362,7 @@ const native = {
 // Like the library: between graphBegin and graphEnd compute calls are recorded, not executed;
 // alloc/free work, but a buffer freed meanwhile keeps its storage for the graph's lifetime;
 // calls that need device data on the host throw and spoil the capture.
-const RECORDED = ["copy", "gemm", "gemmEx", "linearGroup", "conv2d", "binary", "unary", "softmax", "attention", "layernorm", "layernormAdd", "reduceMean", "reduceAxis", "maxpool2d",
+const RECORDED = ["copy", "gemm", "gemmEx", "linearGroup", "conv2d", "conv2dEx", "binary", "unary", "softmax", "attention", "layernorm", "layernormAdd", "reduceMean", "reduceAxis", "maxpool2d",
   "globalAvgpool", "transpose", "gather", "cast", "stridedCopy"];
 const REFUSED = ["write", "read", "sync", "trim", "eventRecord", "eventElapsedMs"];
 const graphs = new Map();

@@ -1146,6 +1146,98 @@ def test_conv_1x1_in_place_with_a_ragged_last_tile(ctx, n, cin, h, w, cout, grou
     assert_bit_exact(fused, np.maximum(got + R, 0) + 0.0, "ragged in-place 1x1 + residual + relu")
 
 
+WINOGRAD_CONVS = [
+    # n, cin, h, w, cout, pads
+    (32, 256, 14, 14, 256, [1, 1, 1, 1]),     # ResNet-50 stage 3
+    (8, 512, 7, 7, 512, [1, 1, 1, 1]),        # odd output planes: the last 2x2 block of a row and column is half empty
+    (4, 128, 28, 28, 128, [1, 1, 1, 1]),
+    (1, 128, 25, 34, 160, [1, 1, 1, 1]),      # a DETR plane
+    (2, 32, 9, 11, 48, [1, 1, 1, 1]),         # below the channel count the plan picks by itself
+    (2, 16, 8, 8, 16, [0, 0, 0, 0]),          # no padding
+    (3, 48, 10, 7, 16, [2, 0, 1, 2]),         # unequal pads, wider than the filter's reach on one side
+    (1, 16, 3, 3, 32, [1, 1, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("shape", WINOGRAD_CONVS)
+def test_conv3x3_by_minimal_filtering(ctx, shape):
+    """3x3 stride-1 convs as F(2x2, 3x3): transformed filters and input patches, 16 batched products, results
+    transformed back under bias + residual + Relu.  Not the direct form's sums, so the bar is the Gemm/Conv
+    tolerance against the oracle -- for the forced form, for what the plan picks, and with the filters kept
+    from a first call (WDH_CONV_CONSTANT_WEIGHTS)."""
+    n, cin, h, w, cout, pads = shape
+    X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin, 3), nrm(cout)
+    want0 = ref.conv(X, W, B, pads=pads)
+    R = nrm(*want0.shape)
+    want = ref.unary("Relu", ref.binary("Add", want0, R))
+    try:
+        ctx.set_option("conv3x3_winograd", 2)
+        got = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+        assert ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)"), ctx.last_plan()
+        assert_close_max(got, want, GEMM_TOL, "F(2x2,3x3) %s" % (shape,))
+        assert_close_max(hip_conv(ctx, X, W, None, pads=pads), ref.conv(X, W, None, pads=pads), GEMM_TOL, "no bias")
+        # filters kept across calls: same bits as computing them every time; other weights in the same
+        # buffer (wdh_write) or in a new buffer are seen
+        tx, tw, tb, tr = (ctx.move_tensor(v) for v in (X, W, B, R))
+        kept = [H.conv(ctx, tx, tw, tb, pads=pads, epilogue="relu", residual=tr, constant_weights=True).get_data()
+                for _ in range(3)]
+        for k in kept:
+            assert_bit_exact(k, got, "kept filters")
+        W2 = he(cout, cin, 3)
+        capi.call("wdh_write", tw.handle, 0, W2.ctypes.data, W2.nbytes)
+        want2 = ref.unary("Relu", ref.binary("Add", ref.conv(X, W2, B, pads=pads), R))
+        again = H.conv(ctx, tx, tw, tb, pads=pads, epilogue="relu", residual=tr, constant_weights=True).get_data()
+        assert_close_max(again, want2, GEMM_TOL, "weights rewritten in place")
+        for t in (tx, tw, tb, tr):
+            t.dispose()
+    finally:
+        ctx.set_option("conv3x3_winograd", 1)
+    auto = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+    assert_close_max(auto, want, GEMM_TOL, "the plan's own choice %s" % (ctx.last_plan()["form"],))
+    picked = ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
+    assert picked == (cin >= 128 and cout >= 128), ctx.last_plan()
+    try:
+        ctx.set_option("conv3x3_winograd", 0)
+        direct = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+        assert not ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
+        assert_close_max(direct, want, GEMM_TOL, "direct form")
+    finally:
+        ctx.set_option("conv3x3_winograd", 1)
+
+
+def test_conv3x3_minimal_filtering_keeps_special_values_local_and_replays(ctx):
+    """An Inf in the input reaches only the outputs whose receptive field holds it... in the transform domain
+    it meets finite values of its 4x4 patch, so the 2x2 block it belongs to may turn NaN, never a block further
+    away; and the form replays from a captured graph with kept filters."""
+    X, W, B = uni(2, 128, 12, 12, lo=0), he(128, 128, 3), nrm(128)
+    X[1, 5, 6, 6] = np.inf
+    got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])
+    assert ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
+    bad = ~np.isfinite(got)
+    assert not bad[0].any(), "the other image is untouched"
+    ys, xs = np.nonzero(bad[1].any(axis=0))
+    assert ys.min() >= 4 and ys.max() <= 9 and xs.min() >= 4 and xs.max() <= 9, (ys, xs)
+    Xc = np.where(np.isfinite(X), X, 0).astype(np.float32)
+    tx, tw, tb = (ctx.move_tensor(v) for v in (Xc, W, B))
+    eager = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
+    want = eager.get_data()
+    eager.dispose()
+    ctx.sync()
+    ctx.graph_begin()
+    try:
+        out = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
+    finally:
+        gid = ctx.graph_end()
+    for rep in range(3):
+        ctx.graph_launch(gid)
+        ctx.sync()
+        assert_bit_exact(out.get_data(), want, "replay %d" % rep)
+    out.dispose()
+    ctx.graph_destroy(gid)
+    for t in (tx, tw, tb):
+        t.dispose()
+
+
 @pytest.mark.parametrize("n,cin,h,w,cout,sh,group", [
     (4, 256, 56, 56, 128, 2, 1),       # the stride-2 1x1 convs that open ResNet-50's stages 2 and 3
     (4, 512, 28, 28, 1024, 2, 1),

@@ -18,7 +18,7 @@ ADDON_SRC = os.path.join(ROOT, "webdnn_amd", "napi", "addon.c")
 ADDON = os.path.join(LIBDIR, "webdnn_hip.node")
 
 HIP_SOURCES = ["runtime.hip", "gemm.hip", "contraction_gemm_akc.hip", "contraction_gemm_amc.hip", "contraction_conv_gather.hip",
-               "contraction_conv_pixels.hip", "contraction_conv3x3.hip", "conv_patch.hip", "elementwise.hip", "reduce.hip", "attention.hip", "pool_layout.hip"]
+               "contraction_conv_pixels.hip", "contraction_conv3x3.hip", "conv_patch.hip", "winograd.hip", "elementwise.hip", "reduce.hip", "attention.hip", "pool_layout.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -56,6 +56,7 @@ SIGNATURES = {
                                    _c.c_int, c_buf]),
     "wdh_linear_group": (_c.c_int, [_c.c_int, _i64p, _i64p, _i64p, _i64p, _i32p, _i32p, _i32p, _c.c_int]),
     "wdh_conv2d": (_c.c_int, [c_buf, c_buf, c_buf, c_buf] + [_c.c_int] * 17 + [c_buf]),
+    "wdh_conv2d_ex": (_c.c_int, [c_buf, c_buf, c_buf, c_buf] + [_c.c_int] * 17 + [c_buf, _c.c_int]),
     "wdh_binary": (_c.c_int, [_c.c_int, _c.c_int, c_buf, c_buf, c_buf, _c.c_int, _i32p, _i64p, _i64p]),
     "wdh_unary": (_c.c_int, [_c.c_int, _c.c_int, c_buf, c_buf, _c.c_size_t]),
     "wdh_softmax": (_c.c_int, [c_buf, c_buf, _c.c_int64, _c.c_int]),

@@ -27,6 +27,8 @@ int init_attention();
 // Device resources of the contraction kernels that outlive a call (called by wdh_init / at shutdown).
 int init_contraction(int device);
 void release_contraction();
+// The buffer behind `h` is about to be freed or overwritten: drops what the conv code derived from it.
+void conv_forget_weights(wdh_buf h);
 // After a synchronisation: fails if a contraction kernel reported that it gave up a wait.
 int contraction_check();
 
@@ -43,6 +45,14 @@ bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh,
                         int pt, int pl, int oh, int ow);
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
                       int h, int w, int oh, int ow, int pt, int pl, int relu);
+
+// The transforms of the F(2x2, 3x3) form of a 3x3 stride-1 conv (winograd.hip): filters -> U [16][cout][c],
+// input -> V [16][c][tiles], products M [16][cout][tiles] (+ bias, residual, Relu) -> Y.
+long long wino_tiles(int n, int oh, int ow);
+int wino_filter_launch(const float *W, float *U, int cout, int c);
+int wino_input_launch(const float *X, float *V, int n, int c, int h, int w, int oh, int ow, int pt, int pl);
+int wino_output_launch(const float *M, const float *Bias, const float *R, float *Y, int n, int cout, int oh, int ow,
+                       int relu);
 
 // Frees the per-geometry tap tables of the conv kernel (called at shutdown).
 void release_conv_tables();

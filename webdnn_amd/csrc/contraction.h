@@ -1718,6 +1718,7 @@ const int kTileN[] = {128, 256, 128, 64, 64};
 
 // ---- state and planning shared by the translation units (defined in gemm.hip) -------------
 extern int g_forced_tile;    // >= 0: overrides the tile choice (tuning hook)
+extern int g_tile_hint;      // >= 0: tile for the next Gemm / MatMul launch, set by a caller inside the library
 extern int g_forced_split;   // >= 1: overrides the split-K heuristic
 extern int g_last_form;
 extern bool g_static_scratch;  // set for the duration of a wdh_gemm_static call
@@ -1881,7 +1882,7 @@ int launch(Params &p, int nz, bool vec) {
   // accumulator tiles per wavefront
   const TileId conv_tile = (p.m >= 256 && p.k >= 2048) ? T128x64 : T64x64;
   TileId t = g_forced_tile >= 0 ? (TileId)g_forced_tile
-                                : (conv ? conv_tile : pick_tile(p.m, p.n, nz));
+                                : (conv ? conv_tile : (g_tile_hint >= 0 ? (TileId)g_tile_hint : pick_tile(p.m, p.n, nz)));
   switch (t) {
     case T128x128: return launch_tile<128, 128, 2, 2, A_KC, BMODE>(p, nz, vec);
     case T64x256: return launch_tile<64, 256, 1, 4, A_KC, BMODE>(p, nz, vec);

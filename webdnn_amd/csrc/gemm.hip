@@ -112,6 +112,7 @@ TileId pick_tile(int m, int n, int nz) {
   return tiles128 >= 2LL * wdh::compute_units() && filled >= 0.8 ? T128x128 : T64x64;
 }
 int g_forced_tile = -1;   // >= 0: overrides pick_tile (tuning hook)
+int g_tile_hint = -1;     // >= 0: the caller inside the library knows the tile for its next product
 int g_forced_split = -1;  // >= 1: overrides the split-K heuristic
 int g_descriptors = 1;    // 0: every operand is treated as if it spanned 2 GiB or more
 // what launch_planned decided for the most recent launch (wdh_last_plan)
@@ -131,6 +132,7 @@ struct GroupQueue {
 } g_group;
 int g_stem = 1;           // 0: the 7x7 stride-2 stem conv gathers its taps like any other geometry
 int g_pixels_s2 = 1;      // 0: 1x1 convs with a column stride of 2 gather their taps like any other geometry
+int g_winograd = 1;       // 3x3 stride-1 convs as F(2x2, 3x3): 0 never, 1 where it was measured to win, 2 wherever legal
 int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
 int g_stream = 1;         // launches scheduled as streams of K slabs: 0 never, 1 where the plan below gains, 2 wherever legal
 int g_stream_wgs = 4;     // workgroups per CU of a stream launch (at most what the kernel's resources allow)
@@ -335,6 +337,11 @@ extern "C" int wdh_set_option(const char *name, int value) {
     if (value != 0 && value != 1)
       return fail(WDH_EINVAL, "wdh_set_option: conv_stem %d (use 0 or 1)", value);
     g_stem = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "conv3x3_winograd") == 0) {
+    if (value < 0 || value > 2) return fail(WDH_EINVAL, "wdh_set_option: conv3x3_winograd %d (use 0, 1 or 2)", value);
+    g_winograd = value;
     return WDH_OK;
   }
   if (strcmp(name, "conv1x1_stride2_in_place") == 0) {
@@ -612,6 +619,14 @@ struct KtabVal {
 
 std::map<KtabKey, KtabVal> g_ktabs;
 
+// Transformed filters (U of the F(2x2, 3x3) form) of weight buffers whose owner promised not to
+// write to them (WDH_CONV_CONSTANT_WEIGHTS): weight handle -> a pool block that holds U.
+struct FilterEntry {
+  wdh_buf u;
+  int cout, c;
+};
+std::map<wdh_buf, FilterEntry> g_filters;
+
 }  // namespace
 
 namespace wdh {
@@ -624,6 +639,16 @@ void release_conv_tables() {
 // The word a stream launch sets when one of its workgroups gave up waiting for a partial tile
 // lives in pinned host memory the device writes to directly, so the host can look at it after
 // any synchronisation without a copy.
+// The buffer behind `h` is about to be freed or written to: data derived from it is stale.
+void conv_forget_weights(wdh_buf h) {
+  if (g_filters.empty()) return;
+  auto it = g_filters.find(h);
+  if (it == g_filters.end()) return;
+  const wdh_buf u = it->second.u;
+  g_filters.erase(it);  // first: wdh_free comes back here for `u`
+  (void)wdh_free(u);
+}
+
 int init_contraction(int device) {
   if (g_stream_error) return WDH_OK;
   void *host = nullptr, *dev = nullptr;
@@ -646,6 +671,7 @@ int init_contraction(int device) {
   return WDH_OK;
 }
 void release_contraction() {
+  g_filters.clear();  // (the blocks go with the pool)
   if (g_stream_error) (void)hipHostFree(g_stream_error);
   g_stream_error = g_stream_error_dev = nullptr;
 }
@@ -664,7 +690,16 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
                           int n, int c, int h, int w, int cout, int kh, int kw,
                           int pt, int pl, int pb, int pr, int sh, int sw,
                           int dh, int dw, int group, int epilogue, wdh_buf hR) {
+  return wdh_conv2d_ex(hX, hW, hBias, hY, n, c, h, w, cout, kh, kw, pt, pl, pb, pr, sh, sw, dh, dw, group, epilogue,
+                       hR, 0);
+}
+
+extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
+                             int n, int c, int h, int w, int cout, int kh, int kw,
+                             int pt, int pl, int pb, int pr, int sh, int sw,
+                             int dh, int dw, int group, int epilogue, wdh_buf hR, int flags) {
   WDH_REQUIRE_INIT();
+  if (flags & ~WDH_CONV_CONSTANT_WEIGHTS) return fail(WDH_EINVAL, "wdh_conv2d_ex: unknown flags %d", flags);
   if (n < 0 || c <= 0 || h <= 0 || w <= 0 || cout <= 0 || kh <= 0 || kw <= 0 ||
       sh <= 0 || sw <= 0 || dh <= 0 || dw <= 0 || group <= 0 || pt < 0 ||
       pl < 0 || pb < 0 || pr < 0)
@@ -759,6 +794,63 @@ extern "C" int wdh_conv2d(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     p.c_bytes = cout * 4;
     set_wide(p, true);
     return launch_conv_pixels(p, group, true, in_place_s2);
+  }
+  // 3x3, stride 1, no dilation, one group, many channels: F(2x2, 3x3) -- filters and 4x4 input patches
+  // are transformed, the 16 positions of the transform domain are one batched product
+  // M[xi] = U[xi] [cout, c] x V[xi] [c, tiles] with 4/9 of the direct form's multiplications, and the
+  // products are transformed back under the epilogue (winograd.hip).
+  if (g_winograd && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 && group == 1 && c % BK == 0 &&
+      g_forced_tile < 0 && g_forced_split < 0 && (g_winograd == 2 || (c >= 128 && cout >= 128))) {
+    const long long tiles = wdh::wino_tiles(n, oh, ow);
+    const size_t u_bytes = (size_t)16 * cout * c * 4, v_bytes = (size_t)16 * c * tiles * 4,
+                 m_bytes = (size_t)16 * cout * tiles * 4;
+    if (tiles < 0x7fffffffLL && v_bytes < ((size_t)1 << 33) && m_bytes < ((size_t)1 << 33)) {
+      // the transformed filters: kept from call to call when the caller vouches for the weights
+      // (a block allocated while a graph is being recorded belongs to that graph, so nothing is kept then)
+      wdh_buf hU = 0;
+      bool u_kept = false, u_ready = false;
+      if (flags & WDH_CONV_CONSTANT_WEIGHTS) {
+        auto it = g_filters.find(hW);
+        if (it != g_filters.end() && it->second.cout == cout && it->second.c == c) {
+          hU = it->second.u;
+          u_kept = u_ready = true;
+        } else if (!wdh::capturing()) {
+          wdh::conv_forget_weights(hW);
+          hU = wdh_alloc(u_bytes);
+          if (hU) {
+            g_filters[hW] = FilterEntry{hU, cout, c};
+            u_kept = true;
+          }
+        }
+      }
+      if (!hU) hU = wdh_alloc(u_bytes);
+      const wdh_buf hV = wdh_alloc(v_bytes), hM = wdh_alloc(m_bytes);
+      int rc = hU && hV && hM ? WDH_OK : WDH_ENOMEM;
+      if (rc == WDH_OK) {
+        float *U = (float *)wdh::resolve(hU, nullptr), *V = (float *)wdh::resolve(hV, nullptr);
+        if (!u_ready) rc = wdh::wino_filter_launch(p.A, U, cout, c);
+        if (rc == WDH_OK) rc = wdh::wino_input_launch(p.B, V, n, c, h, w, oh, ow, pt, pl);
+      }
+      if (rc == WDH_OK) {
+        // (64x64 tiles: the 16 products have K = c, short against their extent; measured best on
+        // every 3x3 layer shape of ResNet-50 and DETR, 35 against 44 us where the general choice
+        // takes 128x128)
+        g_tile_hint = T64x64;
+        rc = wdh_gemm(hU, hV, 0, hM, 16, cout, (int)tiles, c, (int64_t)cout * c, c, 1, (int64_t)c * tiles, tiles, 1, 0, 0,
+                      1.0f, 1.0f, WDH_EPI_NONE, 0);
+        g_tile_hint = -1;
+      }
+      if (rc == WDH_OK) {
+        g_last_plan.form = WDH_FORM_CONV3X3_WINOGRAD;
+        rc = wdh::wino_output_launch((const float *)wdh::resolve(hM, nullptr), p.C, p.R, p.Y, n, cout, oh, ow,
+                                     epilogue == WDH_EPI_RELU);
+      }
+      // (the blocks go back to the pool at once: whoever gets them next is ordered behind these kernels)
+      if (hU && !u_kept) (void)wdh_free(hU);
+      if (hV) (void)wdh_free(hV);
+      if (hM) (void)wdh_free(hM);
+      return rc;
+    }
   }
   // 3x3, stride 1, no dilation, input channels in blocks of 8: taps read from an input
   // tile staged in LDS (conv3x3_halo_kernel)

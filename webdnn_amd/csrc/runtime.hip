@@ -383,6 +383,7 @@ int wdh_free(wdh_buf h) {
   if (h <= 0 || (size_t)h > g.slots.size() || g.slots[h - 1].ptr == nullptr)
     return fail(WDH_EINVAL, "wdh_free: unknown buffer handle %lld",
                 (long long)h);
+  wdh::conv_forget_weights(h);
   Slot &s = g.slots[h - 1];
   if (s.cap) {
     if (s.arena && g.graphs[s.arena - 1].live) {
@@ -490,6 +491,7 @@ int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
     return fail(WDH_EINVAL, "wdh_write: %zu bytes at offset %zu exceed buffer of %zu",
                 bytes, dst_offset, have);
   if (bytes && !src) return fail(WDH_EINVAL, "wdh_write: src is NULL");
+  wdh::conv_forget_weights(h);
   const char *s = (const char *)src;
   size_t done = 0;
   while (done < bytes) {
@@ -567,6 +569,7 @@ int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
   if (dst_offset > dhave || bytes > dhave - dst_offset || src_offset > shave ||
       bytes > shave - src_offset)
     return fail(WDH_EINVAL, "wdh_copy: range exceeds a buffer");
+  wdh::conv_forget_weights(dst);
   if (bytes)
     WDH_HIP_CHECK(hipMemcpyAsync(d + dst_offset, s + src_offset, bytes,
                                  hipMemcpyDeviceToDevice, g.stream));

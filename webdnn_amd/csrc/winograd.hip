@@ -1,0 +1,187 @@
+// 3x3 stride-1 convolution by the minimal-filtering algorithm F(2x2, 3x3) (Winograd): the
+// transforms around the products.
+//
+// Semantics are those of the reference's Conv (src/descriptor_runner/operators/cpu/operators/
+// standard/conv.ts:134-221: im2col + matrix product, i.e. Y[o][oy][ox] = bias[o] +
+// sum_{c,ky,kx} W[o][c][ky][kx] X[c][oy+ky-pt][ox+kx-pl]); what differs is the arithmetic.  A
+// 2x2 block of outputs of one (output, input) channel pair needs 36 multiplications done
+// directly and 16 like this:
+//     Y = At [ (G g Gt) .* (Bt d B) ] A          d: the 4x4 input patch, g: the 3x3 filter
+//     Bt = | 1  0 -1  0 |   G = | 1    0    0  |   At = | 1  1  1  0 |
+//          | 0  1  1  0 |       | 1/2  1/2  1/2 |        | 0  1 -1 -1 |
+//          | 0 -1  1  0 |       | 1/2 -1/2  1/2 |
+//          | 0  1  0 -1 |       | 0    0    1  |
+// Summed over the input channels, the element-wise products at each of the 16 positions xi of
+// the 4x4 transform domain are one matrix product M[xi] = U[xi] x V[xi] with U[xi] [cout, c] the
+// transformed filters and V[xi] [c, tiles] the transformed input patches of all 2x2 output
+// blocks ("tiles") of the batch: 16 independent products, run as one batched wdh_gemm on the
+// matrix cores with 4/9 of the direct form's multiplications.  The three kernels here are the
+// bandwidth-bound rest: filters -> U, input -> V, M (+ bias, residual, Relu) -> Y.  The
+// transforms only add, subtract and halve, so their rounding is a few units in the last place
+// of the patch values; results stay within the Gemm/Conv tolerance of the oracle (tested), but
+// the sums are not the direct form's sums.
+#include "common.h"
+#include "fastdiv.h"
+
+namespace {
+
+using wdh::FastDiv;
+using wdh::fdiv;
+
+struct WinoGeom {
+  int n, c, h, w, cout, oh, ow, pt, pl;
+  int th, tw;          // 2x2 output blocks per image: ceil(oh/2) x ceil(ow/2)
+  int tiles;           // n * th * tw
+  FastDiv fd_tw, fd_thw;
+};
+
+// U[xi][o][ci] = (G g Gt)[xi] for filter g = W[o][ci]; one thread per (o, ci)
+__global__ __launch_bounds__(256) void wino_filter_kernel(const float *__restrict__ W, float *__restrict__ U,
+                                                          int cout, int c) {
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= cout * c) return;
+  const float *g = W + (long long)idx * 9;
+  float t[4][3];
+#pragma unroll
+  for (int j = 0; j < 3; j++) {
+    const float g0 = g[j], g1 = g[3 + j], g2 = g[6 + j];
+    t[0][j] = g0;
+    t[1][j] = 0.5f * (g0 + g1 + g2);
+    t[2][j] = 0.5f * (g0 - g1 + g2);
+    t[3][j] = g2;
+  }
+  const long long plane = (long long)cout * c;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float a = t[i][0], b = t[i][1], d = t[i][2];
+    U[(4 * i + 0) * plane + idx] = a;
+    U[(4 * i + 1) * plane + idx] = 0.5f * (a + b + d);
+    U[(4 * i + 2) * plane + idx] = 0.5f * (a - b + d);
+    U[(4 * i + 3) * plane + idx] = d;
+  }
+}
+
+// V[xi][ci][t] = (Bt d B)[xi] for the 4x4 patch d of channel ci whose corner is input pixel
+// (2 ty - pt, 2 tx - pl) of the tile's image; pixels outside the image are 0.
+// grid (ceil(tiles / 256), c): consecutive threads take consecutive tiles of one channel.
+__global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict__ X, float *__restrict__ V, WinoGeom g) {
+  const int t = blockIdx.x * 256 + threadIdx.x, ci = blockIdx.y;
+  if (t >= g.tiles) return;
+  const int img = fdiv(t, g.fd_thw), r = t - img * (g.th * g.tw);
+  const int ty = fdiv(r, g.fd_tw), tx = r - ty * g.tw;
+  const int iy0 = 2 * ty - g.pt, ix0 = 2 * tx - g.pl;
+  const float *base = X + ((long long)img * g.c + ci) * g.h * g.w;
+  float d[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int iy = iy0 + i;
+    const bool row_in = (unsigned)iy < (unsigned)g.h;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int ix = ix0 + j;
+      const bool in = row_in && (unsigned)ix < (unsigned)g.w;
+      d[i][j] = in ? base[(long long)iy * g.w + ix] : 0.0f;
+    }
+  }
+  float s[4][4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {  // Bt d
+    s[0][j] = d[0][j] - d[2][j];
+    s[1][j] = d[1][j] + d[2][j];
+    s[2][j] = d[2][j] - d[1][j];
+    s[3][j] = d[1][j] - d[3][j];
+  }
+  const long long plane = (long long)g.c * g.tiles;
+  float *out = V + (long long)ci * g.tiles + t;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {  // (Bt d) B
+    out[(4 * i + 0) * plane] = s[i][0] - s[i][2];
+    out[(4 * i + 1) * plane] = s[i][1] + s[i][2];
+    out[(4 * i + 2) * plane] = s[i][2] - s[i][1];
+    out[(4 * i + 3) * plane] = s[i][1] - s[i][3];
+  }
+}
+
+// Y block of tile t, channel o = At M[.][o][t] A, + bias, + residual, Relu.
+// grid (ceil(tiles / 256), cout).
+__global__ __launch_bounds__(256) void wino_output_kernel(const float *__restrict__ M, const float *__restrict__ Bias,
+                                                          const float *__restrict__ R, float *__restrict__ Y,
+                                                          WinoGeom g, int relu) {
+  const int t = blockIdx.x * 256 + threadIdx.x, o = blockIdx.y;
+  if (t >= g.tiles) return;
+  const long long plane = (long long)g.cout * g.tiles;
+  const float *in = M + (long long)o * g.tiles + t;
+  float m[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) m[i][j] = in[(4 * i + j) * plane];
+  float s[2][4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {  // At m
+    s[0][j] = m[0][j] + m[1][j] + m[2][j];
+    s[1][j] = m[1][j] - m[2][j] - m[3][j];
+  }
+  const int img = fdiv(t, g.fd_thw), r = t - img * (g.th * g.tw);
+  const int ty = fdiv(r, g.fd_tw), tx = r - ty * g.tw;
+  const float bias = Bias ? Bias[o] : 0.0f;
+  const long long base = ((long long)img * g.cout + o) * g.oh * g.ow;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int oy = 2 * ty + i;
+    if (oy >= g.oh) break;
+    float y[2] = {s[i][0] + s[i][1] + s[i][2], s[i][1] - s[i][2] - s[i][3]};
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int ox = 2 * tx + j;
+      if (ox >= g.ow) break;
+      const long long off = base + (long long)oy * g.ow + ox;
+      float v = y[j];
+      if (Bias) v = v + bias;
+      if (R) v = v + R[off];
+      if (relu) v = v <= 0.0f ? 0.0f : v;   // Math.max(v, 0): NaN stays, -0 becomes +0
+      Y[off] = v;
+    }
+  }
+}
+
+}  // namespace
+
+namespace wdh {
+
+long long wino_tiles(int n, int oh, int ow) { return (long long)n * ((oh + 1) / 2) * ((ow + 1) / 2); }
+
+int wino_filter_launch(const float *W, float *U, int cout, int c) {
+  const long long total = (long long)cout * c;
+  hipLaunchKernelGGL(wino_filter_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream(), W, U, cout, c);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+static WinoGeom make_geom(int n, int c, int h, int w, int cout, int oh, int ow, int pt, int pl) {
+  WinoGeom g;
+  g.n = n; g.c = c; g.h = h; g.w = w; g.cout = cout; g.oh = oh; g.ow = ow; g.pt = pt; g.pl = pl;
+  g.th = (oh + 1) / 2; g.tw = (ow + 1) / 2;
+  g.tiles = (int)wino_tiles(n, oh, ow);
+  g.fd_tw = make_fastdiv(g.tw);
+  g.fd_thw = make_fastdiv((long long)g.th * g.tw);
+  return g;
+}
+
+int wino_input_launch(const float *X, float *V, int n, int c, int h, int w, int oh, int ow, int pt, int pl) {
+  const WinoGeom g = make_geom(n, c, h, w, 0, oh, ow, pt, pl);
+  hipLaunchKernelGGL(wino_input_kernel, dim3((unsigned)((g.tiles + 255) / 256), (unsigned)c), dim3(256), 0, stream(), X, V, g);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+int wino_output_launch(const float *M, const float *Bias, const float *R, float *Y, int n, int cout, int oh, int ow,
+                       int relu) {
+  const WinoGeom g = make_geom(n, 0, 0, 0, cout, oh, ow, 0, 0);
+  hipLaunchKernelGGL(wino_output_kernel, dim3((unsigned)((g.tiles + 255) / 256), (unsigned)cout), dim3(256), 0, stream(),
+                     M, Bias, R, Y, g, relu);
+  WDH_LAUNCH_CHECK();
+  return WDH_OK;
+}
+
+}  // namespace wdh

@@ -154,7 +154,7 @@ class HipContext:
 
     FORMS = ("gemm, B k-contiguous", "gemm, B n-contiguous", "conv, gathered taps", "conv, gathered taps (32-63)",
              "conv, gathered taps (flat loads)", "conv 1x1, X in place", "conv 3x3, LDS tile",
-             "conv 7x7 s2 stem, weights and patch in LDS", "conv 1x1 stride 2, X in place")
+             "conv 7x7 s2 stem, weights and patch in LDS", "conv 1x1 stride 2, X in place", "conv 3x3, F(2x2,3x3) transforms + batched product")
 
     def last_plan(self):
         """Layout of the most recent Gemm / Conv launch: tile, whole tiles, tiles cut along K, chunks, form."""
@@ -327,18 +327,19 @@ def conv_shape(dims_x, dims_w, dilations=None, group=1, kernel_shape=None, pads=
 
 
 def conv(ctx, x, w, b=None, dilations=None, group=1, kernel_shape=None, pads=None, strides=None,
-         epilogue=None, residual=None):
-    """Conv: cpu conv.ts:134-221; 2-D only."""
+         epilogue=None, residual=None, constant_weights=False):
+    """Conv: cpu conv.ts:134-221; 2-D only.  constant_weights: `w` is not written to while it lives (what the
+    runner says of an initializer's device copy), so the library may keep forms derived from it."""
     _require_f32(x, w, b, residual)
     if x.ndim != 4:
         raise OperatorError("Conv other than 2D is not yet supported")
     s = conv_shape(x.dims, w.dims, dilations, group, kernel_shape, pads, strides)
     y = ctx.empty_tensor([s["batch"], s["ch_out"], s["out_shape"][0], s["out_shape"][1]])
-    call("wdh_conv2d", x.handle, w.handle, b.handle if b is not None else 0, y.handle,
+    call("wdh_conv2d_ex", x.handle, w.handle, b.handle if b is not None else 0, y.handle,
          s["batch"], s["ch_in"], s["in_shape"][0], s["in_shape"][1], s["ch_out"],
          s["kernel_shape"][0], s["kernel_shape"][1], s["pads"][0], s["pads"][1], s["pads"][2],
          s["pads"][3], s["strides"][0], s["strides"][1], s["dilations"][0], s["dilations"][1],
-         group, EPI[epilogue], residual.handle if residual is not None else 0)
+         group, EPI[epilogue], residual.handle if residual is not None else 0, 1 if constant_weights else 0)
     return y
 
 

@@ -378,6 +378,9 @@ class RunnerImpl {
                     otherT,
                     this.tensorMoveOptions[inputName] || {}
                   );
+                  // the device copy of an initializer keeps its contents for as long as it lives
+                  // (operators may keep forms derived from it: see HipConv)
+                  if (this.initializerTensors.has(inputName)) movedT.constant = true;
                   tensorsForBackends[reqBackend].set(inputName, movedT);
                   operatorInputs.push(movedT);
                   found = true;

@@ -54,6 +54,10 @@ export interface HipNative {
   conv2d(X: Handle, W: Handle, bias: Handle, Y: Handle, n: number, c: number, h: number, w: number, cout: number,
          kh: number, kw: number, pt: number, pl: number, pb: number, pr: number, sh: number, sw: number,
          dh: number, dw: number, group: number, epilogue: number, R: Handle): void;
+  /** flags bit 0: W is not written to while its handle lives (derived forms of it may be kept) */
+  conv2dEx(X: Handle, W: Handle, bias: Handle, Y: Handle, n: number, c: number, h: number, w: number, cout: number,
+           kh: number, kw: number, pt: number, pl: number, pb: number, pr: number, sh: number, sw: number,
+           dh: number, dw: number, group: number, epilogue: number, R: Handle, flags: number): void;
   attention(Q: Handle, K: Handle, V: Handle, Y: Handle, batch: number, tq: number, tk: number, d: number,
             sQb: number, sQi: number, sKb: number, sKj: number, sVb: number, sVj: number, sYb: number, sYi: number,
             alpha: number): void;

@@ -57,10 +57,13 @@ class HipConv extends Conv {
     const sameShape = residual && residual.ndim === 4 && residual.dims.every((d, i) => d === outDims[i]);
     const inEpilogue = !residual || sameShape;
     const output = context.emptyTensor(outDims, "float32");
-    context.native.conv2d(inputX.handle, inputW.handle, inputB ? inputB.handle : 0, output.handle,
+    // flags bit 0: the weights are an initializer's device copy, which nobody writes to while it
+    // lives, so the library may keep forms derived from them (transformed filters) across calls
+    context.native.conv2dEx(inputX.handle, inputW.handle, inputB ? inputB.handle : 0, output.handle,
       s.batch, s.chIn, s.inShape[0], s.inShape[1], s.chOut, s.kernelShape[0], s.kernelShape[1],
       s.pads[0], s.pads[1], s.pads[2], s.pads[3], s.strides[0], s.strides[1], s.dilations[0], s.dilations[1],
-      s.group, inEpilogue && this.activation === "Relu" ? 1 : 0, sameShape ? residual.handle : 0);
+      s.group, inEpilogue && this.activation === "Relu" ? 1 : 0, sameShape ? residual.handle : 0,
+      inputW.constant ? 1 : 0);
     if (inEpilogue) return [output];
     return [addThenActivate(context, output, residual, this.activation)];
   }

@@ -311,6 +311,18 @@ FN(js_conv2d) {
   return make_undefined(env);
 }
 
+FN(js_conv2d_ex) {
+  ARGS("wdh_conv2d_ex", 23);
+  I64(0, X); I64(1, W); I64(2, Bias); I64(3, Y);
+  int64_t g[17];
+  for (int i = 0; i < 17; i++)
+    if (!to_i64(env, argv[4 + i], &g[i])) return throw_arg(env, FNAME, "geometry arguments must be integers");
+  I64(21, R); I64(22, flags);
+  CHECK(wdh_conv2d_ex(X, W, Bias, Y, (int)g[0], (int)g[1], (int)g[2], (int)g[3], (int)g[4], (int)g[5],
+                      (int)g[6], (int)g[7], (int)g[8], (int)g[9], (int)g[10], (int)g[11], (int)g[12],
+                      (int)g[13], (int)g[14], (int)g[15], (int)g[16], R, (int)flags));
+  return make_undefined(env);
+}
 FN(js_binary) { /* (op, dtype, L, R, Y, outShape[], stridesL[], stridesR[]) */
   ARGS("wdh_binary", 8);
   I64(0, op); I64(1, dtype); I64(2, L); I64(3, R); I64(4, Y);
@@ -476,7 +488,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"setOption", js_set_option}, {"alloc", js_alloc}, {"free", js_free}, {"write", js_write},
       {"read", js_read}, {"copy", js_copy}, {"sync", js_sync}, {"memStats", js_mem_stats},
       {"trim", js_trim}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
-      {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"linearGroup", js_linear_group}, {"conv2d", js_conv2d}, {"binary", js_binary}, {"unary", js_unary},
+      {"gemm", js_gemm}, {"gemmEx", js_gemm_ex}, {"linearGroup", js_linear_group}, {"conv2d", js_conv2d}, {"conv2dEx", js_conv2d_ex}, {"binary", js_binary}, {"unary", js_unary},
       {"softmax", js_softmax}, {"attention", js_attention}, {"layernorm", js_layernorm}, {"layernormAdd", js_layernorm_add}, {"reduceMean", js_reduce_mean}, {"reduceAxis", js_reduce_axis},
       {"maxpool2d", js_maxpool2d}, {"globalAvgpool", js_global_avgpool},
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
