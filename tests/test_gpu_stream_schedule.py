@@ -30,8 +30,9 @@ def he(cout, cin, k):
 def stream_always(ctx):
     """Every launch that has a stream form takes it, whatever the plan would choose."""
     ctx.set_option("stream_k", 2)
+    ctx.set_option("conv3x3_winograd", 0)       # the direct forms are what is scheduled here
     yield ctx
-    for name, value in (("stream_k", 1), ("stream_wgs", 4), ("contraction_tile", -1)):
+    for name, value in (("stream_k", 1), ("stream_wgs", 4), ("contraction_tile", -1), ("conv3x3_winograd", 1)):
         ctx.set_option(name, value)
 
 

@@ -47,8 +47,9 @@ int conv_patch_launch(const float *X, const float *W, const float *Bias, const f
                       int h, int w, int oh, int ow, int pt, int pl, int relu);
 
 // The transforms of the F(2x2, 3x3) form of a 3x3 stride-1 conv (winograd.hip): filters -> U [16][cout][c],
-// input -> V [16][c][tiles], products M [16][cout][tiles] (+ bias, residual, Relu) -> Y.
+// input -> V [16][c][pitch], products M [16][cout][pitch] (+ bias, residual, Relu) -> Y.
 long long wino_tiles(int n, int oh, int ow);
+long long wino_pitch(long long tiles);
 int wino_filter_launch(const float *W, float *U, int cout, int c);
 int wino_input_launch(const float *X, float *V, int n, int c, int h, int w, int oh, int ow, int pt, int pl);
 int wino_output_launch(const float *M, const float *Bias, const float *R, float *Y, int n, int cout, int oh, int ow,

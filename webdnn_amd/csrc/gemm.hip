@@ -801,7 +801,7 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
   // products are transformed back under the epilogue (winograd.hip).
   if (g_winograd && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 && group == 1 && c % BK == 0 &&
       g_forced_tile < 0 && g_forced_split < 0 && (g_winograd == 2 || (c >= 128 && cout >= 128))) {
-    const long long tiles = wdh::wino_tiles(n, oh, ow);
+    const long long tiles = wdh::wino_pitch(wdh::wino_tiles(n, oh, ow));  // (row length of V and M)
     const size_t u_bytes = (size_t)16 * cout * c * 4, v_bytes = (size_t)16 * c * tiles * 4,
                  m_bytes = (size_t)16 * cout * tiles * 4;
     if (tiles < 0x7fffffffLL && v_bytes < ((size_t)1 << 33) && m_bytes < ((size_t)1 << 33)) {

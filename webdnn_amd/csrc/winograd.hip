@@ -16,7 +16,8 @@
 // transformed filters and V[xi] [c, tiles] the transformed input patches of all 2x2 output
 // blocks ("tiles") of the batch: 16 independent products, run as one batched wdh_gemm on the
 // matrix cores with 4/9 of the direct form's multiplications.  The three kernels here are the
-// bandwidth-bound rest: filters -> U, input -> V, M (+ bias, residual, Relu) -> Y.  The
+// bandwidth-bound rest: filters -> U, input -> V, M (+ bias, residual, Relu) -> Y.  Rows of V and M
+// are `pitch` long (the tile count rounded up to 16).  The
 // transforms only add, subtract and halve, so their rounding is a few units in the last place
 // of the patch values; results stay within the Gemm/Conv tolerance of the oracle (tested), but
 // the sums are not the direct form's sums.
@@ -32,6 +33,7 @@ struct WinoGeom {
   int n, c, h, w, cout, oh, ow, pt, pl;
   int th, tw;          // 2x2 output blocks per image: ceil(oh/2) x ceil(ow/2)
   int tiles;           // n * th * tw
+  int pitch;           // row length of V and M: tiles rounded up (16-byte aligned rows for the product)
   FastDiv fd_tw, fd_thw;
 };
 
@@ -91,8 +93,8 @@ __global__ __launch_bounds__(256) void wino_input_kernel(const float *__restrict
     s[2][j] = d[2][j] - d[1][j];
     s[3][j] = d[1][j] - d[3][j];
   }
-  const long long plane = (long long)g.c * g.tiles;
-  float *out = V + (long long)ci * g.tiles + t;
+  const long long plane = (long long)g.c * g.pitch;
+  float *out = V + (long long)ci * g.pitch + t;
 #pragma unroll
   for (int i = 0; i < 4; i++) {  // (Bt d) B
     out[(4 * i + 0) * plane] = s[i][0] - s[i][2];
@@ -109,8 +111,8 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
                                                           WinoGeom g, int relu) {
   const int t = blockIdx.x * 256 + threadIdx.x, o = blockIdx.y;
   if (t >= g.tiles) return;
-  const long long plane = (long long)g.cout * g.tiles;
-  const float *in = M + (long long)o * g.tiles + t;
+  const long long plane = (long long)g.cout * g.pitch;
+  const float *in = M + (long long)o * g.pitch + t;
   float m[4][4];
 #pragma unroll
   for (int i = 0; i < 4; i++)
@@ -150,6 +152,10 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
 namespace wdh {
 
 long long wino_tiles(int n, int oh, int ow) { return (long long)n * ((oh + 1) / 2) * ((ow + 1) / 2); }
+// Row length of V and M: rows start on 64-byte boundaries whatever the tile count (the columns past the
+// last tile are never written by the input transform and never read by the output transform; what the
+// product makes of them stays in them, every column of a matrix product being independent of the others).
+long long wino_pitch(long long tiles) { return (tiles + 15) / 16 * 16; }
 
 int wino_filter_launch(const float *W, float *U, int cout, int c) {
   const long long total = (long long)cout * c;
@@ -163,6 +169,7 @@ static WinoGeom make_geom(int n, int c, int h, int w, int cout, int oh, int ow, 
   g.n = n; g.c = c; g.h = h; g.w = w; g.cout = cout; g.oh = oh; g.ow = ow; g.pt = pt; g.pl = pl;
   g.th = (oh + 1) / 2; g.tw = (ow + 1) / 2;
   g.tiles = (int)wino_tiles(n, oh, ow);
+  g.pitch = (int)wino_pitch(g.tiles);
   g.fd_tw = make_fastdiv(g.tw);
   g.fd_thw = make_fastdiv((long long)g.th * g.tw);
   return g;
