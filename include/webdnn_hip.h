@@ -81,10 +81,18 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *   "conv3x3_winograd"  how 3x3, stride-1, undilated, ungrouped convolutions whose channel count is a
  *                       multiple of 16 are computed: 1 (default) = those with at least 128 input and
  *                       128 output channels by the minimal-filtering algorithm F(2x2, 3x3) (filters
- *                       and 4x4 input patches transformed, 16 batched matrix products with 4/9 of the
- *                       multiplications, results transformed back under the epilogue); 2 = all of
- *                       them; 0 = none (the direct forms below).  Not the direct form's sums: results
- *                       agree within the Gemm/Conv tolerance, not bit for bit.
+ *                       and 4x4 input patches transformed, 16 batched matrix products with 4/9 of
+ *                       the multiplications, results transformed back under the epilogue; rounding
+ *                       errors like the direct form's, about 1.5e-7 of max|ref|); 2 = all of them
+ *                       that way; 3 = all of them by F(4x4, 3x3) (6x6 patches, 36 products, a quarter
+ *                       of the multiplications; 10-20 % faster than F(2x2, 3x3) from 64 channels on,
+ *                       rounding errors about 1e-6 of max|ref|: inside the Gemm/Conv tolerance, but
+ *                       ResNet-50's logits then differ from the CPU path's by 1.7e-3 where 1e-3 is
+ *                       asked and the other forms give 7e-4); 0 = none (the direct forms below).
+ *                       Not the direct form's sums: no form agrees with another bit for bit.
+ *   "conv3x3_f4x4_channels"  0 (default) or a channel count from which "conv3x3_winograd" 1 takes
+ *                       F(4x4, 3x3) instead (64 is where it starts to win): for callers who can
+ *                       trade the last digit for speed.
  *   "conv_stem"         1 (default) = a 7x7, stride-2, undilated convolution from 3 to 64
  *                       channels (the stem of an image network) runs in a kernel that keeps
  *                       all weights and a tile's input patch in LDS; 0 = it gathers taps
@@ -146,6 +154,7 @@ int wdh_set_option(const char *name, int value);
                                    * every other pixel of a row kept            */
 #define WDH_FORM_CONV3X3_WINOGRAD 9 /* 3x3 stride 1 as F(2x2, 3x3): transforms around a
                                    * batched product (tile and split are the product's) */
+#define WDH_FORM_CONV3X3_WINOGRAD4 10 /* ... as F(4x4, 3x3)                              */
 int wdh_last_plan(int *tile_m, int *tile_n, int64_t *whole_tiles,
                   int64_t *split_tiles, int *split, int *form);
 

@@ -1156,26 +1156,35 @@ WINOGRAD_CONVS = [
     (2, 16, 8, 8, 16, [0, 0, 0, 0]),          # no padding
     (3, 48, 10, 7, 16, [2, 0, 1, 2]),         # unequal pads, wider than the filter's reach on one side
     (1, 16, 3, 3, 32, [1, 1, 1, 1]),
+    (2, 64, 21, 18, 64, [1, 1, 1, 1]),        # neither side a multiple of the block of either form
 ]
 
 
+WINOGRAD_FORMS = {2: "conv 3x3, F(2x2,3x3)", 3: "conv 3x3, F(4x4,3x3)"}
+
+
+@pytest.mark.parametrize("mode", [2, 3])
 @pytest.mark.parametrize("shape", WINOGRAD_CONVS)
-def test_conv3x3_by_minimal_filtering(ctx, shape):
-    """3x3 stride-1 convs as F(2x2, 3x3): transformed filters and input patches, 16 batched products, results
-    transformed back under bias + residual + Relu.  Not the direct form's sums, so the bar is the Gemm/Conv
-    tolerance against the oracle -- for the forced form, for what the plan picks, and with the filters kept
-    from a first call (WDH_CONV_CONSTANT_WEIGHTS)."""
+def test_conv3x3_by_minimal_filtering(ctx, shape, mode):
+    """3x3 stride-1 convs as F(2x2, 3x3) / F(4x4, 3x3): transformed filters and input patches, 16 / 36 batched
+    products, results transformed back under bias + residual + Relu.  Not the direct form's sums, so the bar is
+    the Gemm/Conv tolerance against the oracle -- for the forced form, for what the plan picks, and with the
+    filters kept from a first call (WDH_CONV_CONSTANT_WEIGHTS).  Inputs of both signs as well as the
+    non-negative ones a Relu leaves: the transforms of F(4x4, 3x3) cancel more with mixed signs."""
     n, cin, h, w, cout, pads = shape
     X, W, B = uni(n, cin, h, w, lo=0), he(cout, cin, 3), nrm(cout)
     want0 = ref.conv(X, W, B, pads=pads)
     R = nrm(*want0.shape)
     want = ref.unary("Relu", ref.binary("Add", want0, R))
+    form = WINOGRAD_FORMS[mode]
     try:
-        ctx.set_option("conv3x3_winograd", 2)
+        ctx.set_option("conv3x3_winograd", mode)
         got = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
-        assert ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)"), ctx.last_plan()
-        assert_close_max(got, want, GEMM_TOL, "F(2x2,3x3) %s" % (shape,))
+        assert ctx.last_plan()["form"].startswith(form), ctx.last_plan()
+        assert_close_max(got, want, GEMM_TOL, "%s %s" % (form, shape))
         assert_close_max(hip_conv(ctx, X, W, None, pads=pads), ref.conv(X, W, None, pads=pads), GEMM_TOL, "no bias")
+        Xs = nrm(n, cin, h, w)
+        assert_close_max(hip_conv(ctx, Xs, W, B, pads=pads), ref.conv(Xs, W, B, pads=pads), GEMM_TOL, "signed input")
         # filters kept across calls: same bits as computing them every time; other weights in the same
         # buffer (wdh_write) or in a new buffer are seen
         tx, tw, tb, tr = (ctx.move_tensor(v) for v in (X, W, B, R))
@@ -1188,54 +1197,74 @@ def test_conv3x3_by_minimal_filtering(ctx, shape):
         want2 = ref.unary("Relu", ref.binary("Add", ref.conv(X, W2, B, pads=pads), R))
         again = H.conv(ctx, tx, tw, tb, pads=pads, epilogue="relu", residual=tr, constant_weights=True).get_data()
         assert_close_max(again, want2, GEMM_TOL, "weights rewritten in place")
+        if mode == 3:
+            # filters kept for one form are not taken for the other
+            ctx.set_option("conv3x3_winograd", 2)
+            other = H.conv(ctx, tx, tw, tb, pads=pads, epilogue="relu", residual=tr, constant_weights=True).get_data()
+            assert ctx.last_plan()["form"].startswith(WINOGRAD_FORMS[2])
+            assert_close_max(other, want2, GEMM_TOL, "the other form after kept filters")
         for t in (tx, tw, tb, tr):
             t.dispose()
     finally:
         ctx.set_option("conv3x3_winograd", 1)
-    auto = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
-    assert_close_max(auto, want, GEMM_TOL, "the plan's own choice %s" % (ctx.last_plan()["form"],))
-    picked = ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
-    assert picked == (cin >= 128 and cout >= 128), ctx.last_plan()
-    try:
-        ctx.set_option("conv3x3_winograd", 0)
-        direct = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
-        assert not ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
-        assert_close_max(direct, want, GEMM_TOL, "direct form")
-    finally:
-        ctx.set_option("conv3x3_winograd", 1)
+    if mode == 3:
+        auto = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+        assert_close_max(auto, want, GEMM_TOL, "the plan's own choice %s" % (ctx.last_plan()["form"],))
+        picked = ctx.last_plan()["form"].startswith(WINOGRAD_FORMS[2])
+        assert picked == (cin >= 128 and cout >= 128), ctx.last_plan()
+        try:
+            ctx.set_option("conv3x3_f4x4_channels", 64)     # F(4x4, 3x3) on request, from that many channels on
+            fast = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+            assert_bit_exact(fast, got if cin >= 64 and cout >= 64 else auto, "conv3x3_f4x4_channels")
+        finally:
+            ctx.set_option("conv3x3_f4x4_channels", 0)
+        try:
+            ctx.set_option("conv3x3_winograd", 0)
+            direct = hip_conv(ctx, X, W, B, pads=pads, epilogue="relu", R=R)
+            assert not ctx.last_plan()["form"].startswith("conv 3x3, F("), ctx.last_plan()
+            assert_close_max(direct, want, GEMM_TOL, "direct form")
+        finally:
+            ctx.set_option("conv3x3_winograd", 1)
 
 
-def test_conv3x3_minimal_filtering_keeps_special_values_local_and_replays(ctx):
+@pytest.mark.parametrize("mode", [2, 3])
+def test_conv3x3_minimal_filtering_keeps_special_values_local_and_replays(ctx, mode):
     """An Inf in the input reaches only the outputs whose receptive field holds it... in the transform domain
-    it meets finite values of its 4x4 patch, so the 2x2 block it belongs to may turn NaN, never a block further
-    away; and the form replays from a captured graph with kept filters."""
+    it meets finite values of its input patch, so the output blocks whose patches hold it may turn NaN, never a
+    block further away; and the form replays from a captured graph with kept filters."""
     X, W, B = uni(2, 128, 12, 12, lo=0), he(128, 128, 3), nrm(128)
     X[1, 5, 6, 6] = np.inf
-    got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])
-    assert ctx.last_plan()["form"].startswith("conv 3x3, F(2x2,3x3)")
-    bad = ~np.isfinite(got)
-    assert not bad[0].any(), "the other image is untouched"
-    ys, xs = np.nonzero(bad[1].any(axis=0))
-    assert ys.min() >= 4 and ys.max() <= 9 and xs.min() >= 4 and xs.max() <= 9, (ys, xs)
-    Xc = np.where(np.isfinite(X), X, 0).astype(np.float32)
-    tx, tw, tb = (ctx.move_tensor(v) for v in (Xc, W, B))
-    eager = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
-    want = eager.get_data()
-    eager.dispose()
-    ctx.sync()
-    ctx.graph_begin()
     try:
-        out = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
-    finally:
-        gid = ctx.graph_end()
-    for rep in range(3):
-        ctx.graph_launch(gid)
+        ctx.set_option("conv3x3_winograd", mode)
+        got = hip_conv(ctx, X, W, B, pads=[1, 1, 1, 1])
+        assert ctx.last_plan()["form"].startswith(WINOGRAD_FORMS[mode])
+        bad = ~np.isfinite(got)
+        assert not bad[0].any(), "the other image is untouched"
+        # with one row and column of padding, input (6, 6) lies in the patches of the 2x2 blocks 2 and 3 of its
+        # row and column and in the patch of 4x4 block 1: output rows and columns 4..7 either way
+        ys, xs = np.nonzero(bad[1].any(axis=0))
+        assert ys.min() >= 4 and ys.max() <= 7 and xs.min() >= 4 and xs.max() <= 7, (ys, xs)
+        Xc = np.where(np.isfinite(X), X, 0).astype(np.float32)
+        tx, tw, tb = (ctx.move_tensor(v) for v in (Xc, W, B))
+        eager = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
+        want = eager.get_data()
+        eager.dispose()
         ctx.sync()
-        assert_bit_exact(out.get_data(), want, "replay %d" % rep)
-    out.dispose()
-    ctx.graph_destroy(gid)
-    for t in (tx, tw, tb):
-        t.dispose()
+        ctx.graph_begin()
+        try:
+            out = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
+        finally:
+            gid = ctx.graph_end()
+        for rep in range(3):
+            ctx.graph_launch(gid)
+            ctx.sync()
+            assert_bit_exact(out.get_data(), want, "replay %d" % rep)
+        out.dispose()
+        ctx.graph_destroy(gid)
+        for t in (tx, tw, tb):
+            t.dispose()
+    finally:
+        ctx.set_option("conv3x3_winograd", 1)
 
 
 @pytest.mark.parametrize("n,cin,h,w,cout,sh,group", [

@@ -46,14 +46,15 @@ bool conv_patch_applies(int c, int cout, int kh, int kw, int sh, int sw, int dh,
 int conv_patch_launch(const float *X, const float *W, const float *Bias, const float *R, float *Y, int n,
                       int h, int w, int oh, int ow, int pt, int pl, int relu);
 
-// The transforms of the F(2x2, 3x3) form of a 3x3 stride-1 conv (winograd.hip): filters -> U [16][cout][c],
-// input -> V [16][c][pitch], products M [16][cout][pitch] (+ bias, residual, Relu) -> Y.
-long long wino_tiles(int n, int oh, int ow);
+// The transforms of the minimal-filtering forms of a 3x3 stride-1 conv (winograd.hip), r = 2 for F(2x2, 3x3)
+// (16 positions) or 4 for F(4x4, 3x3) (36 positions): filters -> U [positions][cout][c], input ->
+// V [positions][c][pitch], products M [positions][cout][pitch] (+ bias, residual, Relu) -> Y.
+long long wino_tiles(int r, int n, int oh, int ow);
 long long wino_pitch(long long tiles);
-int wino_filter_launch(const float *W, float *U, int cout, int c);
-int wino_input_launch(const float *X, float *V, int n, int c, int h, int w, int oh, int ow, int pt, int pl);
-int wino_output_launch(const float *M, const float *Bias, const float *R, float *Y, int n, int cout, int oh, int ow,
-                       int relu);
+int wino_filter_launch(int r, const float *W, float *U, int cout, int c);
+int wino_input_launch(int r, const float *X, float *V, int n, int c, int h, int w, int oh, int ow, int pt, int pl);
+int wino_output_launch(int r, const float *M, const float *Bias, const float *R, float *Y, int n, int cout, int oh,
+                       int ow, int relu);
 
 // Frees the per-geometry tap tables of the conv kernel (called at shutdown).
 void release_conv_tables();

@@ -132,7 +132,8 @@ struct GroupQueue {
 } g_group;
 int g_stem = 1;           // 0: the 7x7 stride-2 stem conv gathers its taps like any other geometry
 int g_pixels_s2 = 1;      // 0: 1x1 convs with a column stride of 2 gather their taps like any other geometry
-int g_winograd = 1;       // 3x3 stride-1 convs as F(2x2, 3x3): 0 never, 1 where it was measured to win, 2 wherever legal
+int g_winograd4_channels = 0;  // when not 0: "conv3x3_winograd" 1 takes F(4x4, 3x3) from this many input and output channels on
+int g_winograd = 1;       // 3x3 stride-1 convs by minimal filtering: 0 never, 1 = F(2x2, 3x3) where it wins, 2 / 3 = F(2x2, 3x3) / F(4x4, 3x3) wherever legal
 int g_wide_stores = 1;    // 0: whole tiles store one element per lane and instruction
 int g_stream = 1;         // launches scheduled as streams of K slabs: 0 never, 1 where the plan below gains, 2 wherever legal
 int g_stream_wgs = 4;     // workgroups per CU of a stream launch (at most what the kernel's resources allow)
@@ -340,8 +341,13 @@ extern "C" int wdh_set_option(const char *name, int value) {
     return WDH_OK;
   }
   if (strcmp(name, "conv3x3_winograd") == 0) {
-    if (value < 0 || value > 2) return fail(WDH_EINVAL, "wdh_set_option: conv3x3_winograd %d (use 0, 1 or 2)", value);
+    if (value < 0 || value > 3) return fail(WDH_EINVAL, "wdh_set_option: conv3x3_winograd %d (use 0..3)", value);
     g_winograd = value;
+    return WDH_OK;
+  }
+  if (strcmp(name, "conv3x3_f4x4_channels") == 0) {
+    if (value < 0) return fail(WDH_EINVAL, "wdh_set_option: conv3x3_f4x4_channels %d (use 0 or more)", value);
+    g_winograd4_channels = value;
     return WDH_OK;
   }
   if (strcmp(name, "conv1x1_stride2_in_place") == 0) {
@@ -623,7 +629,7 @@ std::map<KtabKey, KtabVal> g_ktabs;
 // write to them (WDH_CONV_CONSTANT_WEIGHTS): weight handle -> a pool block that holds U.
 struct FilterEntry {
   wdh_buf u;
-  int cout, c;
+  int cout, c, r;  // r: 2 or 4, the form the filters were transformed for
 };
 std::map<wdh_buf, FilterEntry> g_filters;
 
@@ -795,15 +801,24 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
     set_wide(p, true);
     return launch_conv_pixels(p, group, true, in_place_s2);
   }
-  // 3x3, stride 1, no dilation, one group, many channels: F(2x2, 3x3) -- filters and 4x4 input patches
-  // are transformed, the 16 positions of the transform domain are one batched product
-  // M[xi] = U[xi] [cout, c] x V[xi] [c, tiles] with 4/9 of the direct form's multiplications, and the
-  // products are transformed back under the epilogue (winograd.hip).
-  if (g_winograd && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 && group == 1 && c % BK == 0 &&
-      g_forced_tile < 0 && g_forced_split < 0 && (g_winograd == 2 || (c >= 128 && cout >= 128))) {
-    const long long tiles = wdh::wino_pitch(wdh::wino_tiles(n, oh, ow));  // (row length of V and M)
-    const size_t u_bytes = (size_t)16 * cout * c * 4, v_bytes = (size_t)16 * c * tiles * 4,
-                 m_bytes = (size_t)16 * cout * tiles * 4;
+  // 3x3, stride 1, no dilation, one group, many channels: minimal filtering -- filters and input patches
+  // are transformed, the positions of the transform domain (16 for F(2x2, 3x3), 36 for F(4x4, 3x3)) are
+  // one batched product M[xi] = U[xi] [cout, c] x V[xi] [c, tiles] with 4/9 or 1/4 of the direct form's
+  // multiplications, and the products are transformed back under the epilogue (winograd.hip).
+  // g_winograd: 0 never; 1 = F(2x2, 3x3) from 128 channels on (F(4x4, 3x3) from g_winograd4_channels on, when
+  // that is set: faster from 64 channels on, but its rounding errors are about ten times the direct form's,
+  // which a 50-layer network's logits show); 2 / 3 = F(2x2, 3x3) / F(4x4, 3x3) wherever legal.
+  const int wino_min = c < cout ? c : cout;
+  int wino_r = 0;
+  if (g_winograd == 2) wino_r = 2;
+  else if (g_winograd == 3) wino_r = 4;
+  else if (g_winograd == 1) wino_r = g_winograd4_channels && wino_min >= g_winograd4_channels ? 4 : wino_min >= 128 ? 2 : 0;
+  if (wino_r && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 && group == 1 && c % BK == 0 &&
+      g_forced_tile < 0 && g_forced_split < 0) {
+    const int r = wino_r, positions = (r + 2) * (r + 2);
+    const long long tiles = wdh::wino_pitch(wdh::wino_tiles(r, n, oh, ow));  // (row length of V and M)
+    const size_t u_bytes = (size_t)positions * cout * c * 4, v_bytes = (size_t)positions * c * tiles * 4,
+                 m_bytes = (size_t)positions * cout * tiles * 4;
     if (tiles < 0x7fffffffLL && v_bytes < ((size_t)1 << 33) && m_bytes < ((size_t)1 << 33)) {
       // the transformed filters: kept from call to call when the caller vouches for the weights
       // (a block allocated while a graph is being recorded belongs to that graph, so nothing is kept then)
@@ -811,14 +826,14 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       bool u_kept = false, u_ready = false;
       if (flags & WDH_CONV_CONSTANT_WEIGHTS) {
         auto it = g_filters.find(hW);
-        if (it != g_filters.end() && it->second.cout == cout && it->second.c == c) {
+        if (it != g_filters.end() && it->second.cout == cout && it->second.c == c && it->second.r == r) {
           hU = it->second.u;
           u_kept = u_ready = true;
         } else if (!wdh::capturing()) {
           wdh::conv_forget_weights(hW);
           hU = wdh_alloc(u_bytes);
           if (hU) {
-            g_filters[hW] = FilterEntry{hU, cout, c};
+            g_filters[hW] = FilterEntry{hU, cout, c, r};
             u_kept = true;
           }
         }
@@ -828,21 +843,21 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       int rc = hU && hV && hM ? WDH_OK : WDH_ENOMEM;
       if (rc == WDH_OK) {
         float *U = (float *)wdh::resolve(hU, nullptr), *V = (float *)wdh::resolve(hV, nullptr);
-        if (!u_ready) rc = wdh::wino_filter_launch(p.A, U, cout, c);
-        if (rc == WDH_OK) rc = wdh::wino_input_launch(p.B, V, n, c, h, w, oh, ow, pt, pl);
+        if (!u_ready) rc = wdh::wino_filter_launch(r, p.A, U, cout, c);
+        if (rc == WDH_OK) rc = wdh::wino_input_launch(r, p.B, V, n, c, h, w, oh, ow, pt, pl);
       }
       if (rc == WDH_OK) {
         // (64x64 tiles: the 16 products have K = c, short against their extent; measured best on
         // every 3x3 layer shape of ResNet-50 and DETR, 35 against 44 us where the general choice
         // takes 128x128)
         g_tile_hint = T64x64;
-        rc = wdh_gemm(hU, hV, 0, hM, 16, cout, (int)tiles, c, (int64_t)cout * c, c, 1, (int64_t)c * tiles, tiles, 1, 0, 0,
-                      1.0f, 1.0f, WDH_EPI_NONE, 0);
+        rc = wdh_gemm(hU, hV, 0, hM, positions, cout, (int)tiles, c, (int64_t)cout * c, c, 1, (int64_t)c * tiles, tiles, 1,
+                      0, 0, 1.0f, 1.0f, WDH_EPI_NONE, 0);
         g_tile_hint = -1;
       }
       if (rc == WDH_OK) {
-        g_last_plan.form = WDH_FORM_CONV3X3_WINOGRAD;
-        rc = wdh::wino_output_launch((const float *)wdh::resolve(hM, nullptr), p.C, p.R, p.Y, n, cout, oh, ow,
+        g_last_plan.form = r == 2 ? WDH_FORM_CONV3X3_WINOGRAD : WDH_FORM_CONV3X3_WINOGRAD4;
+        rc = wdh::wino_output_launch(r, (const float *)wdh::resolve(hM, nullptr), p.C, p.R, p.Y, n, cout, oh, ow,
                                      epilogue == WDH_EPI_RELU);
       }
       // (the blocks go back to the pool at once: whoever gets them next is ordered behind these kernels)

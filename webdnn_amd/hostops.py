@@ -154,7 +154,8 @@ class HipContext:
 
     FORMS = ("gemm, B k-contiguous", "gemm, B n-contiguous", "conv, gathered taps", "conv, gathered taps (32-63)",
              "conv, gathered taps (flat loads)", "conv 1x1, X in place", "conv 3x3, LDS tile",
-             "conv 7x7 s2 stem, weights and patch in LDS", "conv 1x1 stride 2, X in place", "conv 3x3, F(2x2,3x3) transforms + batched product")
+             "conv 7x7 s2 stem, weights and patch in LDS", "conv 1x1 stride 2, X in place", "conv 3x3, F(2x2,3x3) transforms + batched product",
+             "conv 3x3, F(4x4,3x3) transforms + batched product")
 
     def last_plan(self):
         """Layout of the most recent Gemm / Conv launch: tile, whole tiles, tiles cut along K, chunks, form."""
