@@ -13,10 +13,14 @@ run is eager, the second records the run's kernels into a HIP graph, every timed
 graph (same kernels, same order, one launch) and reads the logits.  `value` = 32 * steps / total time.
 
 `roofline` is for the dominant kernels of that workload, the implicit-GEMM contraction kernels (the
-1x1 convs read X in place, the 3x3 stride-1 convs stage input rows in LDS, the rest gather taps; all
-share one tile schedule and epilogue): their algorithmic FLOPs (2*M*N*K per Conv/Gemm node, summed over the node list) over the device time of
+1x1 convs read X in place, the 3x3 stride-1 convs stage input rows in LDS or, from 128 channels on,
+run as F(2x2, 3x3) minimal filtering -- transforms around a batched product of the same kernel -- the
+rest gather taps; all share one tile schedule and epilogue): their algorithmic FLOPs (2*M*N*K per
+Conv/Gemm node as the direct sum needs them, summed over the node list) over the device time of
 the timed steps, measured with one HIP event pair on the library's stream around each graph replay
-(the step's three other kernels are inside that bracket, which makes the figure a lower bound).
+(the step's other kernels are inside that bracket, which makes the figure a lower bound).  Minimal
+filtering issues fewer multiplications than that numerator counts: `mfma_flops_issued_per_step` and
+`frac_issued` give what the matrix cores really execute per step and its share of the peak.
 Inside `roofline`, so that one record holds everything the metric names:
   kernels        Gemm 4096^3 and the config-3 Conv as single-kernel figures (ms, GFLOP/s, fraction of the
                  fp32 MFMA peak), each timed as replays of a HIP graph that holds the launches back to back,
@@ -27,7 +31,7 @@ Inside `roofline`, so that one record holds everything the metric names:
                  ({graph: false}), and the network at batch 128;
   other_configs  configs 2 and 5 with their device time;
   bandwidth_kernels_frac_of_8TBps  the HBM-bound kernels at the configs' shapes.
-`python bench.py --only layers` prints the per-layer table of the step's 54 contraction launches,
+`python bench.py --only layers` prints the per-layer table of the step's 54 Conv / Gemm nodes,
 `--only bandwidth` the bandwidth kernels in full, `--only kernels` the two single kernels (for profiler runs).
 `cpu_baseline` times the JavaScript restatement of the reference's CPU operators (oracle/js) through
 the same runner with backendOrder ["cpu"] in Node.js on one host core, on three images of the batch (one per run, about 20 s).
@@ -48,19 +52,25 @@ import numpy as np  # noqa: E402
 
 METRIC = "fp32 Gemm/Conv GFLOP/s (% MFMA peak) + ResNet-50 b32 images/sec, 1 MI355X"
 PEAK_FP32_MFMA_TFLOPS = 157.3
-# HBM-side bytes per contraction launch of the ResNet-50 step, averaged over its 54 launches (reduce
-# passes included): rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), factors from a 256 MiB
-# device copy; recorded in profiles/contraction_kernel_resnet50_b32.txt (bench.py cannot read
-# counters itself).  The partial sums of tiles cut along K are in it (written once, read once).
-TRAFFIC_BYTES_PER_LAUNCH = 86.8e6  # (86.81 in the latest profile)
+# HBM-side bytes of the ResNet-50 step per Conv / Gemm node (54 nodes; contraction kernels, reduce passes
+# and the transforms of the minimal-filtering convs): rocprofv3 --pmc FETCH_SIZE (x2.000) + WRITE_SIZE
+# (x1.000), factors from a 256 MiB device copy; recorded in profiles/contraction_kernel_resnet50_b32.txt
+# (bench.py cannot read counters itself).  The transform-domain tensors of the 13 minimal-filtering convs
+# (four times the conv's input and output, written once, read once or twice) and the partial sums of
+# tiles cut along K are in it; both live between consecutive launches and are counted in front of the
+# Infinity Cache.
+TRAFFIC_BYTES_PER_LAUNCH = 110.6e6  # (110.56 in the latest profile)
 CLI = os.path.join(ROOT, "webdnn_amd", "js", "cli", "run_model.js")
 ORACLE_JS = os.path.join(ROOT, "oracle", "js", "cpuOperators.js")
 
 
-def node_run(model_dir, input_path, backend, runs, warmup, extra):
+def node_run(model_dir, input_path, backend, runs, warmup, extra, options=None):
     cmd = ["node", CLI, "--model", model_dir, "--backend", backend, "--inputs", input_path,
            "--runs", str(runs), "--warmup", str(warmup)] + extra
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    env = dict(os.environ)
+    if options:
+        env["WDH_OPTIONS"] = options     # library options of the child process (wdh_set_option names)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env)
     if proc.returncode != 0:
         raise RuntimeError("node runner failed: %s" % proc.stderr[-2000:])
     return json.loads(proc.stdout.strip().splitlines()[-1])
@@ -100,7 +110,13 @@ def bench_resnet(steps, warmup, workdir):
     # no option at all: what a caller written for the reference does (the runner records the third run)
     host_in_graph = node_run(workdir, inp, "hip", steps, max(warmup, 3), ["--strict"])
     assert host_in_graph["graph"]["captured"], host_in_graph["graph"]
+    # the opt-in F(4x4, 3x3) form of the 3x3 convs: faster, but its logits miss the 1e-3 bar (1.7e-3)
+    f4 = node_run(workdir, inp, "hip", max(3, steps // 2), max(warmup, 2),
+                  ["--strict", "--resident-inputs", "--graph", "--measure-all"], options="conv3x3_f4x4_channels=64")
     return {
+        "f4x4_ms_per_step": sum(f4["msPerRun"]) / len(f4["msPerRun"]),
+        "f4x4_device_ms": sum(f4["deviceMsPerRun"]) / len(f4["deviceMsPerRun"]),
+        "flops_saved": g.flops_saved,
         "batch": batch, "flops": g.flops, "nodes": timed["nodes"], "ms_per_step": total_ms / steps,
         "images_per_s": batch * steps / total_ms * 1e3, "contraction_ms": contraction_ms,
         "contraction_launches": launches, "device_ms": all_ms,
@@ -460,9 +476,9 @@ def main():
     bandwidth = bench_bandwidth(args.steps, args.warmup)
 
     # The timed steps are graph replays: one HIP event pair brackets each replay on the library's
-    # stream.  That device time covers the 54 contraction launches plus the step's three other kernels
-    # (MaxPool, GlobalAveragePool, one copy: about 1 % of it), so FLOPs over it is a lower bound for
-    # the contraction kernels alone.
+    # stream.  That device time covers the 54 Conv / Gemm nodes (contraction launches, reduce passes,
+    # transforms) plus the step's three other kernels (MaxPool, GlobalAveragePool, one copy: about 1.5 %
+    # of it), so FLOPs over it is a lower bound for the contraction kernels alone.
     achieved = resnet["flops"] / resnet["graph_device_ms"] / 1e9
     batch = resnet["batch"]
     pick = lambda d, *keys: {k: d[k] for k in keys}
@@ -486,16 +502,24 @@ def main():
                                % resnet["nodes"]},
         "roofline": {
             "bound": "mfma",
-            "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3, gathered forms, stem; Gemm "
-                      "head), %d launches per step; device time = HIP events around each timed graph replay "
-                      "(whole step, MaxPool and GlobalAveragePool included)" % resnet["contraction_launches"],
+            "kernel": "contraction kernels (implicit-GEMM Conv: in-place 1x1, LDS-tile 3x3, F(2x2,3x3) minimal filtering "
+                      "for 3x3 from 128 channels on, gathered forms, stem; Gemm head), %d Conv/Gemm nodes per step; device "
+                      "time = HIP events around each timed graph replay (whole step: transforms, MaxPool and "
+                      "GlobalAveragePool included); achieved = direct-sum FLOPs (2MNK per node) / that time"
+                      % resnet["contraction_launches"],
             "achieved": round(achieved, 2),
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-            "traffic_note": "bytes/launch from rocprofv3 FETCH_SIZE+WRITE_SIZE, see profiles/; algorithmic 64.1e6",
+            "traffic_note": "bytes per Conv/Gemm node from rocprofv3 FETCH_SIZE+WRITE_SIZE, see profiles/; algorithmic "
+                            "64.1e6; the excess is the transform-domain tensors of the 13 F(2x2,3x3) convs (36.6e6 per "
+                            "node), which pass between consecutive launches through the Infinity Cache",
             "flops_per_step": resnet["flops"],
+            # what the matrix cores execute: minimal filtering replaces 36 multiplications per 2x2 block by 16
+            "mfma_flops_issued_per_step": resnet["flops"] - resnet["flops_saved"],
+            "frac_issued": round((resnet["flops"] - resnet["flops_saved"]) / resnet["graph_device_ms"] / 1e9
+                                 / PEAK_FP32_MFMA_TFLOPS, 4),
             "avg_launch_ms": round(resnet["graph_device_ms"] / resnet["contraction_launches"], 5),
             "step_device_ms": round(resnet["graph_device_ms"], 4),
             # the two single-kernel figures the metric names (graph replays of back-to-back launches)
@@ -513,6 +537,10 @@ def main():
                                    "and replays it (graph \"auto\")",
                 "host_input_node_loop_images_per_s": round(batch / resnet["ms_per_step_host_input_eager"] * 1e3, 1),
                 "resident_input_node_loop_ms_per_step": round(resnet["ms_per_step_eager"], 4),
+                "f4x4_option_images_per_s": round(batch / resnet["f4x4_ms_per_step"] * 1e3, 1),
+                "f4x4_option_device_ms": round(resnet["f4x4_device_ms"], 4),
+                "f4x4_option_note": "WDH_OPTIONS=conv3x3_f4x4_channels=64: 3x3 convs as F(4x4,3x3); not the default "
+                                    "because its logits differ from the CPU path's by 1.7e-3 (bar 1e-3)",
                 "batch128_device_frac_mfma_peak": large_batch["device_frac_mfma_peak"],
                 "batch128_images_per_s": large_batch["images_per_s"],
             },

@@ -255,6 +255,10 @@ class GraphBuilder:
         self.nodes, self.initializers, self.counter = [], [], 0
         self.seed = seed
         self.flops = 0          # 2*M*N*K of every Gemm / MatMul / Conv
+        # What the hip library's default plan saves of that on the matrix cores: its 3x3 stride-1 convs with
+        # at least 128 input and output channels run as F(2x2, 3x3), 16 products per 2x2 output block in place
+        # of 36 (flops - flops_saved is what the matrix cores execute; the transforms run on the vector units).
+        self.flops_saved = 0
         self.conv_gemm_nodes = 0
 
     def rng(self):
@@ -346,6 +350,9 @@ def _resnet_trunk(g, x, batch, size, width=64, blocks=(3, 4, 6, 3), init="he"):
         oh = (size[0] + 2 * pad - k) // stride + 1
         ow = (size[1] + 2 * pad - k) // stride + 1
         g.flops += 2 * batch * oh * ow * cout * cin * k * k
+        if k == 3 and stride == 1 and cin >= 128 and cout >= 128 and cin % 16 == 0:
+            blocks = (batch * ((oh + 1) // 2) * ((ow + 1) // 2) + 15) // 16 * 16
+            g.flops_saved += 2 * batch * oh * ow * cout * cin * 9 - 2 * blocks * cout * cin * 16
         g.conv_gemm_nodes += 1
         y = g.op("Conv", [x, name + "_w", name + "_b"], name, kernel_shape=[k, k], pads=[pad] * 4,
                  strides=[stride, stride], dilations=[1, 1], group=1)
