@@ -93,6 +93,10 @@ int wdh_device_info(char *name, int name_cap, int *compute_units,
  *   "conv3x3_f4x4_channels"  0 (default) or a channel count from which "conv3x3_winograd" 1 takes
  *                       F(4x4, 3x3) instead (64 is where it starts to win): for callers who can
  *                       trade the last digit for speed.
+ *   "memory_limit_mib"  0 (default) = no limit, or the most device memory, in MiB, that the buffer pool
+ *                       asks the driver for: an allocation beyond it first gives cached blocks back, then
+ *                       fails with WDH_ENOMEM.  Workspaces are subject to it: a conv that cannot get
+ *                       the tensors of its minimal-filtering form takes a direct form instead.
  *   "conv_stem"         1 (default) = a 7x7, stride-2, undilated convolution from 3 to 64
  *                       channels (the stem of an image network) runs in a kernel that keeps
  *                       all weights and a tile's input patch in LDS; 0 = it gathers taps

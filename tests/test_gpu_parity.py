@@ -1267,6 +1267,40 @@ def test_conv3x3_minimal_filtering_keeps_special_values_local_and_replays(ctx, m
         ctx.set_option("conv3x3_winograd", 1)
 
 
+def test_memory_limit_and_the_direct_form_as_fallback(ctx):
+    """memory_limit_mib caps what the pool asks of the driver: an allocation beyond it fails with WDH_ENOMEM
+    (after cached blocks went back), one inside it works, and a 3x3 conv that cannot get the transform-domain
+    tensors of its minimal-filtering form (here 2 x 16 x 256 x 3136 floats = 98 MiB) takes a direct form
+    instead of failing -- also when the caller vouches for the weights, and without leaving half-made kept
+    filters behind for the call after the limit is lifted."""
+    X, W, B = uni(16, 256, 28, 28, lo=0), he(256, 256, 3), nrm(256)
+    want = ref.conv(X, W, B, pads=[1, 1, 1, 1])
+    tx, tw, tb = (ctx.move_tensor(v) for v in (X, W, B))
+    ctx.sync()
+    capi.call("wdh_trim", 0)
+    stats = ctx.mem_stats()
+    reserved = stats["in_use"] + stats["cached"]
+    try:
+        ctx.set_option("memory_limit_mib", (reserved >> 20) + 64)
+        assert capi.load().wdh_alloc(128 << 20) == 0
+        assert "memory_limit_mib" in capi.last_error()
+        small = capi.load().wdh_alloc(8 << 20)
+        assert small > 0
+        capi.call("wdh_free", small)
+        for flag in (False, True):
+            y = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=flag)
+            assert ctx.last_plan()["form"] == "conv 3x3, LDS tile", ctx.last_plan()
+            assert_close_max(y.get_data(), want, GEMM_TOL, "direct form under the limit")
+            y.dispose()
+    finally:
+        ctx.set_option("memory_limit_mib", 0)
+    y = H.conv(ctx, tx, tw, tb, pads=[1, 1, 1, 1], constant_weights=True)
+    assert ctx.last_plan()["form"].startswith(WINOGRAD_FORMS[2]), ctx.last_plan()
+    assert_close_max(y.get_data(), want, GEMM_TOL, "minimal filtering once the limit is lifted")
+    for t in (y, tx, tw, tb):
+        t.dispose()
+
+
 @pytest.mark.parametrize("n,cin,h,w,cout,sh,group", [
     (4, 256, 56, 56, 128, 2, 1),       # the stride-2 1x1 convs that open ResNet-50's stages 2 and 3
     (4, 512, 28, 28, 1024, 2, 1),

@@ -19,6 +19,8 @@ void poison_capture();   // the open capture cannot be completed (wdh_graph_end 
 hipStream_t stream();
 int compute_units();
 int device();           // the device wdh_init selected
+// The pool asks the driver for at most `bytes` in total (0 = no limit); blocks it already holds stay.
+void set_memory_limit(uint64_t bytes);
 // Looks up the device address of the static workspace of wdh_gemm_static for `device`,
 // which must be the current device (called by wdh_init).
 int init_static_scratch(int device);

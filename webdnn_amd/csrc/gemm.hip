@@ -378,6 +378,11 @@ extern "C" int wdh_set_option(const char *name, int value) {
     g_halo = value;
     return WDH_OK;
   }
+  if (strcmp(name, "memory_limit_mib") == 0) {
+    if (value < 0) return fail(WDH_EINVAL, "wdh_set_option: memory_limit_mib %d (use 0 for none, or a size)", value);
+    wdh::set_memory_limit((uint64_t)value << 20);
+    return WDH_OK;
+  }
   return fail(WDH_EINVAL, "wdh_set_option: unknown option \"%s\"", name);
 }
 
@@ -841,8 +846,17 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
       }
       if (!hU) hU = wdh_alloc(u_bytes);
       const wdh_buf hV = wdh_alloc(v_bytes), hM = wdh_alloc(m_bytes);
-      int rc = hU && hV && hM ? WDH_OK : WDH_ENOMEM;
-      if (rc == WDH_OK) {
+      int rc = WDH_OK;
+      if (!(hU && hV && hM)) {
+        // no room for the transform-domain tensors: the direct forms below need none
+        if (hU && !u_kept) (void)wdh_free(hU);
+        if (u_kept && !u_ready) wdh::conv_forget_weights(hW);  // (registered above, never filled)
+        if (hV) (void)wdh_free(hV);
+        if (hM) (void)wdh_free(hM);
+        wdh::clear_error();
+        goto direct_forms;
+      }
+      {
         float *U = (float *)wdh::resolve(hU, nullptr), *V = (float *)wdh::resolve(hV, nullptr);
         if (!u_ready) rc = wdh::wino_filter_launch(r, p.A, U, cout, c);
         if (rc == WDH_OK) rc = wdh::wino_input_launch(r, p.B, V, n, c, h, w, oh, ow, pt, pl);
@@ -862,12 +876,14 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
                                      epilogue == WDH_EPI_RELU);
       }
       // (the blocks go back to the pool at once: whoever gets them next is ordered behind these kernels)
+      if (rc != WDH_OK && u_kept && !u_ready) wdh::conv_forget_weights(hW);  // (may not have been filled)
       if (hU && !u_kept) (void)wdh_free(hU);
       if (hV) (void)wdh_free(hV);
       if (hM) (void)wdh_free(hM);
       return rc;
     }
   }
+direct_forms:
   // 3x3, stride 1, no dilation, input channels in blocks of 8: taps read from an input
   // tile staged in LDS (conv3x3_halo_kernel)
   if (g_halo && small && kh == 3 && kw == 3 && sh == 1 && sw == 1 && dh == 1 && dw == 1 &&

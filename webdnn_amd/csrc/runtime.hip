@@ -58,6 +58,7 @@ struct Runtime {
   // pool: capacity -> cached blocks
   std::multimap<size_t, void *> cache;
   uint64_t in_use = 0, cached = 0, reserved = 0, peak = 0;
+  uint64_t limit = 0;  // "memory_limit_mib": the pool asks the driver for no more than this (0 = no limit)
   // pinned staging, ping-pong
   void *stage[2] = {nullptr, nullptr};
   hipEvent_t stage_done[2] = {nullptr, nullptr};   // downloads: one event per buffer
@@ -81,6 +82,12 @@ size_t round_up(size_t bytes) {
   size_t gran = bytes < (1u << 20) ? kSmallGranule : kLargeGranule;
   return (bytes + gran - 1) / gran * gran;
 }
+
+}  // namespace
+namespace wdh {
+void set_memory_limit(uint64_t bytes) { g.limit = bytes; }
+}  // namespace wdh
+namespace {
 
 void release_cache(size_t keep) {
   // Blocks may still be referenced by enqueued work: drain the stream first.
@@ -344,6 +351,12 @@ wdh_buf wdh_alloc(size_t bytes) {
         g.cache.erase(it);
       } else {
         void *p = nullptr;
+        if (g.limit && g.reserved + cap > g.limit && !g.capturing) release_cache(0);
+        if (g.limit && g.reserved + cap > g.limit) {
+          fail(WDH_ENOMEM, "wdh_alloc: %zu bytes on top of %llu reserved exceed memory_limit_mib (%llu MiB)", cap,
+               (unsigned long long)g.reserved, (unsigned long long)(g.limit >> 20));
+          return 0;
+        }
         hipError_t e = hipMalloc(&p, cap);
         if (e != hipSuccess && !g.capturing) {
           // give cached blocks back to the driver and retry once (this drains
