@@ -182,6 +182,42 @@ def test_conv_random_geometry(ctx, i):
                      % (n, cin, h, w, cout, k, pads, strides, dil, group))
 
 
+@pytest.mark.parametrize("i", range(24))
+def test_conv3x3_minimal_filtering_random_geometry(ctx, i):
+    """3x3 stride-1 convs through both minimal-filtering forms (and, every third case, through whatever the
+    plan picks) on random planes, pads 0..2 per side, channel counts in multiples of 16, with and without
+    bias, residual and Relu."""
+    r = rng_for("wino", i)
+    mode = [2, 3, 1][i % 3]
+    cin = 16 * int(r.integers(1, 13 if mode != 1 else 17))
+    cout = 16 * int(r.integers(1, 13 if mode != 1 else 17)) if i % 4 else int(r.integers(1, 40))
+    pads = [int(r.integers(0, 3)) for _ in range(4)]
+    h, w = int(r.integers(3, 30)), int(r.integers(3, 30))
+    n = int(r.integers(1, 6))
+    X = f32(r, (n, cin, h, w), -1 if i % 2 else 0, 1)
+    W = (f32(r, (cout, cin, 3, 3), -1, 1) * np.float32(np.sqrt(2.0 / (cin * 9)))).astype(np.float32)
+    Bs = f32(r, (cout,)) if i % 5 else None
+    want = ref.conv(X, W, Bs, None, 1, None, pads, None)
+    R = f32(r, want.shape) if i % 2 else None
+    if R is not None:
+        want = ref.binary("Add", want, R)
+    if i % 3 == 0:
+        want = ref.unary("Relu", want)
+    try:
+        ctx.set_option("conv3x3_winograd", mode)
+        got = H.conv(ctx, ctx.move_tensor(X), ctx.move_tensor(W), ctx.move_tensor(Bs) if Bs is not None else None,
+                     None, 1, None, pads, None, "relu" if i % 3 == 0 else None,
+                     ctx.move_tensor(R) if R is not None else None)
+        form = ctx.last_plan()["form"]
+    finally:
+        ctx.set_option("conv3x3_winograd", 1)
+    if mode != 1:
+        assert form.startswith("conv 3x3, F(%dx%d,3x3)" % ((2, 2) if mode == 2 else (4, 4))), form
+    assert tuple(got.dims) == want.shape
+    assert_close_max(got.get_data(), want, 1e-4, "3x3 n%d cin%d %dx%d cout%d pads%s mode %d (%s)"
+                     % (n, cin, h, w, cout, pads, mode, form))
+
+
 @pytest.mark.parametrize("i", range(20))
 def test_row_reductions_random_lengths(ctx, i):
     r = rng_for("rows", i)
