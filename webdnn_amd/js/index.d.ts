@@ -1,7 +1,6 @@
 // Entry points of the package (index.js).  Reference: src/descriptor_runner/index.ts:23-149 and
 // interface/core/runner.ts; `backendOptions.hip` and the `graph` run option are the additions.
-import { Backend } from "./interface/core/constants";
-import { Tensor } from "./interface/core/tensor";
+import { Backend, Tensor } from "./interface/core/contracts";
 import { WebDNNHipContext, WebDNNHipContextOption } from "./interface/backend/hip/hipContext";
 
 export interface InitOption {

@@ -1,9 +1,7 @@
 // Context of the hip backend (backend/hip/hipContextImpl.js) and the options that reach it through
 // WebDNN.load(directory, {backendOrder: ["hip", "cpu"], backendOptions: {hip: ...}}).  Shaped after
 // src/descriptor_runner/interface/backend/wasm/wasmContext.ts.
-import { BackendContext } from "../../core/backendContext";
-import { DataType } from "../../core/constants";
-import { Tensor } from "../../core/tensor";
+import { BackendContext, DataType, Tensor } from "../../core/contracts";
 import { HipDeviceInfo, HipMemStats, HipNative } from "./hipNative";
 import { HipTensor } from "./hipTensor";
 

@@ -1,7 +1,7 @@
 // Device tensor of the hip backend (backend/hip/hipTensorImpl.js).  Shaped after
 // src/descriptor_runner/interface/backend/wasm/wasmTensor.ts; `handle` and `alias` are what the hip
 // operators use beyond the Tensor contract.
-import { Tensor } from "../../core/tensor";
+import { Tensor } from "../../core/contracts";
 
 export interface HipTensor extends Tensor {
   readonly backend: "hip";
