@@ -1,5 +1,6 @@
-// 3x3 stride-1 convolution by the minimal-filtering algorithm F(2x2, 3x3) (Winograd): the
-// transforms around the products.
+// 3x3 stride-1 convolution by the minimal-filtering algorithms F(2x2, 3x3) and F(4x4, 3x3)
+// (Winograd): the transforms around the products.  F(2x2, 3x3) first; F(4x4, 3x3) follows the
+// same scheme further down.
 //
 // Semantics are those of the reference's Conv (src/descriptor_runner/operators/cpu/operators/
 // standard/conv.ts:134-221: im2col + matrix product, i.e. Y[o][oy][ox] = bias[o] +
@@ -151,8 +152,10 @@ __global__ __launch_bounds__(256) void wino_output_kernel(const float *__restric
 // The same scheme with a quarter of the direct form's multiplications per output: 36
 // products per 16 outputs (against 144), and 36 values of V per 16 outputs where F(2x2, 3x3) has
 // 64.  Its transforms multiply by 4, 5, 8 and divide by 6 and 24, so rounding errors are about
-// fifty times those of F(2x2, 3x3): 0.6-1.3e-5 of max|ref| on the ResNet-50 and DETR layers
-// against 1.5e-7 (the direct form: 1.5e-7), an eighth of the Gemm/Conv tolerance.
+// ten times those of F(2x2, 3x3): 0.6-1.9e-6 of max|ref| on the ResNet-50 and DETR layers
+// against 1.0-2.0e-7 (the direct form: 1.2-2.1e-7): a fiftieth of the Gemm/Conv tolerance, but
+// enough to show in the logits of a 50-layer network, which is why the plan does not pick it
+// unless asked.
 //     Bt = | 4  0 -5  0  1  0 |   G = | 1/4    0     0   |   At = | 1  1  1  1  1  0 |
 //          | 0 -4 -4  1  1  0 |       | -1/6  -1/6  -1/6  |        | 0  1 -1  2 -2  0 |
 //          | 0  4 -4 -1  1  0 |       | -1/6   1/6  -1/6  |        | 0  1  1  4  4  0 |
