@@ -28,7 +28,9 @@ Inside `roofline`, so that one record holds everything the metric names:
   end_to_end     the same ResNet-50 step with the batch handed over as a host tensor on every run
                  (runner.run([CPUTensor]) with no option: H2D inside the timed region; the runner's
                  default records the third run and replays it), the same through the node loop only
-                 ({graph: false}), and the network at batch 128;
+                 ({graph: false}), the throughput with two runs in flight (runner.submit / collect: batch
+                 i+1 enqueued on a second stream before batch i's logits are fetched), and the network
+                 at batch 128;
   other_configs  configs 2 and 5 with their device time;
   bandwidth_kernels_frac_of_8TBps  the HBM-bound kernels at the configs' shapes.
 `python bench.py --only layers` prints the per-layer table of the step's 54 Conv / Gemm nodes,
@@ -110,11 +112,22 @@ def bench_resnet(steps, warmup, workdir):
     # no option at all: what a caller written for the reference does (the runner records the third run)
     host_in_graph = node_run(workdir, inp, "hip", steps, max(warmup, 3), ["--strict"])
     assert host_in_graph["graph"]["captured"], host_in_graph["graph"]
+    # two runs in flight (runner.submit / runner.collect: run i+1 is enqueued on the library's second lane
+    # before the outputs of run i are fetched), input resident and input from the host; the first timed
+    # runs record the second lane and are left out of the mean
+    def in_flight(extra):
+        rep = node_run(workdir, inp, "hip", steps + 6, max(warmup, 3), ["--strict", "--in-flight"] + extra)
+        assert rep["graph"]["lanes"] == 2, rep["graph"]
+        tail = rep["msPerRun"][6:]
+        return sum(tail) / len(tail)
+    pipe_resident_ms = in_flight(["--resident-inputs"])
+    pipe_host_ms = in_flight([])
     # the opt-in F(4x4, 3x3) form of the 3x3 convs: faster, but its logits miss the 1e-3 bar (1.7e-3)
     f4 = node_run(workdir, inp, "hip", max(3, steps // 2), max(warmup, 2),
                   ["--strict", "--resident-inputs", "--graph", "--measure-all"], options="conv3x3_f4x4_channels=64")
     return {
         "f4x4_ms_per_step": sum(f4["msPerRun"]) / len(f4["msPerRun"]),
+        "two_in_flight_ms_per_step": pipe_resident_ms, "two_in_flight_host_input_ms_per_step": pipe_host_ms,
         "f4x4_device_ms": sum(f4["deviceMsPerRun"]) / len(f4["deviceMsPerRun"]),
         "flops_saved": g.flops_saved,
         "batch": batch, "flops": g.flops, "nodes": timed["nodes"], "ms_per_step": total_ms / steps,
@@ -537,6 +550,13 @@ def main():
                                    "and replays it (graph \"auto\")",
                 "host_input_node_loop_images_per_s": round(batch / resnet["ms_per_step_host_input_eager"] * 1e3, 1),
                 "resident_input_node_loop_ms_per_step": round(resnet["ms_per_step_eager"], 4),
+                "two_in_flight_images_per_s": round(batch / resnet["two_in_flight_ms_per_step"] * 1e3, 1),
+                "two_in_flight_host_input_images_per_s": round(batch / resnet["two_in_flight_host_input_ms_per_step"] * 1e3, 1),
+                "two_in_flight_frac_mfma_peak": round(resnet["flops"] / resnet["two_in_flight_ms_per_step"] / 1e9
+                                                      / PEAK_FP32_MFMA_TFLOPS, 4),
+                "two_in_flight_note": "runner.submit / runner.collect (an addition to the reference's API): batch i+1 is "
+                                      "enqueued on a second HIP stream before the logits of batch i are fetched; wall "
+                                      "clock per step in steady state, the fraction from that wall clock",
                 "f4x4_option_images_per_s": round(batch / resnet["f4x4_ms_per_step"] * 1e3, 1),
                 "f4x4_option_device_ms": round(resnet["f4x4_device_ms"], 4),
                 "f4x4_option_note": "WDH_OPTIONS=conv3x3_f4x4_channels=64: 3x3 convs as F(4x4,3x3); not the default "
@@ -558,6 +578,8 @@ def main():
         "conv_c3_frac_mfma_peak": kernels["conv_c3"]["frac_mfma_peak"],
         "host_input_images_per_s": round(batch / resnet["ms_per_step_host_input"] * 1e3, 1),
         "host_input_node_loop_images_per_s": round(batch / resnet["ms_per_step_host_input_eager"] * 1e3, 1),
+        "two_in_flight_images_per_s": round(batch / resnet["two_in_flight_ms_per_step"] * 1e3, 1),
+        "two_in_flight_host_input_images_per_s": round(batch / resnet["two_in_flight_host_input_ms_per_step"] * 1e3, 1),
         "device": resnet["device"],
     }
     if baseline is not None:

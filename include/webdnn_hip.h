@@ -183,7 +183,25 @@ int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes);
  * src/shader/wasm/src/kernels/standard/copy.cpp:6-8. */
 int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
              size_t bytes);
+/* Waits for the work of the current lane (see wdh_set_lane). */
 int wdh_sync(void);
+
+/* Lanes: two runs in flight.  No counterpart in the reference (its backends run one graph at a time);
+ * for callers that keep a second batch on its way while the first computes.  A lane is a HIP stream of
+ * default priority; lane 0 is the stream everything runs on unless told otherwise.  wdh_set_lane(1)
+ * makes lane 1 the current one: wdh_write, wdh_read, wdh_copy, wdh_sync, wdh_event_record,
+ * wdh_graph_begin / _end / _launch then work on it, concurrently with what lane 0 still has queued.
+ * Side lanes are for captured runs and their transfers: an operator call (wdh_gemm, wdh_conv2d, ...) on
+ * a side lane is legal only while a graph is being recorded there and fails with WDH_ESTATE otherwise.
+ * What the library guards by itself: a block freed while a side lane has work in flight waits for that
+ * lane first; an allocation or a capture on a side lane waits for lane 0; launches that run as streams
+ * of K slabs use a workspace of the lane's own (WDH_STATIC_SCRATCH_BYTES from the driver when the lane is
+ * first used), so a run recorded on a side lane computes bit for bit what it computes on lane 0;
+ * wdh_gemm_static is refused there (its workspace is lane 0's).  What the caller guards: a buffer written on one lane and read on another needs a
+ * wdh_sync (or wdh_read) on the first in between.  Not possible while capturing. */
+#define WDH_LANES 2
+int wdh_set_lane(int lane);
+
 /* Pool accounting: bytes handed out, bytes cached in the pool, high-water
  * mark of hipMalloc'ed bytes (cf. perfTotalMemory,
  * backend/wasm/wasmTensorImpl.ts:29-35).  Any pointer may be NULL. */

@@ -13,6 +13,7 @@ let inUse = 0, peak = 0;
 const calls = {};
 const graphOwned = new Set(); // handles freed while capturing: their memory stays with the graph
 const options = {};
+let currentLane = 0; // wdh_set_lane: everything here runs at once, so a lane is only remembered
 
 function count(name) {
   calls[name] = (calls[name] || 0) + 1;
@@ -94,6 +95,11 @@ const native = {
     buf(dst).set(buf(src).subarray(soff, soff + bytes), doff);
   },
   sync() {},
+  setLane(lane) {
+    if (lane !== 0 && lane !== 1) throw new Error("wdh_set_lane failed (-2): lane " + lane);
+    count("setLane");
+    currentLane = lane;
+  },
   memStats() {
     return { inUse, cached: 0, peak };
   },

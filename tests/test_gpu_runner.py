@@ -200,9 +200,32 @@ def test_graph_replay_equals_eager_runs(tmp_path):
     eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True)
     for runs, want in ((2, eb), (3, ea), (6, eb), (7, ea)):
         got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs)
-        assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
+        assert rep["graph"] == {"captured": True, "lanes": 1, "unsupported": None}, rep["graph"]
         assert rep["stats"]["graphReplay"] is True
         assert_bit_exact(got[0], want[0], "run %d of a graph-mode session" % runs)
+
+
+def test_two_runs_in_flight_equal_eager_runs(tmp_path):
+    """runner.submit / runner.collect: run i+1 is enqueued on the library's other lane before the outputs of run
+    i are fetched.  Inputs alternate from run to run; whatever the session length, the last run's outputs must
+    equal the eager run of the input it was given bit for bit (each lane replays its own recording of the same
+    node loop: same kernels in the same order, stream-scheduled launches included, which have a workspace
+    per lane), and from the fifth run on (the fourth with {graph: true}) both lanes hold a captured run."""
+    data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    ea, _ = node_runner.run_model(str(tmp_path), [Xa], "hip", strict=True, extra=["--no-graph"])
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True, extra=["--no-graph"])
+    for flags in (("--in-flight",), ("--in-flight", "--graph")):
+        first_both = 5 if flags == ("--in-flight",) else 4   # (auto: two eager runs, then lane 0, lane 0 again, lane 1)
+        for runs, want in ((2, eb), (3, ea), (4, eb), (5, ea), (6, eb), (9, ea), (12, eb)):
+            for resident in (False, True):
+                got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs, resident=resident, flags=flags)
+                assert rep["graph"]["unsupported"] is None, rep["graph"]
+                assert rep["graph"]["lanes"] == (2 if runs >= first_both else (1 if runs >= first_both - 2 else 0)), (flags, runs, rep["graph"])
+                assert list(rep["stats"]["nodesByBackend"]) == ["hip"]
+                assert_bit_exact(got[0], want[0], "run %d of a session with two runs in flight %s" % (runs, flags))
 
 
 def test_runs_without_an_option_are_replayed_from_the_third_on(tmp_path):
@@ -235,7 +258,7 @@ def test_graph_replay_with_two_resident_device_inputs(tmp_path):
     assert np.abs(ea[0] - eb[0]).max() > 0
     for runs, want in ((2, eb), (3, ea), (4, eb), (5, ea), (8, eb)):
         got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs, resident=True)
-        assert rep["graph"] == {"captured": True, "unsupported": None}, rep["graph"]
+        assert rep["graph"] == {"captured": True, "lanes": 1, "unsupported": None}, rep["graph"]
         assert_bit_exact(got[0], want[0], "run %d with resident inputs" % runs)
 
 

@@ -385,12 +385,30 @@ def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native, flags=("--gra
     return g3, g4, eager_a, eager_b, rep4
 
 
+def test_two_runs_in_flight_on_the_host_path(tmp_path):
+    """runner.submit / runner.collect against the stand-in addon: whatever the session length, the last run's
+    outputs equal the eager run of its input; the second lane is recorded once, every pipelined run brackets its
+    work with lane switches, and nothing but the initializer copies outlives disposeGraph."""
+    data, _ = modelgen.resnet50_model(batch=2, image=32, width=8, blocks=(1, 1, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    g5, g8, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"input": Xa}, {"input": Xb}, True,
+                                          flags=("--in-flight",), runs=(5, 8))
+    assert rep["graph"] == {"captured": True, "lanes": 2, "unsupported": None}
+    assert_bit_exact(g5[0], ea[0], "fifth run (first one on the second lane)")
+    assert_bit_exact(g8[0], eb[0], "eighth run")
+    # 8 runs: 2 eager, run 3 records lane 0 and launches, runs 4, 6, 8 replay lane 0, run 5 records lane 1, 7 replays it
+    assert rep["nativeCalls"]["graphBegin"] == 2 and rep["nativeCalls"]["graphLaunch"] == 6
+    assert rep["nativeCalls"]["setLane"] >= 2 * 5
+    assert rep["liveBuffers"] == rep["initializerCopies"]
+
+
 def test_graph_replay_on_the_host_path(tmp_path):
     data, _ = modelgen.resnet50_model(batch=2, image=32, width=8, blocks=(1, 1, 1, 1), classes=10)
     Xa = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
     Xb = np.random.default_rng(3).standard_normal((2, 3, 32, 32)).astype(np.float32)
     g3, g4, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"input": Xa}, {"input": Xb}, True)
-    assert rep["graph"] == {"captured": True, "unsupported": None}
+    assert rep["graph"] == {"captured": True, "lanes": 1, "unsupported": None}
     assert rep["stats"]["graphReplay"] is True and list(rep["stats"]["nodesByBackend"]) == ["hip"]
     assert_bit_exact(g3[0], ea[0], "third run (replay, first input)")
     assert_bit_exact(g4[0], eb[0], "fourth run (replay, second input)")
@@ -406,7 +424,7 @@ def test_a_caller_that_passes_no_option_gets_the_graph_after_two_runs(tmp_path):
     Xa = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
     Xb = np.random.default_rng(3).standard_normal((2, 3, 32, 32)).astype(np.float32)
     g5, g6, ea, eb, rep = _graph_vs_eager(tmp_path, data, {"input": Xa}, {"input": Xb}, True, flags=(), runs=(5, 6))
-    assert rep["graph"] == {"captured": True, "unsupported": None}
+    assert rep["graph"] == {"captured": True, "lanes": 1, "unsupported": None}
     assert rep["stats"]["graphReplay"] is True
     assert_bit_exact(g5[0], ea[0], "fifth run (replay, first input)")
     assert_bit_exact(g6[0], eb[0], "sixth run (replay, second input)")

@@ -34,6 +34,7 @@ SIGNATURES = {
     "wdh_read": (_c.c_int, [c_buf, _c.c_size_t, _c.c_void_p, _c.c_size_t]),
     "wdh_copy": (_c.c_int, [c_buf, _c.c_size_t, c_buf, _c.c_size_t, _c.c_size_t]),
     "wdh_sync": (_c.c_int, []),
+    "wdh_set_lane": (_c.c_int, [_c.c_int]),
     "wdh_mem_stats": (_c.c_int, [_u64p, _u64p, _u64p]),
     "wdh_trim": (_c.c_int, [_c.c_size_t]),
     "wdh_graph_begin": (_c.c_int, []),

@@ -285,6 +285,7 @@ extern "C" int wdh_attention(wdh_buf hQ, wdh_buf hK, wdh_buf hV, wdh_buf hY, int
                              int tk, int d, int64_t sQb, int64_t sQi, int64_t sKb, int64_t sKj,
                              int64_t sVb, int64_t sVj, int64_t sYb, int64_t sYi, float alpha) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (batch < 0 || tq < 0 || tk < 0 || d < 0) return fail(WDH_EINVAL, "wdh_attention: negative extent");
   if (d != 32 && d != 64 && d != 128)
     return fail(WDH_EINVAL, "wdh_attention: head dimension %d (32, 64 and 128 are built)", d);

@@ -19,6 +19,7 @@ void poison_capture();   // the open capture cannot be completed (wdh_graph_end 
 hipStream_t stream();
 int compute_units();
 int device();           // the device wdh_init selected
+int lane();             // the current lane (wdh_set_lane)
 // The pool asks the driver for at most `bytes` in total (0 = no limit); blocks it already holds stay.
 void set_memory_limit(uint64_t bytes);
 // Looks up the device address of the static workspace of wdh_gemm_static for `device`,
@@ -28,6 +29,7 @@ int init_static_scratch(int device);
 int init_attention();
 // Device resources of the contraction kernels that outlive a call (called by wdh_init / at shutdown).
 int init_contraction(int device);
+int contraction_lane_init(int lane);   // (when wdh_set_lane creates a side lane)
 void release_contraction();
 // The buffer behind `h` is about to be freed or overwritten: drops what the conv code derived from it.
 void conv_forget_weights(wdh_buf h);
@@ -68,6 +70,15 @@ void release_conv_tables();
     if (!wdh::initialised())                                                 \
       return wdh::fail(WDH_ESTATE, "%s: wdh_init() has not succeeded",       \
                        __func__);                                            \
+  } while (0)
+
+// Operator entry points: side lanes take recorded work only (their buffers come from a pool whose
+// hand-overs are ordered on lane 0).
+#define WDH_REQUIRE_COMPUTE_LANE()                                           \
+  do {                                                                       \
+    if (wdh::lane() != 0 && !wdh::capturing())                               \
+      return wdh::fail(WDH_ESTATE, "%s: lane %d takes recorded work only (wdh_graph_begin first, or wdh_set_lane(0))", \
+                       __func__, wdh::lane());                               \
   } while (0)
 
 #define WDH_HIP_CHECK(expr)                                                  \

@@ -1728,6 +1728,7 @@ extern LastPlan g_last_plan;
 extern int g_stream_spin;
 extern unsigned *g_stream_error_dev;
 float *static_scratch();     // device address of the static workspace on the current device, or null
+float *stream_workspace();   // slots and flags of stream launches on the current lane: the static workspace on lane 0
 TileId pick_tile(int m, int n, int nz);
 
 // How the tiles of one launch are spread over the chip.
@@ -1758,7 +1759,7 @@ int launch_planned(Params &p, int nz, bool conv, int kgran, int max_wgs_per_cu, 
   const int slabs = (p.k + kgran - 1) / kgran;
   if (const int wgs = tiles <= 0x7fffffffLL && max_wgs_per_cu > 0
                           ? stream_width(tiles, slabs, kgran, w, BM * BN, max_wgs_per_cu) : 0) {
-    float *base = static_scratch();
+    float *base = stream_workspace();
     p.stream = 1;
     p.sk_wgs = wgs;
     p.sk_slabs = slabs;

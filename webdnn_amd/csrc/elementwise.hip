@@ -404,6 +404,7 @@ extern "C" int wdh_binary(int op, int dtype, wdh_buf hL, wdh_buf hR, wdh_buf hY,
                           int ndim, const int32_t *out_shape,
                           const int64_t *strides_l, const int64_t *strides_r) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (op < WDH_BIN_ADD || op > WDH_BIN_POW)
     return fail(WDH_EINVAL, "wdh_binary: unknown op %d", op);
   if (dtype != 0 && dtype != 1)
@@ -480,6 +481,7 @@ extern "C" int wdh_binary(int op, int dtype, wdh_buf hL, wdh_buf hR, wdh_buf hY,
 
 extern "C" int wdh_unary(int op, int dtype, wdh_buf hX, wdh_buf hY, size_t length) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (op < WDH_UN_RELU || op > WDH_UN_RECIPROCAL)
     return fail(WDH_EINVAL, "wdh_unary: unknown op %d", op);
   if (dtype != 0 && dtype != 1)
@@ -513,6 +515,7 @@ extern "C" int wdh_unary(int op, int dtype, wdh_buf hX, wdh_buf hY, size_t lengt
 
 extern "C" int wdh_cast(int from_dtype, int to_dtype, wdh_buf hX, wdh_buf hY, size_t length) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if ((from_dtype != 0 && from_dtype != 1) || (to_dtype != 0 && to_dtype != 1))
     return fail(WDH_EINVAL, "wdh_cast: dtype %d -> %d (0 = float32, 1 = int32)", from_dtype,
                 to_dtype);

@@ -97,6 +97,10 @@ int init_static_scratch(int device) {
 namespace wdhc {
 
 float *static_scratch() { return g_scratch_ptr[wdh::device()]; }
+// Side lanes: a workspace of the same layout from the driver (contraction_lane_init), so that what is
+// recorded on a side lane takes the same kernels and adds in the same order as on lane 0.
+static float *g_lane_workspace[WDH_LANES] = {};
+float *stream_workspace() { return wdh::lane() == 0 ? static_scratch() : g_lane_workspace[wdh::lane()]; }
 
 
 // Tile choice for Gemm / MatMul, from sweeps of all tile shapes over 30 problem sizes:
@@ -234,7 +238,7 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather, int kgra
 // Whether (and how wide) a launch runs as a stream of K slabs: workgroups per XCD, 0 = not.
 // `w` is what the tile-per-workgroup plan would do.
 int stream_width(long long tiles, int slabs, int kgran, const WorkPlan &w, int tile_floats, int max_wgs_per_cu) {
-  if (!g_stream || g_forced_split >= 1 || !g_scratch_ptr[wdh::device()] || !g_stream_error_dev || tiles <= 0 || slabs <= 0) return 0;
+  if (!g_stream || g_forced_split >= 1 || !stream_workspace() || !g_stream_error_dev || tiles <= 0 || slabs <= 0) return 0;
   const long long cus = wdh::compute_units();
   if (g_stream == 1) {
     // Measured on the ResNet-50 and DETR layer shapes: resident workgroups that walk segments
@@ -403,6 +407,10 @@ extern "C" int wdh_gemm_static(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
                                int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
                                float beta, int epilogue, wdh_buf hR) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
+  if (wdh::lane() != 0)
+    return fail(WDH_ESTATE, "wdh_gemm_static: the static workspace belongs to lane 0 (a run recorded on lane %d "
+                            "could be replayed next to one that uses it)", wdh::lane());
   g_static_scratch = true;
   const int rc = wdh_gemm(hA, hB, hC, hY, batch, m, n, k, sAb, sA0, sA1, sBb, sB0, sB1, sC0, sC1,
                           alpha, beta, epilogue, hR);
@@ -425,6 +433,7 @@ extern "C" int wdh_gemm_ex(wdh_buf hA, wdh_buf hB, wdh_buf hC, wdh_buf hY,
                            int64_t sB1, int64_t sC0, int64_t sC1, float alpha,
                            float beta, int epilogue, wdh_buf hR, int64_t sYb, int64_t sY0) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (batch < 0 || m < 0 || n < 0 || k < 0)
     return fail(WDH_EINVAL, "wdh_gemm: negative extent (batch=%d m=%d n=%d k=%d)",
                 batch, m, n, k);
@@ -593,6 +602,7 @@ int flush_group() {
 extern "C" int wdh_linear_group(int count, const wdh_buf *hA, const wdh_buf *hW, const wdh_buf *hBias,
                                 const wdh_buf *hY, const int *m, const int *n, const int *k, int epilogue) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (count < 0 || count > 16) return fail(WDH_EINVAL, "wdh_linear_group: %d problems (0..16)", count);
   if (count > 0 && (!hA || !hW || !hY || !m || !n || !k)) return fail(WDH_EINVAL, "wdh_linear_group: NULL array");
   // the results must be distinct buffers, none of them an input: the products run in no particular order
@@ -682,7 +692,28 @@ int init_contraction(int device) {
   }
   return WDH_OK;
 }
+// A side lane's own slots and flags for launches scheduled as streams of K slabs (they may run next to
+// lane 0's, so they cannot share its static workspace).  Called once, when the lane is created.
+int contraction_lane_init(int lane) {
+  if (lane <= 0 || lane >= WDH_LANES || wdhc::g_lane_workspace[lane]) return WDH_OK;
+  void *ptr = nullptr;
+  if (hipMalloc(&ptr, WDH_STATIC_SCRATCH_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(WDH_ENOMEM, "wdh_set_lane: %u bytes of workspace for lane %d", (unsigned)WDH_STATIC_SCRATCH_BYTES, lane);
+  }
+  if (hipMemset((float *)ptr + SK_PARTIAL_FLOATS, 0, (size_t)SK_FLAG_WORDS * 4) != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipFree(ptr);
+    return fail(WDH_EHIP, "wdh_set_lane: clearing the workspace flags of lane %d", lane);
+  }
+  wdhc::g_lane_workspace[lane] = (float *)ptr;
+  return WDH_OK;
+}
 void release_contraction() {
+  for (float *&ws : wdhc::g_lane_workspace) {
+    if (ws) (void)hipFree(ws);
+    ws = nullptr;
+  }
   g_filters.clear();  // (the blocks go with the pool)
   if (g_stream_error) (void)hipHostFree(g_stream_error);
   g_stream_error = g_stream_error_dev = nullptr;
@@ -693,6 +724,8 @@ int contraction_check() {
   *reinterpret_cast<volatile unsigned *>(g_stream_error) = 0;
   float *base = g_scratch_ptr[device()];
   if (base) (void)hipMemset(base + SK_PARTIAL_FLOATS, 0, (size_t)SK_FLAG_WORDS * 4);
+  for (float *ws : wdhc::g_lane_workspace)
+    if (ws) (void)hipMemset(ws + SK_PARTIAL_FLOATS, 0, (size_t)SK_FLAG_WORDS * 4);
   return fail(WDH_EHIP, "a contraction kernel gave up waiting for a partial tile of a neighbouring workgroup; "
                         "results since the last synchronisation are not valid");
 }
@@ -711,6 +744,7 @@ extern "C" int wdh_conv2d_ex(wdh_buf hX, wdh_buf hW, wdh_buf hBias, wdh_buf hY,
                              int pt, int pl, int pb, int pr, int sh, int sw,
                              int dh, int dw, int group, int epilogue, wdh_buf hR, int flags) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (flags & ~WDH_CONV_CONSTANT_WEIGHTS) return fail(WDH_EINVAL, "wdh_conv2d_ex: unknown flags %d", flags);
   if (n < 0 || c <= 0 || h <= 0 || w <= 0 || cout <= 0 || kh <= 0 || kw <= 0 ||
       sh <= 0 || sw <= 0 || dh <= 0 || dw <= 0 || group <= 0 || pt < 0 ||

@@ -483,6 +483,7 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
                              int oh, int ow, int kh, int kw, int pt, int pl, int sh,
                              int sw, int dh, int dw) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (n < 0 || c < 0 || h <= 0 || w <= 0 || oh < 0 || ow < 0 || kh <= 0 || kw <= 0 ||
       sh <= 0 || sw <= 0 || dh <= 0 || dw <= 0 || pt < 0 || pl < 0)
     return fail(WDH_EINVAL, "wdh_maxpool2d: bad geometry");
@@ -551,6 +552,7 @@ extern "C" int wdh_maxpool2d(wdh_buf hX, wdh_buf hY, int n, int c, int h, int w,
 extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
                              const int32_t *out_shape, const int64_t *in_strides) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (ndim < 0 || ndim > MAXD)
     return fail(WDH_EINVAL, "wdh_transpose: ndim %d outside 0..%d", ndim, MAXD);
   if (ndim > 0 && (!out_shape || !in_strides))
@@ -642,6 +644,7 @@ extern "C" int wdh_transpose(wdh_buf hX, wdh_buf hY, int ndim,
 extern "C" int wdh_gather(wdh_buf hD, wdh_buf hI, wdh_buf hY, int64_t outer,
                           int axis_len, int64_t inner, int64_t n_idx) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (outer < 0 || axis_len < 0 || inner < 0 || n_idx < 0)
     return fail(WDH_EINVAL, "wdh_gather: negative extent");
   const long long total = (long long)outer * n_idx * inner;
@@ -663,6 +666,7 @@ extern "C" int wdh_strided_copy(wdh_buf hX, int64_t x_offset, wdh_buf hY, int64_
                                 int ndim, const int32_t *shape, const int64_t *x_strides,
                                 const int64_t *y_strides) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (ndim < 0 || ndim > MAXD)
     return fail(WDH_EINVAL, "wdh_strided_copy: ndim %d outside 0..%d", ndim, MAXD);
   if (ndim > 0 && (!shape || !x_strides || !y_strides))

@@ -389,6 +389,7 @@ using wdh::fail;
 
 extern "C" int wdh_softmax(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (int rc = check_rows("wdh_softmax", outer, len)) return rc;
   if (outer == 0 || len == 0) return WDH_OK;
   void *px, *py;
@@ -476,18 +477,21 @@ int layernorm_launch(const char *who, wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_bu
 extern "C" int wdh_layernorm(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY,
                              int64_t outer, int len, float eps) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   return layernorm_launch("wdh_layernorm", hX, hG, hB, hY, 0, 0, outer, len, eps);
 }
 
 extern "C" int wdh_layernorm_add(wdh_buf hX, wdh_buf hG, wdh_buf hB, wdh_buf hY, wdh_buf hP, wdh_buf hY2,
                                  int64_t outer, int len, float eps) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (!hP || !hY2) return fail(WDH_EINVAL, "wdh_layernorm_add: P and Y2 are required");
   return layernorm_launch("wdh_layernorm_add", hX, hG, hB, hY, hP, hY2, outer, len, eps);
 }
 
 extern "C" int wdh_reduce_mean(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (int rc = check_rows("wdh_reduce_mean", outer, len)) return rc;
   if (outer == 0) return WDH_OK;
   if (len == 0) return fail(WDH_EINVAL, "wdh_reduce_mean: empty reduction");
@@ -511,6 +515,7 @@ extern "C" int wdh_reduce_mean(wdh_buf hX, wdh_buf hY, int64_t outer, int len) {
 extern "C" int wdh_reduce_axis(wdh_buf hX, wdh_buf hY, int64_t outer, int red, int64_t inner,
                                int64_t divisor) {
   WDH_REQUIRE_INIT();
+  WDH_REQUIRE_COMPUTE_LANE();
   if (outer < 0 || red < 0 || inner < 0) return fail(WDH_EINVAL, "wdh_reduce_axis: negative extent");
   if (divisor <= 0) return fail(WDH_EINVAL, "wdh_reduce_axis: divisor %lld", (long long)divisor);
   const long long results = (long long)outer * inner;

@@ -50,7 +50,12 @@ struct GraphRec {
 struct Runtime {
   bool ready = false;
   int device = -1;
-  hipStream_t stream = nullptr;
+  hipStream_t stream = nullptr;            // the current lane's stream: every call works on this one
+  hipStream_t lanes[WDH_LANES] = {};       // lanes[0] is created by wdh_init, the others on first use
+  int lane = 0;
+  // lanes >= 1: work may have been enqueued since the lane was last waited for.  The pool hands blocks
+  // from lane to lane, so whoever frees a block first waits for these lanes (settle_side_lanes).
+  bool lane_dirty[WDH_LANES] = {};
   hipDeviceProp_t prop;
   // handle table; handle = index + 1
   std::vector<Slot> slots;
@@ -89,10 +94,27 @@ void set_memory_limit(uint64_t bytes) { g.limit = bytes; }
 }  // namespace wdh
 namespace {
 
+// Waits for the work of every lane (pool blocks and graph arenas may be referenced from any of them).
+void drain_lanes() {
+  for (hipStream_t s : g.lanes)
+    if (s) (void)hipStreamSynchronize(s);
+}
+
+// Before a block goes back to the pool (where the next taker may sit on another lane): waits for the side
+// lanes that have work in flight.  Lane 0 needs no wait: what is allocated on a side lane waits for it.
+void settle_side_lanes() {
+  if (g.capturing) return;  // (wdh_graph_begin has settled them, and the host has enqueued nothing since)
+  for (int i = 1; i < WDH_LANES; i++)
+    if (g.lanes[i] && g.lane_dirty[i]) {
+      (void)hipStreamSynchronize(g.lanes[i]);
+      g.lane_dirty[i] = false;
+    }
+}
+
 void release_cache(size_t keep) {
-  // Blocks may still be referenced by enqueued work: drain the stream first.
+  // Blocks may still be referenced by enqueued work: drain the streams first.
   if (g.cached <= keep) return;
-  (void)hipStreamSynchronize(g.stream);
+  drain_lanes();
   for (auto it = g.cache.begin(); it != g.cache.end() && g.cached > keep;) {
     (void)hipFree(it->second);
     g.cached -= it->first;
@@ -104,6 +126,7 @@ void release_cache(size_t keep) {
 // Returns the blocks of graph `id` that no handle holds to the general pool and
 // hands the rest over to their handles.
 void dissolve_graph(int id) {
+  settle_side_lanes();  // (a replay of this graph may be in flight on one of them)
   GraphRec &r = g.graphs[id];
   if (r.exec) (void)hipGraphExecDestroy(r.exec);
   if (r.graph) (void)hipGraphDestroy(r.graph);
@@ -134,6 +157,7 @@ bool initialised() { return g.ready; }
 bool capturing() { return g.capturing != 0; }
 void poison_capture() { g.capture_failed = true; }
 hipStream_t stream() { return g.stream; }
+int lane() { return g.lane; }
 int compute_units() { return g.prop.multiProcessorCount; }
 int device() { return g.device; }
 
@@ -215,7 +239,9 @@ static int init_device(int device) {
     return fail(WDH_ENODEV,
                 "wdh_init: device %d is %s; this library holds gfx950 code only",
                 device, g.prop.gcnArchName);
-  WDH_HIP_CHECK(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
+  WDH_HIP_CHECK(hipStreamCreateWithFlags(&g.lanes[0], hipStreamNonBlocking));
+  g.stream = g.lanes[0];
+  g.lane = 0;
   for (int i = 0; i < 2; i++) {
     if (hipHostMalloc(&g.stage[i], kStagingBytes, hipHostMallocDefault) !=
         hipSuccess)
@@ -271,7 +297,7 @@ static void release_everything() {
     if (dropped) (void)hipGraphDestroy(dropped);
     g.capturing = 0;
   }
-  if (g.stream) (void)hipStreamSynchronize(g.stream);
+  drain_lanes();
   for (size_t i = 0; i < g.graphs.size(); i++)
     if (g.graphs[i].live) dissolve_graph((int)i);
   g.graphs.clear();
@@ -301,8 +327,12 @@ static void release_everything() {
   }
   if (g.dummy) (void)hipFree(g.dummy);
   g.dummy = nullptr;
-  if (g.stream) (void)hipStreamDestroy(g.stream);
+  for (hipStream_t &s : g.lanes) {
+    if (s) (void)hipStreamDestroy(s);
+    s = nullptr;
+  }
   g.stream = nullptr;
+  g.lane = 0;
   g.ready = false;
   g.device = -1;
 }
@@ -328,6 +358,9 @@ wdh_buf wdh_alloc(size_t bytes) {
     s.ptr = g.dummy;
     s.cap = 0;
   } else {
+    // a block taken on a side lane may have been freed by work still in flight on lane 0
+    // (not while recording: wdh_graph_begin has waited, and the host has been on this lane since)
+    if (g.lane != 0 && !g.capturing) (void)hipStreamSynchronize(g.lanes[0]);
     const size_t cap = round_up(bytes);
     const auto fits = [cap](size_t have) { return have <= cap + cap / 4; };
     s.arena = g.capturing;
@@ -399,6 +432,7 @@ int wdh_free(wdh_buf h) {
   wdh::conv_forget_weights(h);
   Slot &s = g.slots[h - 1];
   if (s.cap) {
+    settle_side_lanes();
     if (s.arena && g.graphs[s.arena - 1].live) {
       // memory of a captured graph: stays with it
       g.graphs[s.arena - 1].free_blocks.emplace(s.cap, s.ptr);
@@ -436,6 +470,9 @@ int wdh_graph_begin(void) {
   WDH_REQUIRE_INIT();
   if (g.capturing) return fail(WDH_ESTATE, "wdh_graph_begin: a capture is already open");
   if (int rc = wait_for_uploads()) return rc;
+  // the blocks the capture takes from the pool, or gives back to it, may still be in use on another lane
+  settle_side_lanes();
+  if (g.lane != 0) WDH_HIP_CHECK(hipStreamSynchronize(g.lanes[0]));
   int id = -1;
   for (size_t i = 0; i < g.graphs.size(); i++)
     if (!g.graphs[i].live) id = (int)i;
@@ -478,6 +515,7 @@ int wdh_graph_end(int *graph_id) {
 int wdh_graph_launch(int graph_id) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_graph_launch");
+  if (g.lane) g.lane_dirty[g.lane] = true;  // work is about to be enqueued on a side lane
   if (graph_id < 0 || (size_t)graph_id >= g.graphs.size() || !g.graphs[graph_id].live ||
       !g.graphs[graph_id].exec)
     return fail(WDH_EINVAL, "wdh_graph_launch: unknown graph %d", graph_id);
@@ -497,6 +535,7 @@ int wdh_graph_destroy(int graph_id) {
 int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_write");
+  if (g.lane) g.lane_dirty[g.lane] = true;  // work is about to be enqueued on a side lane
   size_t have = 0;
   char *dst = (char *)wdh::resolve(h, &have);
   if (!dst) return WDH_EINVAL;
@@ -529,6 +568,7 @@ int wdh_write(wdh_buf h, size_t dst_offset, const void *src, size_t bytes) {
 int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_read");
+  if (g.lane) g.lane_dirty[g.lane] = true;  // work is about to be enqueued on a side lane
   size_t have = 0;
   const char *src = (const char *)wdh::resolve(h, &have);
   if (!src) return WDH_EINVAL;
@@ -568,7 +608,8 @@ int wdh_read(wdh_buf h, size_t src_offset, void *dst, size_t bytes) {
     copied += chunk_of[which];
     which = next;
   }
-  return wdh::contraction_check();  // (the stream has drained up to the data just read)
+  g.lane_dirty[g.lane] = false;     // (the stream has drained up to the data just read)
+  return wdh::contraction_check();
 }
 
 int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
@@ -583,9 +624,24 @@ int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
       bytes > shave - src_offset)
     return fail(WDH_EINVAL, "wdh_copy: range exceeds a buffer");
   wdh::conv_forget_weights(dst);
+  if (g.lane) g.lane_dirty[g.lane] = true;
   if (bytes)
     WDH_HIP_CHECK(hipMemcpyAsync(d + dst_offset, s + src_offset, bytes,
                                  hipMemcpyDeviceToDevice, g.stream));
+  return WDH_OK;
+}
+
+int wdh_set_lane(int lane) {
+  WDH_REQUIRE_INIT();
+  WDH_NOT_WHILE_CAPTURING("wdh_set_lane");
+  if (lane < 0 || lane >= WDH_LANES) return fail(WDH_EINVAL, "wdh_set_lane: lane %d (have 0..%d)", lane, WDH_LANES - 1);
+  if (!g.lanes[lane]) {
+    if (int rc = wdh::contraction_lane_init(lane)) return rc;
+    WDH_HIP_CHECK(hipStreamCreateWithFlags(&g.lanes[lane], hipStreamNonBlocking));
+  }
+  g.lane = lane;
+  g.stream = g.lanes[lane];
+  if (lane) g.lane_dirty[lane] = true;
   return WDH_OK;
 }
 
@@ -593,6 +649,7 @@ int wdh_sync(void) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_sync");
   WDH_HIP_CHECK(hipStreamSynchronize(g.stream));
+  g.lane_dirty[g.lane] = false;
   return wdh::contraction_check();
 }
 
@@ -614,6 +671,7 @@ int wdh_trim(size_t keep_bytes) {
 int wdh_event_record(int id) {
   WDH_REQUIRE_INIT();
   WDH_NOT_WHILE_CAPTURING("wdh_event_record");
+  if (g.lane) g.lane_dirty[g.lane] = true;  // work is about to be enqueued on a side lane
   if (id < 0 || id >= WDH_MAX_EVENTS)
     return fail(WDH_EINVAL, "wdh_event_record: id %d out of range", id);
   if (!g.events[id]) WDH_HIP_CHECK(hipEventCreate(&g.events[id]));

@@ -185,6 +185,10 @@ class HipContext:
     def sync(self):
         call("wdh_sync")
 
+    def set_lane(self, lane):
+        """wdh_set_lane: 0 = the default stream, 1 = the second one (recorded work and transfers only)."""
+        call("wdh_set_lane", lane)
+
     def mem_stats(self):
         a, b, c = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
         call("wdh_mem_stats", ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))

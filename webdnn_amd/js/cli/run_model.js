@@ -6,7 +6,7 @@
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
-//        [--graph | --no-graph] [--alt-inputs a2.bin[,b2.bin...]]
+//        [--graph | --no-graph] [--in-flight] [--alt-inputs a2.bin[,b2.bin...]]
 //
 // Inputs are raw little-endian files (float32, or int32 where the graph input says
 // so) in the order of the graph's non-initializer inputs; outputs are written the same
@@ -22,6 +22,9 @@
 // default ("auto") records the third run with inputs of one signature and replays it afterwards.
 // --alt-inputs names a second set of input files used by every other
 // run (odd run numbers), so that replays see changing data.
+// --in-flight keeps two runs in flight: run i+1 is submitted (runner.submit) before the outputs of run i are
+// collected (runner.collect).  msPerRun[i] is then the time from one submission to the next, the last
+// entry including the wait for the last run's outputs; the output file holds the last run's outputs.
 //
 // Methodology follows the reference's harness (example/benchmark/runner/bench.js:130-167):
 // warm-up runs, then timed runner.run() calls.
@@ -43,6 +46,7 @@ function parseArgs(argv) {
     else if (a === "--optimized") args.optimized = true;
     else if (a === "--graph") args.graph = true;
     else if (a === "--no-graph") args.graph = false;
+    else if (a === "--in-flight") args.inFlight = true;
     else if (a === "--alt-inputs") args.altInputs = next().split(",");
     else if (a === "--backend") args.backend = next();
     else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
@@ -119,7 +123,23 @@ async function main() {
   let outputs = null;
   let queueAhead = null;
   const deviceTimes = [];
-  for (let i = 0; i < args.runs; i++) {
+  if (args.inFlight) {
+    let pending = null;
+    let t0 = process.hrtime.bigint();
+    for (let i = 0; i < args.runs; i++) {
+      const ticket = await runner.submit(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs, runOptions({}));
+      if (pending) outputs = await runner.collect(pending);
+      pending = ticket;
+      if (i + 1 === args.runs) {
+        outputs = await runner.collect(pending);
+        pending = null;
+      }
+      const t1 = process.hrtime.bigint();
+      times.push(Number(t1 - t0) / 1e6);
+      t0 = t1;
+    }
+  }
+  for (let i = 0; i < (args.inFlight ? 0 : args.runs); i++) {
     // --queue-ahead MS (with --measure): put about MS milliseconds of streaming kernels on the
     // device queue first, so that the measured run's launches are all queued before the device
     // reaches them.  Its kernels then run back to back and the per-node events time the device
@@ -162,7 +182,8 @@ async function main() {
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
     node: process.version,
-    graph: args.graph !== false ? { captured: !!runner.graphState, unsupported: runner.graphUnsupported } : undefined,
+    graph: args.graph !== false ? { captured: !!runner.graphState, lanes: (runner.graphState ? 1 : 0) + (runner.sideGraphState ? 1 : 0),
+      unsupported: runner.graphUnsupported } : undefined,
   };
   runner.disposeGraph();
   if (queueAhead) {

@@ -53,6 +53,12 @@ class RunnerImpl {
     this.lastPerformance = null;
     // captured run: {id, inputs, ownedInputs, outputs, signature, stats}; see runWithGraph
     this.graphState = null;
+    // two runs in flight (submit / collect): the captured run of the second lane, built like graphState
+    // from the same node loop recorded on the library's lane 1; which lane the next submit takes; and
+    // the submitted runs not collected yet, by lane
+    this.sideGraphState = null;
+    this.submitLane = 0;
+    this.inFlight = [null, null];
     this.graphWarm = false;
     this.graphUnsupported = null; // reason, once a capture has failed for this model
     this.graphRetries = 0; // captures given up for a reason an eager run cures
@@ -151,6 +157,7 @@ class RunnerImpl {
     const opts = options || {};
     if (!this.model || !this.loaded) throw new Error("not initialized");
     if (!inputs) throw new Error("inputs are required");
+    if (this.inFlight[0] || this.inFlight[1]) throw new Error("run: collect the submitted runs first");
     const hipContext = this.backendContexts.hip;
     let mode = opts.graph !== undefined ? opts.graph : this.options.graph;
     if (mode === undefined || mode === null) mode = "auto";
@@ -172,15 +179,19 @@ class RunnerImpl {
     return this.runEager(inputs, opts);
   }
 
-  // Frees the captured run, if any (its output and input buffers included).
+  // Frees the captured runs, if any (their output and input buffers included).
   disposeGraph() {
-    const state = this.graphState;
-    if (!state) return;
-    this.graphState = null;
     const hip = this.backendContexts.hip;
-    for (const t of state.outputs) if (t.backend === "hip") t.dispose();
-    for (const t of state.ownedInputs) t.dispose();
-    hip.native.graphDestroy(state.id);
+    for (const key of ["sideGraphState", "graphState"]) {
+      const state = this[key];
+      if (!state) continue;
+      this[key] = null;
+      for (const t of state.outputs) if (t.backend === "hip") t.dispose();
+      for (const t of state.ownedInputs) t.dispose();
+      hip.native.graphDestroy(state.id);
+    }
+    this.inFlight = [null, null];
+    this.submitLane = 0;
   }
 
   // First call: an ordinary run (it uploads the weights, fills the buffer pool and builds
@@ -207,78 +218,174 @@ class RunnerImpl {
         this.graphWarm = true;
         return this.runEager(inputs, opts);
       }
-      // The graph reads its inputs from buffers the runner owns: a caller's device tensor
-      // is copied in like a host tensor is uploaded, so the caller may overwrite or dispose
-      // it afterwards and later replays never write into caller memory.
-      const graphInputs = [];
-      try {
-        for (const t of inputs) {
-          if (t.backend === "hip") {
-            const own = hip.emptyTensor(t.dims, t.dataType);
-            graphInputs.push(own);
-            hip.native.copy(own.handle, 0, t.handle, 0, own.length * 4);
-          } else {
-            graphInputs.push(await hip.moveTensor(t, {}));
-          }
-        }
-      } catch (error) {
-        for (const t of graphInputs) t.dispose();
-        throw error;
-      }
-      let outputs = null,
-        failure = null;
-      hip.native.graphBegin();
-      try {
-        outputs = await this.runEager(graphInputs, { capture: true });
-      } catch (error) {
-        failure = error;
-      }
-      let id = -1;
-      try {
-        id = hip.native.graphEnd();
-      } catch (error) {
-        failure = failure || error;
-      }
-      if (failure) {
-        if (id >= 0) hip.native.graphDestroy(id);
-        for (const t of outputs || []) if (t.backend === "hip") t.dispose();
-        for (const t of graphInputs) t.dispose();
-        // A geometry met for the first time while recording (its tables need a blocking
-        // copy) is cured by the eager run below; anything else will fail the same way again.
-        const transient = /run it once before capturing/.test(failure.message) && this.graphRetries < 3;
-        if (transient) {
-          this.graphRetries++;
-        } else {
-          this.graphUnsupported = failure.message;
-        }
-        logger.warn(`run could not be captured into a graph (${failure.message}); running eagerly`);
-        return this.runEager(inputs, opts);
-      }
-      this.graphRetries = 0;
-      this.graphState = { id, inputs: graphInputs, ownedInputs: graphInputs, outputs, signature, stats: this.lastRunStats };
+      const state = await this.captureRun(inputs);
+      if (!state) return this.runEager(inputs, opts);
+      this.graphState = state;
     } else {
-      const state = this.graphState;
-      for (let i = 0; i < inputs.length; i++) {
-        const src = inputs[i],
-          dst = state.inputs[i];
-        if (src.backend === "hip") hip.native.copy(dst.handle, 0, src.handle, 0, dst.length * 4);
-        else await dst.setData(await src.getData());
-      }
+      await this.refillGraphInputs(this.graphState, inputs);
     }
     const state = this.graphState;
     if (opts.measurePerformance) hip.native.eventRecord(0);
     hip.native.graphLaunch(state.id);
     if (opts.measurePerformance) hip.native.eventRecord(1);
-    const results = [];
-    for (const t of state.outputs) {
-      // device -> host, the run's only synchronisation; a cpu output (a constant) is copied
-      results.push(await cpu.moveTensor(t, {}));
-    }
+    const results = await this.readGraphOutputs(state);
     if (opts.measurePerformance) {
       this.lastPerformance = [{ opType: "(captured graph)", name: "graph", backend: "hip", deviceElapsed: hip.native.eventElapsedMs(0, 1) }];
     }
     this.lastRunStats = Object.assign({}, state.stats, { graphReplay: true });
     return results;
+  }
+
+  // Records one run of the node loop on the library's current lane.  Returns the captured run
+  // {id, inputs, ownedInputs, outputs, signature, stats}, or null when the run cannot be recorded
+  // (the reason is logged; graphUnsupported is set unless the cause is transient).
+  async captureRun(inputs) {
+    const hip = this.backendContexts.hip;
+    // The graph reads its inputs from buffers the runner owns: a caller's device tensor
+    // is copied in like a host tensor is uploaded, so the caller may overwrite or dispose
+    // it afterwards and later replays never write into caller memory.
+    const graphInputs = [];
+    try {
+      for (const t of inputs) {
+        if (t.backend === "hip") {
+          const own = hip.emptyTensor(t.dims, t.dataType);
+          graphInputs.push(own);
+          hip.native.copy(own.handle, 0, t.handle, 0, own.length * 4);
+        } else {
+          graphInputs.push(await hip.moveTensor(t, {}));
+        }
+      }
+    } catch (error) {
+      for (const t of graphInputs) t.dispose();
+      throw error;
+    }
+    let outputs = null,
+      failure = null;
+    hip.native.graphBegin();
+    try {
+      outputs = await this.runEager(graphInputs, { capture: true });
+    } catch (error) {
+      failure = error;
+    }
+    let id = -1;
+    try {
+      id = hip.native.graphEnd();
+    } catch (error) {
+      failure = failure || error;
+    }
+    if (failure) {
+      if (id >= 0) hip.native.graphDestroy(id);
+      for (const t of outputs || []) if (t.backend === "hip") t.dispose();
+      for (const t of graphInputs) t.dispose();
+      // A geometry met for the first time while recording (its tables need a blocking
+      // copy) is cured by an eager run; anything else will fail the same way again.
+      const transient = /run it once before capturing/.test(failure.message) && this.graphRetries < 3;
+      if (transient) {
+        this.graphRetries++;
+      } else {
+        this.graphUnsupported = failure.message;
+      }
+      logger.warn(`run could not be captured into a graph (${failure.message}); running eagerly`);
+      return null;
+    }
+    this.graphRetries = 0;
+    return { id, inputs: graphInputs, ownedInputs: graphInputs, outputs, signature: inputSignature(inputs), stats: this.lastRunStats };
+  }
+
+  // The caller's inputs go into the captured run's own input buffers (upload or device copy).
+  async refillGraphInputs(state, inputs) {
+    const hip = this.backendContexts.hip;
+    for (let i = 0; i < inputs.length; i++) {
+      const src = inputs[i],
+        dst = state.inputs[i];
+      if (src.backend === "hip") hip.native.copy(dst.handle, 0, src.handle, 0, dst.length * 4);
+      else await dst.setData(await src.getData());
+    }
+  }
+
+  // device -> host, the run's only synchronisation; a cpu output (a constant) is copied
+  async readGraphOutputs(state) {
+    const cpu = this.backendContexts.cpu;
+    const results = [];
+    for (const t of state.outputs) results.push(await cpu.moveTensor(t, {}));
+    return results;
+  }
+
+  // Two runs in flight.  submit() enqueues a run -- inputs uploaded, the captured graph launched -- and
+  // returns a ticket without waiting for the device; collect(ticket) downloads that run's outputs.  A
+  // caller that submits batch i+1 before it collects batch i keeps the device busy while batch i's
+  // results travel and while batch i+1's kernels start: the two runs sit on the library's two lanes
+  // (streams) and overlap where the device has room.  Each lane has its own captured run (own input,
+  // output and workspace buffers).  Until the model has been captured (the first calls, or a model that
+  // cannot be captured, or graph mode off) submit() simply runs and the ticket carries the outputs.
+  // At most one run per lane may be outstanding: collect in the order of submission.
+  async submit(inputs, options) {
+    const opts = options || {};
+    if (!this.model || !this.loaded) throw new Error("not initialized");
+    const hip = this.backendContexts.hip;
+    let mode = opts.graph !== undefined ? opts.graph : this.options.graph;
+    if (mode === undefined || mode === null) mode = "auto";
+    const lanes = hip && hip.initialized && hip.native.setLane && hip.native.graphBegin && !this.graphUnsupported && mode !== false;
+    const signature = lanes ? inputSignature(inputs) : null;
+    if (!lanes || opts.measurePerformance || !this.graphState || this.graphState.signature !== signature) {
+      // not captured yet (or never will be): an ordinary run, which also does the warming up and capturing
+      await this.drainInFlight();
+      return { done: await this.run(inputs, opts) };
+    }
+    const lane = this.submitLane;
+    if (this.inFlight[lane]) throw new Error("submit: two runs are in flight already; collect the older one first");
+    if (this.inputsWithoutInitializer.length !== inputs.length) throw new Error("length of inputs mismatch");
+    let state = lane === 0 ? this.graphState : this.sideGraphState;
+    if (state && state.signature !== signature) state = null; // (cannot happen for lane 0: checked above)
+    hip.native.setLane(lane);
+    try {
+      if (!state) {
+        if (this.sideGraphState) {
+          const old = this.sideGraphState;
+          this.sideGraphState = null;
+          for (const t of old.outputs) if (t.backend === "hip") t.dispose();
+          for (const t of old.ownedInputs) t.dispose();
+          hip.native.graphDestroy(old.id);
+        }
+        state = await this.captureRun(inputs);
+        if (!state) {
+          hip.native.setLane(0);
+          await this.drainInFlight();
+          return { done: await this.run(inputs, opts) };
+        }
+        this.sideGraphState = state;
+      } else {
+        await this.refillGraphInputs(state, inputs);
+      }
+      hip.native.graphLaunch(state.id);
+    } finally {
+      hip.native.setLane(0);
+    }
+    const ticket = { lane, state };
+    this.inFlight[lane] = ticket;
+    this.submitLane = lane ^ 1;
+    return ticket;
+  }
+
+  async collect(ticket) {
+    if (!ticket) throw new Error("collect: no ticket");
+    if (ticket.done) return ticket.done;
+    if (this.inFlight[ticket.lane] !== ticket) throw new Error("collect: this run has been collected already");
+    const hip = this.backendContexts.hip;
+    hip.native.setLane(ticket.lane);
+    try {
+      const results = await this.readGraphOutputs(ticket.state);
+      this.lastRunStats = Object.assign({}, ticket.state.stats, { graphReplay: true, lane: ticket.lane });
+      return results;
+    } finally {
+      this.inFlight[ticket.lane] = null;
+      hip.native.setLane(0);
+    }
+  }
+
+  // Waits for the submitted runs (their outputs are dropped).
+  async drainInFlight() {
+    for (const ticket of this.inFlight) if (ticket) await this.collect(ticket);
   }
 
   // opts.capture (internal): the stream is recording; keep the outputs where they are and

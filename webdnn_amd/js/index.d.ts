@@ -26,6 +26,11 @@ export interface RunStats {
   graphReplay?: boolean;
 }
 
+/** What submit() returns and collect() takes; opaque to callers. */
+export interface RunTicket {
+  readonly lane?: number;
+}
+
 export interface Runner {
   readonly backendName: Backend;
   readonly backendContexts: { cpu: unknown; hip?: WebDNNHipContext };
@@ -36,6 +41,15 @@ export interface Runner {
   getOutputNames(): string[];
   /** outputs come back as CPU tensors, as in the reference */
   run(inputs?: Tensor[], options?: RunOption): Promise<Tensor[]>;
+  /**
+   * Two runs in flight (no counterpart in the reference).  submit() enqueues a run on one of the library's
+   * two lanes and returns without waiting for the device; collect() downloads that run's outputs.  Submit
+   * batch i+1 before collecting batch i and the device works on one while the other's data travels.  At
+   * most two runs may be outstanding; collect them in the order of submission, and before calling run().
+   * Until the model is captured (or if it cannot be) submit() simply runs and the ticket holds the outputs.
+   */
+  submit(inputs: Tensor[], options?: RunOption): Promise<RunTicket>;
+  collect(ticket: RunTicket): Promise<Tensor[]>;
   disposeGraph(): void;
 }
 

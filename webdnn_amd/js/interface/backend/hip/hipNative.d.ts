@@ -32,6 +32,8 @@ export interface HipNative {
   read(h: Handle, srcByteOffset: number, data: ArrayBufferView): void;
   copy(dst: Handle, dstByteOffset: number, src: Handle, srcByteOffset: number, bytes: number): void;
   sync(): void;
+  /** wdh_set_lane: 0 = the stream everything runs on by default, 1 = the second stream (two runs in flight). */
+  setLane(lane: number): void;
   memStats(): HipMemStats;
   trim(keepBytes: number): void;
   eventRecord(id: number): void;

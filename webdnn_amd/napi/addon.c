@@ -218,6 +218,13 @@ FN(js_sync) {
   return make_undefined(env);
 }
 
+FN(js_set_lane) {
+  ARGS("wdh_set_lane", 1);
+  I64(0, lane);
+  CHECK(wdh_set_lane((int)lane));
+  return make_undefined(env);
+}
+
 FN(js_mem_stats) {
   ARGS("wdh_mem_stats", 0);
   uint64_t a = 0, b = 0, c = 0;
@@ -494,6 +501,7 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
       {"stridedCopy", js_strided_copy}, {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end},
       {"graphLaunch", js_graph_launch}, {"graphDestroy", js_graph_destroy},
+      {"setLane", js_set_lane},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {
     napi_value fn;
