@@ -186,10 +186,10 @@ int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
 /* Waits for the work of the current lane (see wdh_set_lane). */
 int wdh_sync(void);
 
-/* Lanes: two runs in flight.  No counterpart in the reference (its backends run one graph at a time);
+/* Lanes: several runs in flight.  No counterpart in the reference (its backends run one graph at a time);
  * for callers that keep a second batch on its way while the first computes.  A lane is a HIP stream of
- * default priority; lane 0 is the stream everything runs on unless told otherwise.  wdh_set_lane(1)
- * makes lane 1 the current one: wdh_write, wdh_read, wdh_copy, wdh_sync, wdh_event_record,
+ * default priority; lane 0 is the stream everything runs on unless told otherwise, lanes 1 .. WDH_LANES - 1
+ * are side lanes, created when first named.  wdh_set_lane(1) makes lane 1 the current one: wdh_write, wdh_read, wdh_copy, wdh_sync, wdh_event_record,
  * wdh_graph_begin / _end / _launch then work on it, concurrently with what lane 0 still has queued.
  * Side lanes are for captured runs and their transfers: an operator call (wdh_gemm, wdh_conv2d, ...) on
  * a side lane is legal only while a graph is being recorded there and fails with WDH_ESTATE otherwise.
@@ -199,7 +199,7 @@ int wdh_sync(void);
  * first used), so a run recorded on a side lane computes bit for bit what it computes on lane 0;
  * wdh_gemm_static is refused there (its workspace is lane 0's).  What the caller guards: a buffer written on one lane and read on another needs a
  * wdh_sync (or wdh_read) on the first in between.  Not possible while capturing. */
-#define WDH_LANES 2
+#define WDH_LANES 4
 int wdh_set_lane(int lane);
 
 /* Pool accounting: bytes handed out, bytes cached in the pool, high-water

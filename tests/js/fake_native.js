@@ -96,7 +96,7 @@ const native = {
   },
   sync() {},
   setLane(lane) {
-    if (lane !== 0 && lane !== 1) throw new Error("wdh_set_lane failed (-2): lane " + lane);
+    if (![0, 1, 2, 3].includes(lane)) throw new Error("wdh_set_lane failed (-2): lane " + lane);
     count("setLane");
     currentLane = lane;
   },

@@ -41,7 +41,9 @@ def test_a_side_lane_takes_recorded_work_and_transfers_only(ctx):
     B = ctx.move_tensor(_rng(2).standard_normal((128, 64)).astype(np.float32))
     want = H.matmul(ctx, A, B).get_data()
     with pytest.raises(capi.HipError):
-        ctx.set_lane(2)
+        ctx.set_lane(4)                                                    # lanes 0..3
+    with pytest.raises(capi.HipError):
+        ctx.set_lane(-1)
     ctx.set_lane(1)
     try:
         with pytest.raises(capi.HipError) as e:

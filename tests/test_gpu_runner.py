@@ -228,6 +228,20 @@ def test_two_runs_in_flight_equal_eager_runs(tmp_path):
                 assert_bit_exact(got[0], want[0], "run %d of a session with two runs in flight %s" % (runs, flags))
 
 
+def test_three_runs_in_flight_equal_eager_runs(tmp_path):
+    """The same with three lanes (load option inFlight = 3): from the sixth run on all three hold a recording."""
+    data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    ea, _ = node_runner.run_model(str(tmp_path), [Xa], "hip", strict=True, extra=["--no-graph"])
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True, extra=["--no-graph"])
+    for runs, want in ((5, ea), (6, eb), (7, ea), (10, eb), (13, ea)):
+        got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], runs, flags=("--in-flight", "3"))
+        assert rep["graph"]["lanes"] == min(3, runs - 3) and rep["graph"]["unsupported"] is None, (runs, rep["graph"])
+        assert_bit_exact(got[0], want[0], "run %d of a session with three runs in flight" % runs)
+
+
 def test_runs_without_an_option_are_replayed_from_the_third_on(tmp_path):
     """runner.run([CPUTensor]) with no option (graph "auto"): two eager runs, the third recorded, the rest
     replayed; each compared run equals the eager run of the input it was given, bit for bit."""

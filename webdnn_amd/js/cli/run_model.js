@@ -6,7 +6,7 @@
 //        --inputs a.bin[,b.bin...] --output out.bin
 //        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
-//        [--graph | --no-graph] [--in-flight] [--alt-inputs a2.bin[,b2.bin...]]
+//        [--graph | --no-graph] [--in-flight [N]] [--alt-inputs a2.bin[,b2.bin...]]
 //
 // Inputs are raw little-endian files (float32, or int32 where the graph input says
 // so) in the order of the graph's non-initializer inputs; outputs are written the same
@@ -22,8 +22,8 @@
 // default ("auto") records the third run with inputs of one signature and replays it afterwards.
 // --alt-inputs names a second set of input files used by every other
 // run (odd run numbers), so that replays see changing data.
-// --in-flight keeps two runs in flight: run i+1 is submitted (runner.submit) before the outputs of run i are
-// collected (runner.collect).  msPerRun[i] is then the time from one submission to the next, the last
+// --in-flight [N] keeps N (2 unless given, at most 4) runs in flight: run i+1 is submitted (runner.submit) before
+// the outputs of run i+2-N are collected (runner.collect).  msPerRun[i] is then the time from one submission to the next, the last
 // entry including the wait for the last run's outputs; the output file holds the last run's outputs.
 //
 // Methodology follows the reference's harness (example/benchmark/runner/bench.js:130-167):
@@ -46,7 +46,10 @@ function parseArgs(argv) {
     else if (a === "--optimized") args.optimized = true;
     else if (a === "--graph") args.graph = true;
     else if (a === "--no-graph") args.graph = false;
-    else if (a === "--in-flight") args.inFlight = true;
+    else if (a === "--in-flight") {
+      // optional count: --in-flight 3
+      args.inFlight = i + 1 < argv.length && /^[0-9]+$/.test(argv[i + 1]) ? parseInt(argv[++i], 10) : 2;
+    }
     else if (a === "--alt-inputs") args.altInputs = next().split(",");
     else if (a === "--backend") args.backend = next();
     else if (a === "--inputs") args.inputs = next().split(",").filter((s) => s.length);
@@ -73,6 +76,7 @@ async function main() {
   if (args.cpuEntries) registerOperators(require(path.resolve(args.cpuEntries)).getOpEntries());
   const hipOption = { strict: !!args.strict, fuse: !args.noFuse };
   if (args.tile != null) hipOption.contractionTile = args.tile;
+  if (args.inFlight) hipOption.inFlight = args.inFlight;
   // --native: another implementation of the addon's interface (host tests without a GPU)
   if (args.native) hipOption.native = require(path.resolve(args.native));
   const runner = await WebDNN.load(args.model, {
@@ -124,16 +128,11 @@ async function main() {
   let queueAhead = null;
   const deviceTimes = [];
   if (args.inFlight) {
-    let pending = null;
+    const pending = []; // tickets in order of submission, at most args.inFlight - 1 while the next is submitted
     let t0 = process.hrtime.bigint();
     for (let i = 0; i < args.runs; i++) {
-      const ticket = await runner.submit(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs, runOptions({}));
-      if (pending) outputs = await runner.collect(pending);
-      pending = ticket;
-      if (i + 1 === args.runs) {
-        outputs = await runner.collect(pending);
-        pending = null;
-      }
+      pending.push(await runner.submit(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs, runOptions({})));
+      while (pending.length >= args.inFlight || (i + 1 === args.runs && pending.length)) outputs = await runner.collect(pending.shift());
       const t1 = process.hrtime.bigint();
       times.push(Number(t1 - t0) / 1e6);
       t0 = t1;
@@ -182,7 +181,7 @@ async function main() {
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
     node: process.version,
-    graph: args.graph !== false ? { captured: !!runner.graphState, lanes: (runner.graphState ? 1 : 0) + (runner.sideGraphState ? 1 : 0),
+    graph: args.graph !== false ? { captured: !!runner.graphState, lanes: (runner.graphState ? 1 : 0) + runner.sideGraphStates.filter((st) => st).length,
       unsupported: runner.graphUnsupported } : undefined,
   };
   runner.disposeGraph();

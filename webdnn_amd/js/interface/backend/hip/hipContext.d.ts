@@ -15,6 +15,8 @@ export interface WebDNNHipContextOption {
   /** captured runs: true = record the second run; "auto" (default) = record the third run with inputs
    *  of one signature; false = always the node loop.  runner.run(inputs, {graph}) overrides it per call. */
   graph?: boolean | "auto";
+  /** how many runs runner.submit keeps in flight (lanes it alternates over): 2 (default) to 4 */
+  inFlight?: number;
   /** tuning hooks handed to wdh_set_option */
   contractionTile?: number;
   splitK?: number;
