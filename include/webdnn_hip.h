@@ -197,7 +197,8 @@ int wdh_sync(void);
  * lane first; an allocation or a capture on a side lane waits for lane 0; launches that run as streams
  * of K slabs use a workspace of the lane's own (WDH_STATIC_SCRATCH_BYTES from the driver when the lane is
  * first used), so a run recorded on a side lane computes bit for bit what it computes on lane 0;
- * wdh_gemm_static is refused there (its workspace is lane 0's).  What the caller guards: a buffer written on one lane and read on another needs a
+ * wdh_gemm_static is refused there (its workspace is lane 0's); a wdh_copy on a side lane first waits
+ * for uploads (wdh_write) still on their way on any lane.  What the caller guards: a buffer written on one lane and read on another needs a
  * wdh_sync (or wdh_read) on the first in between.  Not possible while capturing. */
 #define WDH_LANES 4
 int wdh_set_lane(int lane);

@@ -624,7 +624,13 @@ int wdh_copy(wdh_buf dst, size_t dst_offset, wdh_buf src, size_t src_offset,
       bytes > shave - src_offset)
     return fail(WDH_EINVAL, "wdh_copy: range exceeds a buffer");
   wdh::conv_forget_weights(dst);
-  if (g.lane) g.lane_dirty[g.lane] = true;
+  if (g.lane) {
+    g.lane_dirty[g.lane] = true;
+    // the source may be an upload still on its way on another lane (a tensor moved to the device just
+    // before it is submitted): uploads are the one kind of cross-lane producer the library can see
+    if (!g.capturing)
+      if (int rc = wait_for_uploads()) return rc;
+  }
   if (bytes)
     WDH_HIP_CHECK(hipMemcpyAsync(d + dst_offset, s + src_offset, bytes,
                                  hipMemcpyDeviceToDevice, g.stream));

@@ -320,6 +320,9 @@ class RunnerImpl {
   // (streams) and overlap where the device has room.  Each lane has its own captured run (own input,
   // output and workspace buffers).  Until the model has been captured (the first calls, or a model that
   // cannot be captured, or graph mode off) submit() simply runs and the ticket carries the outputs.
+  // An input that already lives on the device must be complete when it is submitted (uploaded -- the
+  // library waits for uploads by itself -- or produced by work that has been waited for): the lanes do
+  // not wait for each other.
   // At most one run per lane may be outstanding: collect in the order of submission.  A second batch in
   // flight fills most of what one leaves idle (ResNet-50 b32: +12 %); a third and a fourth add 3 % and 1 %.
   async submit(inputs, options) {

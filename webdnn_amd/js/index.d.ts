@@ -42,11 +42,12 @@ export interface Runner {
   /** outputs come back as CPU tensors, as in the reference */
   run(inputs?: Tensor[], options?: RunOption): Promise<Tensor[]>;
   /**
-   * Two runs in flight (no counterpart in the reference).  submit() enqueues a run on one of the library's
+   * Several runs in flight -- two unless backendOptions.hip.inFlight says 3 or 4 (no counterpart in the reference).  submit() enqueues a run on one of the library's
    * two lanes and returns without waiting for the device; collect() downloads that run's outputs.  Submit
    * batch i+1 before collecting batch i and the device works on one while the other's data travels.  At
-   * most two runs may be outstanding; collect them in the order of submission, and before calling run().
+   * most that many runs may be outstanding; collect them in the order of submission, and before calling run().
    * Until the model is captured (or if it cannot be) submit() simply runs and the ticket holds the outputs.
+   * Inputs that already live on the device must be complete (uploaded, or produced by work that was waited for).
    */
   submit(inputs: Tensor[], options?: RunOption): Promise<RunTicket>;
   collect(ticket: RunTicket): Promise<Tensor[]>;
