@@ -203,6 +203,20 @@ int wdh_sync(void);
 #define WDH_LANES 4
 int wdh_set_lane(int lane);
 
+/* Side branches of a recorded run.  No counterpart in the reference.  Between wdh_graph_begin and
+ * wdh_graph_end, the calls made between wdh_branch_begin and wdh_branch_end are recorded as a branch that
+ * depends only on what was recorded before wdh_branch_begin; the calls after wdh_branch_end do not depend
+ * on the branch until wdh_branch_join, so a replay may run the branch next to them (a projection shortcut
+ * next to the convolutions it bypasses).  One branch at a time.  The caller promises that nothing recorded
+ * between _end and _join reads what the branch writes or writes what it reads.  The library keeps the
+ * buffers apart: a block freed while a branch is open is handed out again only after the join, and no
+ * launch takes the stream-of-K-slabs form while one is open (that form's workspace is one per lane).
+ * Outside a recording the three calls do nothing: the work simply runs in the order of the calls, with the
+ * same results bit for bit.  wdh_graph_end joins a branch that was left open. */
+int wdh_branch_begin(void);
+int wdh_branch_end(void);
+int wdh_branch_join(void);
+
 /* Pool accounting: bytes handed out, bytes cached in the pool, high-water
  * mark of hipMalloc'ed bytes (cf. perfTotalMemory,
  * backend/wasm/wasmTensorImpl.ts:29-35).  Any pointer may be NULL. */

@@ -95,6 +95,15 @@ const native = {
     buf(dst).set(buf(src).subarray(soff, soff + bytes), doff);
   },
   sync() {},
+  branchBegin() {
+    count("branchBegin");
+  },
+  branchEnd() {
+    count("branchEnd");
+  },
+  branchJoin() {
+    count("branchJoin");
+  },
   setLane(lane) {
     if (![0, 1, 2, 3].includes(lane)) throw new Error("wdh_set_lane failed (-2): lane " + lane);
     count("setLane");

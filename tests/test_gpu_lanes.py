@@ -151,3 +151,84 @@ def test_runs_recorded_on_both_lanes_agree_and_overlap(ctx):
     ctx.graph_destroy(graphs[0][0])
     for t in filler + xs + [t for pair in weights for t in pair]:
         t.dispose()
+
+
+def test_side_branch_of_a_recorded_run(ctx):
+    """wdh_branch_begin / _end / _join: a projection shortcut recorded as a side branch of a residual block.
+    Outside a recording the calls do nothing; a replay of the recording with the branch equals the eager result
+    bit for bit, ten replays with fresh inputs; a branch left open is joined by wdh_graph_end; opening two at
+    once or joining nothing abandons the recording."""
+    r = _rng(11)
+    def wb(co, ci, k):
+        return (ctx.move_tensor((r.standard_normal((co, ci, k, k)) * np.sqrt(2.0 / (ci * k * k))).astype(np.float32)),
+                ctx.move_tensor(r.standard_normal(co).astype(np.float32)))
+    (w1, b1), (w2, b2), (w3, b3), (wd, bd) = wb(128, 256, 1), wb(128, 128, 3), wb(512, 128, 1), wb(512, 256, 1)
+    X = r.uniform(0, 1, (8, 256, 28, 28)).astype(np.float32)
+    x = ctx.move_tensor(X)
+
+    def block(branch, join=True):
+        if branch:
+            capi.call("wdh_branch_begin")
+        sc = H.conv(ctx, x, wd, bd, strides=[2, 2], constant_weights=True)
+        if branch:
+            capi.call("wdh_branch_end")
+        t1 = H.conv(ctx, x, w1, b1, strides=[2, 2], epilogue="relu", constant_weights=True)
+        t2 = H.conv(ctx, t1, w2, b2, pads=[1, 1, 1, 1], epilogue="relu", constant_weights=True)
+        t1.dispose()
+        if branch and join:
+            capi.call("wdh_branch_join")
+        y = H.conv(ctx, t2, w3, b3, epilogue="relu", residual=sc, constant_weights=True)
+        t2.dispose()
+        sc.dispose()
+        return y
+
+    def eager():
+        y = block(False)
+        out = y.get_data()
+        y.dispose()
+        return out
+
+    want = eager()
+    y = block(True)                                        # executing: the three calls are no-ops
+    assert_bit_exact(y.get_data(), want, "eager with the branch calls")
+    y.dispose()
+    sc_ref = ref.conv(X[:1], wd.get_data(), bd.get_data(), strides=[2, 2])
+    main = ref.unary("Relu", ref.conv(ref.unary("Relu", ref.conv(X[:1], w1.get_data(), b1.get_data(), strides=[2, 2])),
+                                      w2.get_data(), b2.get_data(), pads=[1, 1, 1, 1]))
+    assert_close_max(want[:1], ref.unary("Relu", ref.binary("Add", ref.conv(main, w3.get_data(), b3.get_data()), sc_ref)),
+                     1e-4, "the block against the oracle")
+    ctx.sync()
+    for join in (True, False):                             # False: wdh_graph_end joins the branch itself
+        ctx.graph_begin()
+        try:
+            out = block(True, join=join)
+        finally:
+            gid = ctx.graph_end()
+        for rep in range(10):
+            if rep:
+                Xn = r.uniform(0, 1, X.shape).astype(np.float32)
+                capi.call("wdh_write", x.handle, 0, Xn.ctypes.data, Xn.nbytes)
+            ctx.graph_launch(gid)
+            got = out.get_data()
+            if not join:
+                continue   # (its last conv is not ordered behind the shortcut: only the recording's end is)
+            assert_bit_exact(got, eager(), "replay %d with a side branch" % rep)
+        out.dispose()
+        ctx.graph_destroy(gid)
+        capi.call("wdh_write", x.handle, 0, X.ctypes.data, X.nbytes)
+    for misuse in ("twice", "join"):
+        ctx.graph_begin()
+        with pytest.raises(capi.HipError):
+            if misuse == "twice":
+                capi.call("wdh_branch_begin")
+                capi.call("wdh_branch_begin")
+            else:
+                capi.call("wdh_branch_join")
+        with pytest.raises(capi.HipError) as e:
+            ctx.graph_end()
+        assert "abandoned" in str(e.value)
+    y = block(True)
+    assert_bit_exact(y.get_data(), want, "the library works on after an abandoned recording")
+    y.dispose()
+    for t in (x, w1, b1, w2, b2, w3, b3, wd, bd):
+        t.dispose()

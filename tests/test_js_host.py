@@ -385,6 +385,26 @@ def _graph_vs_eager(tmp_path, data, feeds_a, feeds_b, fake_native, flags=("--gra
     return g3, g4, eager_a, eager_b, rep4
 
 
+def test_projection_shortcuts_become_side_branches(tmp_path):
+    """modelTransform.hoistSideBranches: in a ResNet the projection shortcut of each stage's first block is moved
+    up to the block's start and bracketed with branchBegin / branchEnd, its consumer preceded by branchJoin;
+    results equal the cpu path bit for bit in the node loop, in a recorded run, and with the pass switched off."""
+    data, _ = modelgen.resnet50_model(batch=2, image=32, width=8, blocks=(1, 2, 1, 1), classes=10)
+    X = np.random.default_rng(2).standard_normal((2, 3, 32, 32)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    want, _ = node_runner.run_model(str(tmp_path), [X], "cpu", oracle_cpu=True)
+    kw = dict(strict=True, fake_native=True)
+    eager, rep = node_runner.run_model(str(tmp_path), [X], "hip", extra=["--no-graph"], **kw)
+    assert rep["nativeCalls"]["branchBegin"] == 4 and rep["nativeCalls"]["branchEnd"] == 4 and rep["nativeCalls"]["branchJoin"] == 4
+    assert_bit_exact(eager[0], want[0], "node loop with the shortcuts moved up")
+    replay, rep = node_runner.run_model(str(tmp_path), [X], "hip", runs=4, extra=["--graph"], **kw)
+    assert rep["graph"]["captured"] and rep["nativeCalls"]["branchBegin"] == 2 * 4    # one eager run, one recording
+    assert_bit_exact(replay[0], want[0], "replay with side branches")
+    plain, rep = node_runner.run_model(str(tmp_path), [X], "hip", runs=3, extra=["--graph", "--no-side-branches"], **kw)
+    assert "branchBegin" not in rep["nativeCalls"]
+    assert_bit_exact(plain[0], want[0], "pass switched off")
+
+
 def test_two_runs_in_flight_on_the_host_path(tmp_path):
     """runner.submit / runner.collect against the stand-in addon: whatever the session length, the last run's
     outputs equal the eager run of its input; the second lane is recorded once, every pipelined run brackets its

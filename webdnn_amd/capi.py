@@ -35,6 +35,9 @@ SIGNATURES = {
     "wdh_copy": (_c.c_int, [c_buf, _c.c_size_t, c_buf, _c.c_size_t, _c.c_size_t]),
     "wdh_sync": (_c.c_int, []),
     "wdh_set_lane": (_c.c_int, [_c.c_int]),
+    "wdh_branch_begin": (_c.c_int, []),
+    "wdh_branch_end": (_c.c_int, []),
+    "wdh_branch_join": (_c.c_int, []),
     "wdh_mem_stats": (_c.c_int, [_u64p, _u64p, _u64p]),
     "wdh_trim": (_c.c_int, [_c.c_size_t]),
     "wdh_graph_begin": (_c.c_int, []),

@@ -20,6 +20,7 @@ hipStream_t stream();
 int compute_units();
 int device();           // the device wdh_init selected
 int lane();             // the current lane (wdh_set_lane)
+bool branch_open();     // a side branch of the run being recorded is open (wdh_branch_begin .. wdh_branch_join)
 // The pool asks the driver for at most `bytes` in total (0 = no limit); blocks it already holds stay.
 void set_memory_limit(uint64_t bytes);
 // Looks up the device address of the static workspace of wdh_gemm_static for `device`,

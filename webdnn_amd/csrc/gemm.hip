@@ -239,6 +239,9 @@ WorkPlan plan_work(long long tiles, int k, int bm, int bn, bool gather, int kgra
 // `w` is what the tile-per-workgroup plan would do.
 int stream_width(long long tiles, int slabs, int kgran, const WorkPlan &w, int tile_floats, int max_wgs_per_cu) {
   if (!g_stream || g_forced_split >= 1 || !stream_workspace() || !g_stream_error_dev || tiles <= 0 || slabs <= 0) return 0;
+  // while a side branch is open two launches of one recording may run at the same time, and the lane has
+  // one set of slots and flags: neither side takes the stream form then
+  if (wdh::branch_open()) return 0;
   const long long cus = wdh::compute_units();
   if (g_stream == 1) {
     // Measured on the ResNet-50 and DETR layer shapes: resident workgroups that walk segments

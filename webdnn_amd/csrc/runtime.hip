@@ -56,6 +56,16 @@ struct Runtime {
   // lanes >= 1: work may have been enqueued since the lane was last waited for.  The pool hands blocks
   // from lane to lane, so whoever frees a block first waits for these lanes (settle_side_lanes).
   bool lane_dirty[WDH_LANES] = {};
+  // A side branch of the run being recorded (wdh_branch_begin / _end / _join): work recorded between begin
+  // and end goes to branch_stream and depends only on what was recorded before begin; the join makes what
+  // follows depend on it.  0 = none, 1 = recording the branch, 2 = branch recorded, not joined yet.
+  int branch = 0;
+  hipStream_t branch_stream = nullptr, trunk_stream = nullptr;
+  hipEvent_t branch_fork = nullptr, branch_done = nullptr;
+  // blocks freed while a branch is open: nobody may take them before the join, because the two sides of
+  // the fork are not ordered against each other
+  struct FreedBlock { size_t cap; void *ptr; int arena; };
+  std::vector<FreedBlock> branch_freed;
   hipDeviceProp_t prop;
   // handle table; handle = index + 1
   std::vector<Slot> slots;
@@ -158,6 +168,7 @@ bool capturing() { return g.capturing != 0; }
 void poison_capture() { g.capture_failed = true; }
 hipStream_t stream() { return g.stream; }
 int lane() { return g.lane; }
+bool branch_open() { return g.branch != 0; }
 int compute_units() { return g.prop.multiProcessorCount; }
 int device() { return g.device; }
 
@@ -331,6 +342,14 @@ static void release_everything() {
     if (s) (void)hipStreamDestroy(s);
     s = nullptr;
   }
+  if (g.branch_stream) (void)hipStreamDestroy(g.branch_stream);
+  if (g.branch_fork) (void)hipEventDestroy(g.branch_fork);
+  if (g.branch_done) (void)hipEventDestroy(g.branch_done);
+  g.branch_stream = nullptr;
+  g.branch_fork = g.branch_done = nullptr;
+  g.branch = 0;
+  for (auto &b : g.branch_freed) (void)hipFree(b.ptr);  // (held by neither a handle nor the pool)
+  g.branch_freed.clear();
   g.stream = nullptr;
   g.lane = 0;
   g.ready = false;
@@ -424,6 +443,18 @@ wdh_buf wdh_alloc(size_t bytes) {
   return idx + 1;
 }
 
+// A block nobody holds any more: to the graph it belongs to, or to the pool.
+static void give_back(size_t cap, void *ptr, int arena) {
+  if (arena && g.graphs[arena - 1].live) {
+    // memory of a captured graph: stays with it
+    g.graphs[arena - 1].free_blocks.emplace(cap, ptr);
+  } else {
+    g.cache.emplace(cap, ptr);
+    g.cached += cap;
+    g.in_use -= cap;
+  }
+}
+
 int wdh_free(wdh_buf h) {
   WDH_REQUIRE_INIT();
   if (h <= 0 || (size_t)h > g.slots.size() || g.slots[h - 1].ptr == nullptr)
@@ -433,14 +464,10 @@ int wdh_free(wdh_buf h) {
   Slot &s = g.slots[h - 1];
   if (s.cap) {
     settle_side_lanes();
-    if (s.arena && g.graphs[s.arena - 1].live) {
-      // memory of a captured graph: stays with it
-      g.graphs[s.arena - 1].free_blocks.emplace(s.cap, s.ptr);
-    } else {
-      g.cache.emplace(s.cap, s.ptr);
-      g.cached += s.cap;
-      g.in_use -= s.cap;
-    }
+    if (g.branch && g.capturing)
+      g.branch_freed.push_back({s.cap, s.ptr, s.arena});
+    else
+      give_back(s.cap, s.ptr, s.arena);
   }
   s = Slot();
   g.free_slots.push_back(h - 1);
@@ -489,9 +516,73 @@ int wdh_graph_begin(void) {
   return WDH_OK;
 }
 
+// The blocks freed while the branch was open become available (to the graph being recorded, or to the pool).
+static void branch_release_blocks() {
+  for (auto &b : g.branch_freed) give_back(b.cap, b.ptr, b.arena);
+  g.branch_freed.clear();
+}
+
+int wdh_branch_begin(void) {
+  WDH_REQUIRE_INIT();
+  if (!g.capturing) return WDH_OK;  // executing, not recording: one stream, the order of the calls
+  if (g.branch) {
+    g.capture_failed = true;
+    return fail(WDH_ESTATE, "wdh_branch_begin: a branch is open already (one at a time)");
+  }
+  if (!g.branch_stream) {
+    WDH_HIP_CHECK(hipStreamCreateWithFlags(&g.branch_stream, hipStreamNonBlocking));
+    WDH_HIP_CHECK(hipEventCreateWithFlags(&g.branch_fork, hipEventDisableTiming));
+    WDH_HIP_CHECK(hipEventCreateWithFlags(&g.branch_done, hipEventDisableTiming));
+  }
+  // the branch stream joins the capture behind everything recorded so far
+  WDH_HIP_CHECK(hipEventRecord(g.branch_fork, g.stream));
+  WDH_HIP_CHECK(hipStreamWaitEvent(g.branch_stream, g.branch_fork, 0));
+  g.trunk_stream = g.stream;
+  g.stream = g.branch_stream;
+  g.branch = 1;
+  return WDH_OK;
+}
+
+int wdh_branch_end(void) {
+  WDH_REQUIRE_INIT();
+  if (!g.capturing) return WDH_OK;
+  if (g.branch != 1) {
+    g.capture_failed = true;
+    return fail(WDH_ESTATE, "wdh_branch_end: no branch is being recorded");
+  }
+  WDH_HIP_CHECK(hipEventRecord(g.branch_done, g.branch_stream));
+  g.stream = g.trunk_stream;
+  g.branch = 2;
+  return WDH_OK;
+}
+
+int wdh_branch_join(void) {
+  WDH_REQUIRE_INIT();
+  if (!g.capturing) return WDH_OK;
+  if (g.branch != 2) {
+    g.capture_failed = true;
+    return fail(WDH_ESTATE, "wdh_branch_join: no recorded branch to join (wdh_branch_begin, _end first)");
+  }
+  WDH_HIP_CHECK(hipStreamWaitEvent(g.stream, g.branch_done, 0));
+  g.branch = 0;
+  branch_release_blocks();
+  return WDH_OK;
+}
+
 int wdh_graph_end(int *graph_id) {
   WDH_REQUIRE_INIT();
   if (!g.capturing) return fail(WDH_ESTATE, "wdh_graph_end: no capture is open");
+  // a branch left open (a run that failed half way): close it, so that the capture can end
+  if (g.branch == 1) {
+    (void)hipEventRecord(g.branch_done, g.branch_stream);
+    g.stream = g.trunk_stream;
+    g.branch = 2;
+  }
+  if (g.branch == 2) {
+    (void)hipStreamWaitEvent(g.stream, g.branch_done, 0);
+    g.branch = 0;
+  }
+  branch_release_blocks();
   const int id = g.capturing - 1;
   g.capturing = 0;
   hipGraph_t graph = nullptr;

@@ -4,7 +4,7 @@
 //
 //   node run_model.js --model DIR [--onnx model.onnx | --optimized] [--backend hip|cpu]
 //        --inputs a.bin[,b.bin...] --output out.bin
-//        [--strict] [--no-fuse] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
+//        [--strict] [--no-fuse] [--no-side-branches] [--warmup W] [--runs N] [--measure [--queue-ahead MS]] [--measure-all]
 //        [--resident-inputs] [--cpu-entries module.js] [--native module.js]
 //        [--graph | --no-graph] [--in-flight [N]] [--alt-inputs a2.bin[,b2.bin...]]
 //
@@ -56,6 +56,7 @@ function parseArgs(argv) {
     else if (a === "--output") args.output = next();
     else if (a === "--strict") args.strict = true;
     else if (a === "--no-fuse") args.noFuse = true;
+    else if (a === "--no-side-branches") args.noSideBranches = true;
     else if (a === "--warmup") args.warmup = parseInt(next(), 10);
     else if (a === "--runs") args.runs = parseInt(next(), 10);
     else if (a === "--queue-ahead") args.queueAhead = parseFloat(next());
@@ -77,6 +78,7 @@ async function main() {
   const hipOption = { strict: !!args.strict, fuse: !args.noFuse };
   if (args.tile != null) hipOption.contractionTile = args.tile;
   if (args.inFlight) hipOption.inFlight = args.inFlight;
+  if (args.noSideBranches) hipOption.sideBranches = false;
   // --native: another implementation of the addon's interface (host tests without a GPU)
   if (args.native) hipOption.native = require(path.resolve(args.native));
   const runner = await WebDNN.load(args.model, {

@@ -18,6 +18,59 @@ function modelTransform(model, backendOrder, options) {
   if (backendOrder.includes("hip") && opt.fuse !== false) {
     fuseForHip(model);
   }
+  if (backendOrder.includes("hip") && opt.sideBranches !== false) {
+    hoistSideBranches(model.graph);
+  }
+}
+
+// Side branches.  A convolution whose inputs are ready well before its turn -- the projection shortcut of a
+// residual block reads the block's input, and only the block's last convolution wants its result -- is moved
+// up to where its inputs become ready and marked `hipSide`; the first node that reads its result is marked
+// `hipJoin`.  The runner brackets a hipSide node with branchBegin / branchEnd and calls branchJoin before a
+// hipJoin node, so that a recorded run may execute the shortcut next to the convolutions it used to wait
+// behind (one launch then fills what the other leaves idle at its start and its end).  The nodes in between
+// come before the moved node in the original order, so none of them reads its result.  One branch at a time.
+// An eager run executes the new order on one stream: the same kernels on the same data, the same bits.
+const SIDE_BRANCH_OPS = new Set(["Conv", "WebDNNHipFusedConv"]);
+function hoistSideBranches(graph) {
+  const order = [];
+  const producedAt = new Map(); // tensor name -> index in `order` of its producer
+  let pending = null; // outputs of the branch waiting for its join
+  let barrier = 0; // no branch starts before the last join
+  let count = 0;
+  const place = (node, at) => {
+    order.splice(at, 0, node);
+    for (let i = at; i < order.length; i++) for (const name of order[i].output) producedAt.set(name, i);
+  };
+  for (const node of graph.node) {
+    if (pending && node.input.some((name) => pending.has(name))) {
+      node.hipJoin = true;
+      pending = null;
+      barrier = order.length;
+    }
+    if (!pending && !node.hipJoin && SIDE_BRANCH_OPS.has(node.opType)) {
+      let ready = barrier;
+      for (const name of node.input) if (producedAt.has(name)) ready = Math.max(ready, producedAt.get(name) + 1);
+      const between = order.slice(ready);
+      if (between.length >= 2 && between.every((n) => SIDE_BRANCH_OPS.has(n.opType))) {
+        node.hipSide = true;
+        pending = new Set(node.output);
+        place(node, ready);
+        count++;
+        continue;
+      }
+    }
+    place(node, order.length);
+  }
+  if (pending) {
+    // nobody reads the branch's result (a graph output): it is joined at the end of the run anyway
+    for (const n of order) if (n.hipSide && n.output.some((name) => pending.has(name))) delete n.hipSide;
+  }
+  if (count) {
+    graph.node = order;
+    logger.info(`hip: ${count} convolutions run as side branches of recorded runs`);
+  }
+  return count;
 }
 
 function renameDuplicatedNode(model) {
@@ -416,4 +469,4 @@ function findTensorReleaseTiming(model, initializerTensorNames) {
   return timing;
 }
 
-module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention, fuseLayerNormAdd, groupLinears };
+module.exports = { modelTransform, findTensorReleaseTiming, fuseForHip, fuseAttention, fuseLayerNormAdd, groupLinears, hoistSideBranches };

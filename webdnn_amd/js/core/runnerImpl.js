@@ -83,7 +83,7 @@ class RunnerImpl {
   loadModelFromBytes(bytes, directory) {
     this.model = decodeModel(new Uint8Array(bytes.buffer, bytes.byteOffset, bytes.byteLength));
     this.operatorCache.clear();
-    modelTransform(this.model, this.backendOrder, { fuse: this.options.fuse });
+    modelTransform(this.model, this.backendOrder, { fuse: this.options.fuse, sideBranches: this.options.sideBranches });
     if (this.model.opsetImport.length !== 1) {
       logger.warn("Specifying multiple opset_import is not supported. Using first one.");
     }
@@ -503,6 +503,10 @@ class RunnerImpl {
 
             const context = this.contextFor(operator.backend);
             logger.debug(`Running ${node.name}(${opType}) on ${operator.backend}`);
+            // side branches of a recorded run (modelTransform.hoistSideBranches); no-ops while executing
+            const branches = operator.backend === "hip" && hip && hip.native.branchBegin;
+            if (branches && node.hipJoin) hip.native.branchJoin();
+            if (branches && node.hipSide) hip.native.branchBegin();
             // one event per node boundary: node i's device time runs from event i to event i+1
             // (every event costs the stream a small bubble, so as few as possible)
             if (useEvents) hip.native.eventRecord(i);
@@ -516,6 +520,7 @@ class RunnerImpl {
               throw error;
             } finally {
               if (context.stopTracking) context.stopTracking();
+              if (branches && node.hipSide) hip.native.branchEnd();
             }
             actualInputDims = operatorInputs.map((t) => t.dims);
             actualOutputDims = operatorOutputs.map((t) => t.dims);

@@ -65,6 +65,7 @@ async function load(directory, options) {
     fuse: hipOption.fuse,
     graph: hipOption.graph, // true | false | "auto" (default): see RunnerImpl.run
     inFlight: hipOption.inFlight, // 2 (default) .. 4: lanes runner.submit alternates over
+    sideBranches: hipOption.sideBranches, // false: keep the graph's node order (no side branches in recorded runs)
   });
   // An optimized-model directory holds one graph per backend, named after it, and keeps the
   // weights in WDN2 tensor files (separateBuild/coreOnly.ts:200-204).

@@ -15,6 +15,9 @@ export interface WebDNNHipContextOption {
   /** captured runs: true = record the second run; "auto" (default) = record the third run with inputs
    *  of one signature; false = always the node loop.  runner.run(inputs, {graph}) overrides it per call. */
   graph?: boolean | "auto";
+  /** false: keep the graph's node order; by default a convolution whose inputs are ready early (a projection
+   *  shortcut) is moved up and recorded as a side branch that a replay may run next to the main chain */
+  sideBranches?: boolean;
   /** how many runs runner.submit keeps in flight (lanes it alternates over): 2 (default) to 4 */
   inFlight?: number;
   /** tuning hooks handed to wdh_set_option */

@@ -34,6 +34,10 @@ export interface HipNative {
   sync(): void;
   /** wdh_set_lane: 0 = the stream everything runs on by default, 1 = the second stream (two runs in flight). */
   setLane(lane: number): void;
+  /** wdh_branch_begin / _end / _join: a side branch of the run being recorded (no-ops outside a recording). */
+  branchBegin(): void;
+  branchEnd(): void;
+  branchJoin(): void;
   memStats(): HipMemStats;
   trim(keepBytes: number): void;
   eventRecord(id: number): void;

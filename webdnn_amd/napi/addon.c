@@ -225,6 +225,24 @@ FN(js_set_lane) {
   return make_undefined(env);
 }
 
+FN(js_branch_begin) {
+  ARGS("wdh_branch_begin", 0);
+  CHECK(wdh_branch_begin());
+  return make_undefined(env);
+}
+
+FN(js_branch_end) {
+  ARGS("wdh_branch_end", 0);
+  CHECK(wdh_branch_end());
+  return make_undefined(env);
+}
+
+FN(js_branch_join) {
+  ARGS("wdh_branch_join", 0);
+  CHECK(wdh_branch_join());
+  return make_undefined(env);
+}
+
 FN(js_mem_stats) {
   ARGS("wdh_mem_stats", 0);
   uint64_t a = 0, b = 0, c = 0;
@@ -501,7 +519,8 @@ static napi_value init_module(napi_env env, napi_value exports) {
       {"transpose", js_transpose}, {"gather", js_gather}, {"cast", js_cast},
       {"stridedCopy", js_strided_copy}, {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end},
       {"graphLaunch", js_graph_launch}, {"graphDestroy", js_graph_destroy},
-      {"setLane", js_set_lane},
+      {"setLane", js_set_lane}, {"branchBegin", js_branch_begin}, {"branchEnd", js_branch_end},
+      {"branchJoin", js_branch_join},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {
     napi_value fn;
