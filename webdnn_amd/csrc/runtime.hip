@@ -304,6 +304,7 @@ void wdh_shutdown(void) {
 static void release_everything() {
   if (g.capturing) {
     hipGraph_t dropped = nullptr;
+    if (g.branch == 1) g.stream = g.trunk_stream;  // (the capture began on the trunk)
     (void)hipStreamEndCapture(g.stream, &dropped);
     if (dropped) (void)hipGraphDestroy(dropped);
     g.capturing = 0;
