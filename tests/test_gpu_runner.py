@@ -228,6 +228,23 @@ def test_two_runs_in_flight_equal_eager_runs(tmp_path):
                 assert_bit_exact(got[0], want[0], "run %d of a session with two runs in flight %s" % (runs, flags))
 
 
+def test_many_runs_in_flight_every_output_checked(tmp_path):
+    """300 runs with alternating inputs, two and three in flight, from the host and resident: every collected
+    output equals, byte for byte, the first output seen for its input (an eager run), so a hand-over between the
+    lanes, a recycled block or a side branch that is wrong once in a hundred runs shows."""
+    data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)
+    Xa = np.random.default_rng(2).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    Xb = np.random.default_rng(3).standard_normal((8, 3, 64, 64)).astype(np.float32)
+    (tmp_path / "model.onnx").write_bytes(data)
+    eb, _ = node_runner.run_model(str(tmp_path), [Xb], "hip", strict=True, extra=["--no-graph"])
+    for lanes in ("2", "3"):
+        for resident in (False, True):
+            got, rep = _graph_runs(tmp_path, data, [Xa], [Xb], 300, resident=resident, flags=("--in-flight", lanes, "--check-each"))
+            assert rep["checkEach"] == {"checkedRuns": 298, "mismatchedRuns": 0}, (lanes, resident, rep["checkEach"])
+            assert rep["graph"]["lanes"] == int(lanes)
+            assert_bit_exact(got[0], eb[0], "the last of 300 runs")
+
+
 def test_three_runs_in_flight_equal_eager_runs(tmp_path):
     """The same with three lanes (load option inFlight = 3): from the sixth run on all three hold a recording."""
     data, _ = modelgen.resnet50_model(batch=8, image=64, width=16, blocks=(1, 2, 1, 1), classes=10)

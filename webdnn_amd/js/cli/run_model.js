@@ -57,6 +57,7 @@ function parseArgs(argv) {
     else if (a === "--strict") args.strict = true;
     else if (a === "--no-fuse") args.noFuse = true;
     else if (a === "--no-side-branches") args.noSideBranches = true;
+    else if (a === "--check-each") args.checkEach = true;
     else if (a === "--warmup") args.warmup = parseInt(next(), 10);
     else if (a === "--runs") args.runs = parseInt(next(), 10);
     else if (a === "--queue-ahead") args.queueAhead = parseFloat(next());
@@ -123,6 +124,21 @@ async function main() {
     }
     runner.backendContexts.hip.sync();
   }
+  // --check-each: every timed run's outputs are compared, byte for byte, with the first outputs seen for the
+  // same input set (even runs: --inputs, odd runs: --alt-inputs); the report counts the runs that differ
+  const firstSeen = [null, null];
+  let mismatchedRuns = 0, checkedRuns = 0;
+  const checkRun = (index, outs) => {
+    if (!args.checkEach) return;
+    const which = runAltInputs && index % 2 === 1 ? 1 : 0;
+    const bytes = outs.map((t) => Buffer.from(t.data.buffer, t.data.byteOffset, t.data.byteLength));
+    if (!firstSeen[which]) {
+      firstSeen[which] = bytes.map((b) => Buffer.from(b));
+      return;
+    }
+    checkedRuns++;
+    if (bytes.length !== firstSeen[which].length || bytes.some((b, k) => !b.equals(firstSeen[which][k]))) mismatchedRuns++;
+  };
   const runOptions = (extra) => (args.graph === undefined ? extra : Object.assign({ graph: args.graph }, extra));
   for (let i = 0; i < args.warmup; i++) await runner.run(runInputs, runOptions({}));
   const times = [];
@@ -130,11 +146,15 @@ async function main() {
   let queueAhead = null;
   const deviceTimes = [];
   if (args.inFlight) {
-    const pending = []; // tickets in order of submission, at most args.inFlight - 1 while the next is submitted
+    const pending = []; // [run index, ticket] in order of submission, at most args.inFlight - 1 while the next is submitted
     let t0 = process.hrtime.bigint();
     for (let i = 0; i < args.runs; i++) {
-      pending.push(await runner.submit(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs, runOptions({})));
-      while (pending.length >= args.inFlight || (i + 1 === args.runs && pending.length)) outputs = await runner.collect(pending.shift());
+      pending.push([i, await runner.submit(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs, runOptions({}))]);
+      while (pending.length >= args.inFlight || (i + 1 === args.runs && pending.length)) {
+        const [index, ticket] = pending.shift();
+        outputs = await runner.collect(ticket);
+        checkRun(index, outputs);
+      }
       const t1 = process.hrtime.bigint();
       times.push(Number(t1 - t0) / 1e6);
       t0 = t1;
@@ -161,6 +181,7 @@ async function main() {
     outputs = await runner.run(runAltInputs && i % 2 === 1 ? runAltInputs : runInputs,
       runOptions({ measurePerformance: !!args.measureAll || (!!args.measure && i === args.runs - 1) }));
     times.push(Number(process.hrtime.bigint() - t0) / 1e6);
+    checkRun(i, outputs);
     // --measure-all: device time of every timed run (HIP events on the library's stream; a replayed
     // graph is bracketed by one pair, an eager run has one event per node boundary)
     if (args.measureAll && runner.lastPerformance) {
@@ -182,6 +203,7 @@ async function main() {
     deviceMsPerRun: args.measureAll ? deviceTimes : undefined,
     stats: runner.lastRunStats,
     nodes: runner.model.graph.node.length,
+    checkEach: args.checkEach ? { checkedRuns, mismatchedRuns } : undefined,
     node: process.version,
     graph: args.graph !== false ? { captured: !!runner.graphState, lanes: (runner.graphState ? 1 : 0) + runner.sideGraphStates.filter((st) => st).length,
       unsupported: runner.graphUnsupported } : undefined,
