@@ -324,7 +324,8 @@ class RunnerImpl {
   // library waits for uploads by itself -- or produced by work that has been waited for): the lanes do
   // not wait for each other.
   // At most one run per lane may be outstanding: collect in the order of submission.  A second batch in
-  // flight fills most of what one leaves idle (ResNet-50 b32: +12 %); a third and a fourth add 3 % and 1 %.
+  // flight fills most of what one leaves idle (ResNet-50 b32: +11 %, a batch-1 DETR +33 %); a third adds little
+  // once recordings have side branches, and four lanes are more than a process has hardware queues for.
   async submit(inputs, options) {
     const opts = options || {};
     if (!this.model || !this.loaded) throw new Error("not initialized");
