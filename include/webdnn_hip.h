@@ -198,7 +198,9 @@ int wdh_sync(void);
  * of K slabs use a workspace of the lane's own (WDH_STATIC_SCRATCH_BYTES from the driver when the lane is
  * first used), so a run recorded on a side lane computes bit for bit what it computes on lane 0;
  * wdh_gemm_static is refused there (its workspace is lane 0's); a wdh_copy on a side lane first waits
- * for uploads (wdh_write) still on their way on any lane.  What the caller guards: a buffer written on one lane and read on another needs a
+ * for uploads (wdh_write) still on their way on any lane.  A recorded run may be launched on any lane, but it
+ * keeps using the stream workspace of the lane it was recorded on: launch two recordings at the same time
+ * only if they were made on different lanes (runner.submit does).  What the caller guards: a buffer written on one lane and read on another needs a
  * wdh_sync (or wdh_read) on the first in between.  Not possible while capturing. */
 #define WDH_LANES 4
 int wdh_set_lane(int lane);
