@@ -218,6 +218,41 @@ def test_conv3x3_minimal_filtering_random_geometry(ctx, i):
                      % (n, cin, h, w, cout, pads, mode, form))
 
 
+@pytest.mark.parametrize("i", range(40))
+def test_conv_random_network_sized_geometry(ctx, i):
+    """1x1 and 3x3 convs with the channel counts, planes and batches of real networks (16 .. 512 channels, planes up
+    to 59 x 59, stride 1 or 2, ragged output channels, with and without bias, residual and Relu): whichever form
+    the plan picks -- in place, in place with stride 2, LDS tile, minimal filtering, gathered; whole tiles, tiles
+    cut along K, small products -- against the oracle."""
+    r = rng_for("netconv", i)
+    k = int(r.choice([1, 1, 3, 3, 3]))
+    s = int(r.choice([1, 1, 2]))
+    n = int(r.choice([1, 2, 4, 8, 16, 32]))
+    cin = 16 * int(r.integers(1, 33))
+    cout = int(r.choice([16 * int(r.integers(1, 33)), int(r.integers(1, 600))]))
+    h, w = int(r.integers(max(k, 4), 60)), int(r.integers(max(k, 4), 60))
+    pads = [int(r.integers(0, k)) for _ in range(4)] if k == 3 else [0] * 4
+    macs = n * cin * cout * (h // s) * (w // s) * k * k
+    if macs > 6e8:
+        n = max(1, int(n * 6e8 / macs))          # (keeps the oracle's share of a case under a second)
+    X = f32(r, (n, cin, h, w), -1 if i % 2 else 0, 1)
+    W = (f32(r, (cout, cin, k, k), -1, 1) * np.float32(np.sqrt(2.0 / (cin * k * k)))).astype(np.float32)
+    Bs = f32(r, (cout,)) if i % 3 else None
+    want = ref.conv(X, W, Bs, None, 1, None, pads, [s, s])
+    R = f32(r, want.shape) if i % 2 else None
+    if R is not None:
+        want = ref.binary("Add", want, R)
+    relu = i % 5 < 3
+    if relu:
+        want = ref.unary("Relu", want)
+    got = H.conv(ctx, ctx.move_tensor(X), ctx.move_tensor(W), ctx.move_tensor(Bs) if Bs is not None else None, None, 1, None,
+                 pads, [s, s], "relu" if relu else None, ctx.move_tensor(R) if R is not None else None)
+    plan = ctx.last_plan()
+    assert tuple(got.dims) == want.shape
+    assert_close_max(got.get_data(), want, 1e-4, "conv n%d cin%d %dx%d cout%d k%d s%d pads%s (%s, %s, split %d)"
+                     % (n, cin, h, w, cout, k, s, pads, plan["form"], plan["tile"], plan["split"]))
+
+
 @pytest.mark.parametrize("i", range(20))
 def test_row_reductions_random_lengths(ctx, i):
     r = rng_for("rows", i)
