@@ -10,4 +10,8 @@ export interface HipTensor extends Tensor {
   /** Another view of the same device buffer with other dims (Reshape, Flatten, Squeeze, Unsqueeze);
    *  the buffer is freed when the last view is disposed. */
   alias(dims: ReadonlyArray<number>): HipTensor;
+  /** Set by the runner on the device copy of an initializer: the contents stay as they are for as long as the
+   *  tensor lives, so an operator may let the library keep what it derives from them (Conv passes
+   *  WDH_CONV_CONSTANT_WEIGHTS). */
+  constant?: boolean;
 }
