@@ -315,8 +315,8 @@ int wdh_linear_group(int count, const wdh_buf *A, const wdh_buf *W, const wdh_bu
  * unsplit launches use no workspace).  All calls on a GPU share the one workspace,
  * which keeps the previous call's contents: the kernels write every partial sum
  * they later read, so nothing has to be cleared, but two such calls that overlap
- * on one GPU (other streams, other threads) race; the library's single stream
- * orders them. */
+ * on one GPU (other streams, other threads) race; lane 0, the only lane that takes
+ * this call, orders them. */
 #define WDH_STATIC_SCRATCH_BYTES ((32u << 20) + (160u << 10))
 int wdh_gemm_static(wdh_buf A, wdh_buf B, wdh_buf C, wdh_buf Y, int batch, int m,
                     int n, int k, int64_t sAb, int64_t sA0, int64_t sA1,
